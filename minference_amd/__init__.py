@@ -1,0 +1,13 @@
+"""minference_amd -- MI355X (gfx950) dynamic sparse prefill attention.
+
+Same operator surface as microsoft/MInference (minference/__init__.py:9-11):
+``vertical_slash_sparse_attention``, ``block_sparse_attention`` and
+``streaming_forward``, backed by hand-written HIP kernels in
+``libminf_hip.so`` (C ABI in include/minf_hip.h) instead of Triton/CUDA.
+Importing the package needs neither a GPU nor the built library; calling an
+operator without them raises.
+"""
+from .index import convert_vertical_slash_indexes
+
+__all__ = ["convert_vertical_slash_indexes"]
+__version__ = "0.1.0"

@@ -1,0 +1,57 @@
+"""ctypes binding of libminf_hip.so (the C ABI declared in include/minf_hip.h).
+
+The library is never built implicitly and there is no fallback: if it is
+missing, or a call returns a non-zero status, a RuntimeError is raised.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libminf_hip.so")
+_lib = None
+
+c_int = ctypes.c_int
+c_i64 = ctypes.c_int64
+c_f32 = ctypes.c_float
+c_ptr = ctypes.c_void_p
+
+# name -> (restype, argtypes); must list every symbol of include/minf_hip.h
+SIGNATURES = {
+    "minf_version": (c_int, []),
+    "minf_status_string": (ctypes.c_char_p, [c_int]),
+    "minf_vs_index_build": (c_int, [c_ptr] * 7 + [c_int] * 6 + [c_ptr, c_ptr]),
+}
+
+
+class MinfError(RuntimeError):
+    pass
+
+
+def load():
+    """Load libminf_hip.so once; raise if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise MinfError(
+                f"{LIB_PATH} not found: build it with `python -m minference_amd.build` "
+                "(there is no fallback path)")
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+def check(status: int, what: str):
+    if status != 0:
+        msg = load().minf_status_string(status)
+        raise MinfError(f"{what} failed: {msg.decode() if msg else status} ({status})")
+
+
+def stream_ptr(device=None):
+    import torch
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
