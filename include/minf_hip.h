@@ -72,6 +72,71 @@ int minf_vs_index_build(const int32_t *seqlens, const int32_t *vertical_idx,
                         int nnz_v, int nnz_s, int zero_fill, int32_t *error_flag,
                         void *stream);
 
+/*
+ * Sparse flash-attention forward on one shared 64x64 bf16/f16 MFMA tile
+ * engine.  Common arguments of the four entry points below:
+ *
+ *   q [batch, heads_q, n, head_dim], k/v [batch, heads_kv, n, head_dim],
+ *   o [batch, heads_q, n, head_dim]: base pointers + element strides
+ *   {batch, head, token} (head_dim stride is 1); heads_q % heads_kv == 0 and
+ *   query head h reads kv head h / (heads_q / heads_kv) (no repeat_kv copy is
+ *   needed; the reference always expands K/V first,
+ *   minference/modules/forward.py:128-132).  head_dim must be 128.
+ *   seqlens [batch] int32 may be NULL (= n for every batch).  Rows >= seqlen
+ *   are written as zeros (the reference leaves its zeros_like buffer untouched).
+ *   sm_scale multiplies q.k before the softmax (reference: head_dim^-0.5).
+ *   Every o element of every row < n is written; nothing else is.
+ */
+typedef struct minf_qkvo {
+    const void *q, *k, *v;
+    void *o;
+    int64_t q_stride[3], k_stride[3], v_stride[3], o_stride[3];   /* batch, head, token */
+    int batch, heads_q, heads_kv, n, head_dim, dtype;
+    const int32_t *seqlens;
+    float sm_scale;
+} minf_qkvo;
+
+/*
+ * Mixed block-sparse + column-sparse forward over the tensors produced by
+ * minf_vs_index_build.  Replaces _triton_mixed_sparse_attention /
+ * _triton_mixed_sparse_attn_fwd_kernel
+ *   (reference minference/ops/pit_sparse_flash_attention_v2.py:48-192).
+ * Row r of row block m attends {c in [off, off+64) for the first
+ * block_count[m] offsets : c <= r, c < seqlen} plus the first column_count[m]
+ * entries of column_index (no causal test on those, as in the reference).
+ * Index tensors are indexed by QUERY head: [batch, heads_q, rows, nnz_*].
+ */
+int minf_vs_attn_fwd(const minf_qkvo *t, const int32_t *block_count,
+                     const int32_t *block_offset, const int32_t *column_count,
+                     const int32_t *column_index, int rows, int nnz_s, int nnz_v,
+                     void *stream);
+
+/*
+ * Block-sparse forward.  Replaces _triton_block_sparse_attention
+ *   (reference minference/ops/block_sparse_flash_attention.py:29-148).
+ * block_index [batch, heads_q, rows, max_blocks] int32, each row ascending;
+ * rows >= ceil(n/64) (the reference builds it on a padded sequence);
+ * row block m visits its first min(m+1, max_blocks) entries, element-wise
+ * causal (reference :81-96).
+ */
+int minf_bs_attn_fwd(const minf_qkvo *t, const int32_t *block_index, int rows,
+                     int max_blocks, void *stream);
+
+/*
+ * A-shape (attention sink + sliding window) forward in one pass.  Replaces
+ * streaming_forward's two-stage TritonMultiStageDotProductionAttention
+ *   (reference minference/ops/streaming_kernel.py:26-239, 611-646).
+ * Row r attends {c : r - n_local < c <= r} plus {c < n_init : c <= r - n_local}.
+ */
+int minf_ashape_attn_fwd(const minf_qkvo *t, int n_init, int n_local, void *stream);
+
+/*
+ * Dense causal forward on the same tile engine (the in-house comparator for
+ * the sparse-vs-dense speed-up; the reference uses flash_attn_func,
+ * minference/modules/minference_forward.py:666).
+ */
+int minf_dense_attn_fwd(const minf_qkvo *t, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -8,6 +8,13 @@ Importing the package needs neither a GPU nor the built library; calling an
 operator without them raises.
 """
 from .index import convert_vertical_slash_indexes
+from .ops import (block_sparse_attention, block_sparse_attention_from_index, dense_causal_attention,
+                  streaming_forward, vertical_slash_attention_from_index,
+                  vertical_slash_sparse_attention)
 
-__all__ = ["convert_vertical_slash_indexes"]
+__all__ = [
+    "vertical_slash_sparse_attention", "block_sparse_attention", "streaming_forward",
+    "convert_vertical_slash_indexes", "vertical_slash_attention_from_index",
+    "block_sparse_attention_from_index", "dense_causal_attention",
+]
 __version__ = "0.1.0"

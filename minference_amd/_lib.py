@@ -22,7 +22,26 @@ SIGNATURES = {
     "minf_version": (c_int, []),
     "minf_status_string": (ctypes.c_char_p, [c_int]),
     "minf_vs_index_build": (c_int, [c_ptr] * 7 + [c_int] * 6 + [c_ptr, c_ptr]),
+    "minf_vs_attn_fwd": (c_int, [c_ptr] * 5 + [c_int] * 3 + [c_ptr]),
+    "minf_bs_attn_fwd": (c_int, [c_ptr, c_ptr, c_int, c_int, c_ptr]),
+    "minf_ashape_attn_fwd": (c_int, [c_ptr, c_int, c_int, c_ptr]),
+    "minf_dense_attn_fwd": (c_int, [c_ptr, c_ptr]),
 }
+
+
+class QKVO(ctypes.Structure):
+    """struct minf_qkvo of include/minf_hip.h."""
+    _fields_ = [
+        ("q", c_ptr), ("k", c_ptr), ("v", c_ptr), ("o", c_ptr),
+        ("q_stride", c_i64 * 3), ("k_stride", c_i64 * 3), ("v_stride", c_i64 * 3), ("o_stride", c_i64 * 3),
+        ("batch", c_int), ("heads_q", c_int), ("heads_kv", c_int), ("n", c_int),
+        ("head_dim", c_int), ("dtype", c_int),
+        ("seqlens", c_ptr),
+        ("sm_scale", c_f32),
+    ]
+
+
+MINF_BF16, MINF_F16 = 0, 1
 
 
 class MinfError(RuntimeError):

@@ -1,0 +1,488 @@
+// Sparse flash-attention forward for gfx950: one 64x64 tile engine, four tile
+// sources (vertical-slash block+column lists, block-sparse lists, analytic
+// A-shape ranges, dense causal).
+//
+// Work split: one workgroup (2 wavefronts) per (batch, query head, 64-row
+// block); each wavefront owns 32 query rows.  Everything is computed in the
+// TRANSPOSED orientation so that softmax statistics are per lane:
+//
+//   S^T[token][qrow] = K_tile . Q^T      v_mfma_f32_32x32x16 (A = K from LDS, B = Q in VGPRs)
+//   O^T[d][qrow]    += V_tile^T . P^T    (A = V^T via ds_read_b64_tr_b16, B = P straight from
+//                                          the S^T accumulators, converted to bf16/f16)
+//
+// In the 32x32 accumulator layout lane l holds column n = l%32 (one query row)
+// and rows 8*(r/4) + 4*(l/32) + r%4, so the running max / sum / rescale factor
+// of a query row live in lanes l and l^32 and never need a row broadcast, and
+// the probabilities of a lane are exactly the B operand of the second MFMA once
+// the contraction (token) index is permuted the same way on the V side.
+//
+// LDS: K and V tiles are [64 tokens][128] 16-bit, 256 B per row, no padding;
+// 16-byte chunks are XOR-swizzled (K: chunk ^ row%16, V: chunk ^ 4*(row%4)) so
+// that ds_read_b128 of 16 rows and the 4-row transpose reads hit distinct banks.
+// Global->LDS goes through registers, prefetched one tile ahead.
+#include "minf_common.h"
+#include <math.h>
+
+namespace {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(short)))) short short4_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
+
+enum { MODE_VS = 0, MODE_BS = 1, MODE_ASHAPE = 2, MODE_DENSE = 3 };
+
+constexpr int BM = 64;        // query rows per workgroup
+constexpr int BN = 64;        // keys per tile
+constexpr int HD = 128;       // head_dim
+constexpr int NTHREADS = 128; // 2 wavefronts
+constexpr int ROW_BYTES = HD * 2;
+
+struct AttnParams {
+    const char *q, *k, *v;
+    char *o;
+    long long qs[3], ks[3], vs[3], os[3];   // element strides: batch, head, token
+    int batch, hq, hk, n;
+    const int *seqlens;
+    float scale_log2;
+    int rows;
+    // vertical-slash
+    const int *bc, *bo, *cc, *ci;
+    int nnz_s, nnz_v;
+    // block-sparse
+    const int *bidx;
+    int max_blocks, bidx_rows;
+    // a-shape
+    int n_init, n_local;
+    long long total_wg;
+};
+
+template <typename T> struct Mma;
+template <> struct Mma<__bf16> {
+    typedef bf16x8_t vec;
+    static __device__ __forceinline__ f32x16_t mfma(vec a, vec b, f32x16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+};
+template <> struct Mma<_Float16> {
+    typedef f16x8_t vec;
+    static __device__ __forceinline__ f32x16_t mfma(vec a, vec b, f32x16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+};
+
+union Frag {
+    uint4 u;
+    bf16x8_t b;
+    f16x8_t h;
+    short4_t s4[2];
+};
+
+template <typename T> __device__ __forceinline__ typename Mma<T>::vec frag_as(const Frag &f);
+template <> __device__ __forceinline__ bf16x8_t frag_as<__bf16>(const Frag &f) { return f.b; }
+template <> __device__ __forceinline__ f16x8_t frag_as<_Float16>(const Frag &f) { return f.h; }
+
+template <typename T> __device__ __forceinline__ void cvt8(const float *x, Frag &f);
+template <> __device__ __forceinline__ void cvt8<__bf16>(const float *x, Frag &f) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) f.b[j] = (__bf16)x[j];
+}
+template <> __device__ __forceinline__ void cvt8<_Float16>(const float *x, Frag &f) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) f.h[j] = (_Float16)x[j];
+}
+
+// One tile of keys: either 64 consecutive tokens from `start`, or 64 gathered
+// token ids read from `gather` (entries >= nvalid are padding).
+struct Tile {
+    int start;          // first token (contiguous) / first list position (gathered)
+    int gathered;       // 0/1
+    int nvalid;         // gathered: number of valid list entries in this tile
+};
+
+template <int MODE>
+__device__ __forceinline__ int tile_count(const AttnParams &p, long long ridx, int m, int &nblk) {
+    if constexpr (MODE == MODE_VS) {
+        nblk = p.bc[ridx];
+        return nblk + ((p.cc[ridx] + BN - 1) >> 6);
+    } else if constexpr (MODE == MODE_BS) {
+        nblk = min(m + 1, p.max_blocks);
+        return nblk;
+    } else if constexpr (MODE == MODE_ASHAPE) {
+        // window tiles t_lo..m, preceded by the sink tiles that lie before t_lo
+        int lo_key = m * BM - p.n_local + 1;
+        int t_lo = lo_key > 0 ? (lo_key >> 6) : 0;
+        int sink_tiles = (p.n_init + BN - 1) >> 6;
+        nblk = min(sink_tiles, t_lo);            // number of leading sink tiles
+        return nblk + (m - t_lo + 1);
+    } else {
+        nblk = m + 1;
+        return nblk;
+    }
+}
+
+template <int MODE>
+__device__ __forceinline__ Tile tile_at(const AttnParams &p, long long ridx, int m, int nblk, int it) {
+    Tile t;
+    t.gathered = 0;
+    t.nvalid = BN;
+    if constexpr (MODE == MODE_VS) {
+        if (it < nblk) {
+            t.start = p.bo[ridx * p.nnz_s + it];
+        } else {
+            t.gathered = 1;
+            t.start = (it - nblk) * BN;
+            t.nvalid = min(BN, p.cc[ridx] - t.start);
+        }
+    } else if constexpr (MODE == MODE_BS) {
+        t.start = p.bidx[((ridx / p.rows) * p.bidx_rows + m) * p.max_blocks + it] * BN;
+    } else if constexpr (MODE == MODE_ASHAPE) {
+        int lo_key = m * BM - p.n_local + 1;
+        int t_lo = lo_key > 0 ? (lo_key >> 6) : 0;
+        t.start = (it < nblk ? it : t_lo + (it - nblk)) * BN;
+    } else {
+        t.start = it * BN;
+    }
+    return t;
+}
+
+template <typename T, int MODE>
+__global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams p) {
+    __shared__ __attribute__((aligned(16))) char lds_k[BN * ROW_BYTES];
+    __shared__ __attribute__((aligned(16))) char lds_v[BN * ROW_BYTES];
+
+    // ---- which (batch, head, row block): XCD-aware remap --------------------
+    // Consecutive workgroup ids are dealt round-robin to the 8 XCDs; give each
+    // XCD one contiguous range of the logical order (batch, kv head, row block,
+    // query head inside the GQA group) so that the row blocks and the query
+    // heads that share K/V also share an L2.
+    const long long per_xcd = (p.total_wg + 7) >> 3;
+    const long long logical = (long long)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (logical >= p.total_wg) return;
+    const int group = p.hq / p.hk;
+    long long rest = logical;
+    const int hin = (int)(rest % group); rest /= group;
+    const int m = p.rows - 1 - (int)(rest % p.rows); rest /= p.rows;   // heavy (late) rows first
+    const int hkv = (int)(rest % p.hk);
+    const int b = (int)(rest / p.hk);
+    const int h = hkv * group + hin;
+
+    const int tid = (int)threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int l32 = lane & 31;
+    const int g = lane >> 5;
+
+    const int seqlen = p.seqlens ? min(p.seqlens[b], p.n) : p.n;
+    const int row0 = m * BM;
+    const int qrow = row0 + wave * 32 + l32;          // this lane's query row
+    char *o_base = p.o + ((long long)b * p.os[0] + (long long)h * p.os[1]) * 2;
+
+    if (row0 >= seqlen) {
+        // row block past the sequence: zeros (16 B per lane-step)
+        for (int i = tid; i < BM * 16; i += NTHREADS) {
+            int r = row0 + (i >> 4);
+            if (r < p.n) *reinterpret_cast<uint4 *>(o_base + (long long)r * p.os[2] * 2 + (i & 15) * 16) = make_uint4(0, 0, 0, 0);
+        }
+        return;
+    }
+
+    const char *q_base = p.q + ((long long)b * p.qs[0] + (long long)h * p.qs[1]) * 2;
+    const char *k_base = p.k + ((long long)b * p.ks[0] + (long long)hkv * p.ks[1]) * 2;
+    const char *v_base = p.v + ((long long)b * p.vs[0] + (long long)hkv * p.vs[1]) * 2;
+    const long long k_row = p.ks[2] * 2, v_row = p.vs[2] * 2;
+    const long long ridx = ((long long)b * p.hq + h) * p.rows + m;
+
+    // ---- Q fragments (B operand of S^T): row qrow, d = 16*ks + 8*g + 0..7 ----
+    Frag qf[8];
+    {
+        const bool ok = qrow < seqlen;
+        const char *qp = q_base + (long long)(ok ? qrow : row0) * p.qs[2] * 2 + g * 16;
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) {
+            qf[ks].u = *reinterpret_cast<const uint4 *>(qp + ks * 32);
+            if (!ok) qf[ks].u = make_uint4(0, 0, 0, 0);
+        }
+    }
+
+    int nblk = 0;
+    const int ntiles = tile_count<MODE>(p, ridx, m, nblk);
+
+    // ---- global -> register staging: thread covers rows i*8 + tid/16, chunk tid%16
+    const int ld_r = tid >> 4;       // 0..7
+    const int ld_c = tid & 15;       // 16-byte chunk in the row
+    uint4 kreg[8], vreg[8];
+
+    auto issue_loads = [&](const Tile &t) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int r = i * 8 + ld_r;
+            int tok;
+            bool ok;
+            if (MODE == MODE_VS && t.gathered) {
+                ok = r < t.nvalid;
+                tok = ok ? p.ci[ridx * p.nnz_v + t.start + r] : 0;
+            } else {
+                tok = t.start + r;
+                ok = tok < seqlen;
+                if (!ok) tok = 0;
+            }
+            kreg[i] = *reinterpret_cast<const uint4 *>(k_base + tok * k_row + ld_c * 16);
+            vreg[i] = *reinterpret_cast<const uint4 *>(v_base + tok * v_row + ld_c * 16);
+            if (!ok) {
+                kreg[i] = make_uint4(0, 0, 0, 0);
+                vreg[i] = make_uint4(0, 0, 0, 0);
+            }
+        }
+    };
+    auto store_lds = [&]() {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int r = i * 8 + ld_r;
+            *reinterpret_cast<uint4 *>(lds_k + r * ROW_BYTES + ((ld_c ^ (r & 15)) << 4)) = kreg[i];
+            *reinterpret_cast<uint4 *>(lds_v + r * ROW_BYTES + ((ld_c ^ ((r & 3) << 2)) << 4)) = vreg[i];
+        }
+    };
+
+    // ---- accumulators -------------------------------------------------------
+    f32x16_t oacc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[i][r] = 0.f;
+    float m_i = -INFINITY;   // running max (log2 domain, scaled)
+    float l_i = 0.f;         // this lane's share of the running sum
+
+    // LDS read addresses that do not depend on the tile
+    // K: row = 32*blk + l32, logical chunk 2*ks + g
+    const int k_rd_row = l32;
+    // V transpose read: row = T0 + (lane%16)/4, col = 32*db + 16*((lane/16)%2) + 4*(lane%4)
+    const int v_rd_rsub = (lane & 15) >> 2;
+    const int v_rd_chunk = (((lane >> 4) & 1) << 1) + ((lane & 3) >> 1);   // + 4*db
+    const int v_rd_byte = (lane & 1) << 3;
+
+    Tile cur, nxt;
+    if (ntiles > 0) {
+        cur = tile_at<MODE>(p, ridx, m, nblk, 0);
+        issue_loads(cur);
+    }
+
+    for (int it = 0; it < ntiles; ++it) {
+        __syncthreads();            // previous tile fully consumed
+        store_lds();
+        __syncthreads();
+        if (it + 1 < ntiles) {
+            nxt = tile_at<MODE>(p, ridx, m, nblk, it + 1);
+            issue_loads(nxt);
+        }
+
+        // ---- S^T = K . Q^T --------------------------------------------------
+        f32x16_t s0, s1;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { s0[r] = 0.f; s1[r] = 0.f; }
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) {
+            const int x = 2 * ks + g;
+            Frag a0, a1;
+            a0.u = *reinterpret_cast<const uint4 *>(lds_k + k_rd_row * ROW_BYTES + ((x ^ (k_rd_row & 15)) << 4));
+            a1.u = *reinterpret_cast<const uint4 *>(lds_k + (32 + k_rd_row) * ROW_BYTES + ((x ^ (k_rd_row & 15)) << 4));
+            s0 = Mma<T>::mfma(frag_as<T>(a0), frag_as<T>(qf[ks]), s0);
+            s1 = Mma<T>::mfma(frag_as<T>(a1), frag_as<T>(qf[ks]), s1);
+        }
+
+        // ---- mask -----------------------------------------------------------
+        // element (blk, r) of this lane is token 32*blk + 8*(r/4) + 4*g + r%4
+        bool need_mask;
+        const int wrow_lo = row0 + wave * 32, wrow_hi = wrow_lo + 31;
+        if (MODE == MODE_VS && cur.gathered) {
+            need_mask = cur.nvalid < BN;
+        } else if constexpr (MODE == MODE_ASHAPE) {
+            const int c_lo = cur.start, c_hi = cur.start + BN - 1;
+            const bool causal_ok = c_hi <= wrow_lo && c_hi < seqlen;
+            const bool in_window = (wrow_hi - c_lo) < p.n_local;
+            const bool in_sink = c_hi < p.n_init;
+            need_mask = !(causal_ok && (in_window || in_sink));
+        } else {
+            need_mask = (cur.start + BN - 1 > wrow_lo) || (cur.start + BN > seqlen);
+        }
+        if (need_mask) {
+#pragma unroll
+            for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int tk = 32 * blk + 8 * (r >> 2) + 4 * g + (r & 3);
+                    bool keep;
+                    if (MODE == MODE_VS && cur.gathered) {
+                        keep = tk < cur.nvalid;
+                    } else {
+                        const int c = cur.start + tk;
+                        keep = (c <= qrow) && (c < seqlen);
+                        if constexpr (MODE == MODE_ASHAPE)
+                            keep = keep && ((qrow - c) < p.n_local || c < p.n_init);
+                    }
+                    if (!keep) { if (blk == 0) s0[r] = -INFINITY; else s1[r] = -INFINITY; }
+                }
+        }
+
+        // ---- online softmax (exp2 domain) -------------------------------------
+        float mx = s0[0];
+#pragma unroll
+        for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s0[r]);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s1[r]);
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(m_i, mx * p.scale_log2);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f(m_i - m_use);
+        m_i = m_new;
+        float psum = 0.f;
+        float pv[32];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            pv[r] = __builtin_amdgcn_exp2f(fmaf(s0[r], p.scale_log2, -m_use));
+            pv[16 + r] = __builtin_amdgcn_exp2f(fmaf(s1[r], p.scale_log2, -m_use));
+        }
+#pragma unroll
+        for (int r = 0; r < 32; ++r) psum += pv[r];
+        l_i = l_i * alpha + psum;
+        if (__any(alpha != 1.0f)) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
+        }
+
+        // ---- O^T += V^T . P^T -------------------------------------------------
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            Frag pf;
+            cvt8<T>(&pv[8 * s], pf);     // slots j <-> regs 8*(s%2)+j of block s/2 == pv[8*s + j]
+#pragma unroll
+            for (int db = 0; db < 4; ++db) {
+                Frag vf;
+#pragma unroll
+                for (int jj = 0; jj < 2; ++jj) {
+                    const int row = 16 * s + 8 * jj + 4 * g + v_rd_rsub;
+                    const int chunk = (4 * db + v_rd_chunk) ^ ((row & 3) << 2);
+                    vf.s4[jj] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        (__attribute__((address_space(3))) short4_t *)(lds_v + row * ROW_BYTES + (chunk << 4) + v_rd_byte));
+                }
+                oacc[db] = Mma<T>::mfma(frag_as<T>(vf), frag_as<T>(pf), oacc[db]);
+            }
+        }
+        cur = nxt;
+    }
+
+    // ---- epilogue: O = O^T / l, store ------------------------------------------
+    float l_tot = l_i + __shfl_xor(l_i, 32);
+    const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+    if (qrow < p.n) {
+        const bool live = qrow < seqlen;
+        char *orow = o_base + (long long)qrow * p.os[2] * 2;
+#pragma unroll
+        for (int db = 0; db < 4; ++db)
+#pragma unroll
+            for (int rq = 0; rq < 4; ++rq) {
+                // d = 32*db + 8*rq + 4*g + 0..3
+                union { T e[4]; uint2 u; } out4;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) out4.e[e] = live ? (T)(oacc[db][rq * 4 + e] * inv) : (T)0.f;
+                *reinterpret_cast<uint2 *>(orow + (32 * db + 8 * rq + 4 * g) * 2) = out4.u;
+            }
+    }
+}
+
+int check_tensors(const minf_qkvo *t) {
+    if (!t || !t->q || !t->k || !t->v || !t->o) return MINF_ERR_INVALID_ARG;
+    if (t->batch < 0 || t->heads_q <= 0 || t->heads_kv <= 0 || t->n < 0) return MINF_ERR_INVALID_ARG;
+    if (t->heads_q % t->heads_kv != 0) return MINF_ERR_INVALID_ARG;
+    if (t->head_dim != HD) return MINF_ERR_UNSUPPORTED;
+    if (t->dtype != MINF_BF16 && t->dtype != MINF_F16) return MINF_ERR_UNSUPPORTED;
+    const void *ptrs[4] = {t->q, t->k, t->v, t->o};
+    const int64_t *strides[4] = {t->q_stride, t->k_stride, t->v_stride, t->o_stride};
+    for (int i = 0; i < 4; ++i) {
+        if (((uintptr_t)ptrs[i]) & 15) return MINF_ERR_ALIGNMENT;
+        for (int j = 0; j < 3; ++j)
+            if (strides[i][j] < 0 || (strides[i][j] & 7)) return MINF_ERR_ALIGNMENT;
+    }
+    return MINF_OK;
+}
+
+void fill_params(AttnParams &p, const minf_qkvo *t) {
+    p.q = (const char *)t->q; p.k = (const char *)t->k; p.v = (const char *)t->v; p.o = (char *)t->o;
+    for (int j = 0; j < 3; ++j) {
+        p.qs[j] = t->q_stride[j]; p.ks[j] = t->k_stride[j];
+        p.vs[j] = t->v_stride[j]; p.os[j] = t->o_stride[j];
+    }
+    p.batch = t->batch; p.hq = t->heads_q; p.hk = t->heads_kv; p.n = t->n;
+    p.seqlens = t->seqlens;
+    p.scale_log2 = t->sm_scale * 1.4426950408889634f;
+    p.rows = (t->n + BM - 1) / BM;
+    p.bc = p.bo = p.cc = p.ci = nullptr; p.nnz_s = p.nnz_v = 0;
+    p.bidx = nullptr; p.max_blocks = 0; p.bidx_rows = 0;
+    p.n_init = p.n_local = 0;
+    p.total_wg = (long long)t->batch * t->heads_q * p.rows;
+}
+
+template <int MODE> int launch(const AttnParams &p, int dtype, void *stream) {
+    if (p.total_wg == 0) return MINF_OK;
+    const long long per_xcd = (p.total_wg + 7) >> 3;
+    const long long grid = per_xcd * 8;
+    if (grid > 0x7fffffffLL) return MINF_ERR_UNSUPPORTED;
+    if (dtype == MINF_BF16)
+        hipLaunchKernelGGL((attn_fwd_kernel<__bf16, MODE>), dim3((unsigned)grid), dim3(NTHREADS), 0,
+                           (hipStream_t)stream, p);
+    else
+        hipLaunchKernelGGL((attn_fwd_kernel<_Float16, MODE>), dim3((unsigned)grid), dim3(NTHREADS), 0,
+                           (hipStream_t)stream, p);
+    return minf_launch_status();
+}
+
+}  // namespace
+
+extern "C" int minf_vs_attn_fwd(const minf_qkvo *t, const int32_t *block_count,
+                                const int32_t *block_offset, const int32_t *column_count,
+                                const int32_t *column_index, int rows, int nnz_s, int nnz_v,
+                                void *stream) {
+    int st = check_tensors(t);
+    if (st) return st;
+    if (!block_count || !block_offset || !column_count || !column_index) return MINF_ERR_INVALID_ARG;
+    if (nnz_s < 1 || nnz_v < 1) return MINF_ERR_INVALID_ARG;
+    AttnParams p;
+    fill_params(p, t);
+    if (rows != p.rows) return MINF_ERR_INVALID_ARG;
+    p.bc = block_count; p.bo = block_offset; p.cc = column_count; p.ci = column_index;
+    p.nnz_s = nnz_s; p.nnz_v = nnz_v;
+    return launch<MODE_VS>(p, t->dtype, stream);
+}
+
+extern "C" int minf_bs_attn_fwd(const minf_qkvo *t, const int32_t *block_index, int rows,
+                                int max_blocks, void *stream) {
+    int st = check_tensors(t);
+    if (st) return st;
+    if (!block_index || max_blocks < 1) return MINF_ERR_INVALID_ARG;
+    AttnParams p;
+    fill_params(p, t);
+    if (rows < p.rows) return MINF_ERR_INVALID_ARG;
+    // block_index may have more rows than ceil(n/64) (the reference pads n first)
+    p.bidx = block_index; p.max_blocks = max_blocks; p.bidx_rows = rows;
+    return launch<MODE_BS>(p, t->dtype, stream);
+}
+
+extern "C" int minf_ashape_attn_fwd(const minf_qkvo *t, int n_init, int n_local, void *stream) {
+    int st = check_tensors(t);
+    if (st) return st;
+    if (n_init < 0 || n_local < 1) return MINF_ERR_INVALID_ARG;
+    AttnParams p;
+    fill_params(p, t);
+    p.n_init = n_init; p.n_local = n_local;
+    return launch<MODE_ASHAPE>(p, t->dtype, stream);
+}
+
+extern "C" int minf_dense_attn_fwd(const minf_qkvo *t, void *stream) {
+    int st = check_tensors(t);
+    if (st) return st;
+    AttnParams p;
+    fill_params(p, t);
+    return launch<MODE_DENSE>(p, t->dtype, stream);
+}

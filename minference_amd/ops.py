@@ -1,0 +1,209 @@
+"""The three sparse prefill attention operators, host side.
+
+Same callables, argument names and defaults as the reference package
+(minference/__init__.py:9-11):
+
+* ``vertical_slash_sparse_attention``  minference/ops/pit_sparse_flash_attention_v2.py:195-242
+* ``block_sparse_attention``           minference/ops/block_sparse_flash_attention.py:169-186
+* ``streaming_forward``                minference/ops/streaming_kernel.py:611-646
+
+Inputs are ``[batch, heads, n, head_dim]`` GPU tensors (any strides); the
+result is a new tensor of the query's shape and dtype.  In addition to the
+reference, K/V may have fewer heads than Q (grouped-query attention) and are
+then read in place instead of being expanded.  All arithmetic runs in
+libminf_hip.so on the caller's current stream; torch is only used for memory,
+the index sort and (for the block-sparse index) nothing else.
+"""
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from . import _lib
+from .index import convert_vertical_slash_indexes
+
+_SUPPORTED_D = 128
+
+
+def _prep(t: torch.Tensor) -> torch.Tensor:
+    """16-byte aligned rows with unit head_dim stride (copies only if needed)."""
+    if t.stride(-1) != 1 or any(s % 8 for s in t.stride()[:-1]) or t.data_ptr() % 16:
+        t = t.contiguous()
+    return t
+
+
+def _check_qkv(q, k, v):
+    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
+        raise ValueError("q, k, v must be [batch, heads, n, head_dim]")
+    if not q.is_cuda:
+        raise RuntimeError("sparse attention operators need GPU tensors (there is no CPU path)")
+    if k.shape != v.shape or q.shape[0] != k.shape[0] or q.shape[2:] != k.shape[2:]:
+        raise ValueError(f"shape mismatch: q {tuple(q.shape)} k {tuple(k.shape)} v {tuple(v.shape)}")
+    if q.shape[1] % k.shape[1] != 0:
+        raise ValueError("query heads must be a multiple of key/value heads")
+    if not (q.dtype == k.dtype == v.dtype):
+        raise ValueError("q, k, v must share a dtype")
+
+
+class _Call:
+    """Holds the (possibly cast/padded) tensors of one operator call and the
+    filled ``minf_qkvo`` struct."""
+
+    def __init__(self, q, k, v, seqlens=None):
+        _check_qkv(q, k, v)
+        self.out_dtype = q.dtype
+        self.head_dim = q.shape[-1]
+        if q.dtype == torch.float32:
+            # the tile engine computes on 16-bit operands with fp32 accumulation
+            q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
+        elif q.dtype not in (torch.bfloat16, torch.float16):
+            raise ValueError(f"unsupported dtype {q.dtype}")
+        D = q.shape[-1]
+        if D > _SUPPORTED_D:
+            raise ValueError(f"head_dim {D} > {_SUPPORTED_D} is not supported")
+        if D < _SUPPORTED_D:
+            # zero columns change neither q.k nor the first D output columns
+            pad = _SUPPORTED_D - D
+            q = torch.nn.functional.pad(q, [0, pad])
+            k = torch.nn.functional.pad(k, [0, pad])
+            v = torch.nn.functional.pad(v, [0, pad])
+        self.q, self.k, self.v = _prep(q), _prep(k), _prep(v)
+        B, H, N, _ = self.q.shape
+        self.B, self.H, self.N, self.Hk = B, H, N, self.k.shape[1]
+        self.o = torch.empty((B, H, N, _SUPPORTED_D), dtype=self.q.dtype, device=q.device)
+        s = _lib.QKVO()
+        s.q, s.k, s.v, s.o = self.q.data_ptr(), self.k.data_ptr(), self.v.data_ptr(), self.o.data_ptr()
+        for name, t in (("q_stride", self.q), ("k_stride", self.k), ("v_stride", self.v), ("o_stride", self.o)):
+            getattr(s, name)[:] = list(t.stride()[:3])
+        s.batch, s.heads_q, s.heads_kv, s.n = B, H, self.Hk, N
+        s.head_dim = _SUPPORTED_D
+        s.dtype = _lib.MINF_BF16 if self.q.dtype == torch.bfloat16 else _lib.MINF_F16
+        self.seqlens = seqlens
+        s.seqlens = seqlens.data_ptr() if seqlens is not None else None
+        s.sm_scale = float(self.head_dim) ** -0.5
+        self.struct = s
+
+    @property
+    def ref(self):
+        return ctypes.byref(self.struct)
+
+    def result(self):
+        o = self.o
+        if self.head_dim != _SUPPORTED_D:
+            o = o[..., : self.head_dim]
+        if o.dtype != self.out_dtype:
+            o = o.to(self.out_dtype)
+        return o
+
+
+def vertical_slash_attention_from_index(query, key, value, block_count, block_offset,
+                                        column_count, column_index, seqlens=None):
+    """Mixed block + column sparse attention over prebuilt index tensors
+    (counterpart of _triton_mixed_sparse_attention, pit_sparse_flash_attention_v2.py:156-192)."""
+    c = _Call(query, key, value, seqlens)
+    rows = (c.N + 63) // 64
+    for t in (block_count, block_offset, column_count, column_index):
+        if t.dtype != torch.int32 or not t.is_contiguous():
+            raise ValueError("index tensors must be contiguous int32")
+    if tuple(block_count.shape) != (c.B, c.H, rows) or tuple(block_offset.shape[:3]) != (c.B, c.H, rows) \
+            or tuple(column_index.shape[:3]) != (c.B, c.H, rows):
+        raise ValueError("index tensors must be [batch, heads_q, ceil(n/64), ...]")
+    lib = _lib.load()
+    with torch.cuda.device(c.q.device):
+        st = lib.minf_vs_attn_fwd(c.ref, block_count.data_ptr(), block_offset.data_ptr(),
+                                  column_count.data_ptr(), column_index.data_ptr(), rows,
+                                  block_offset.shape[-1], column_index.shape[-1],
+                                  _lib.stream_ptr(c.q.device))
+    _lib.check(st, "minf_vs_attn_fwd")
+    return c.result()
+
+
+def vertical_slash_sparse_attention(query, key, value, v_idx, s_idx, block_size_M: int = 64,
+                                    block_size_N: int = 64):
+    """Vertical-slash sparse attention (pit_sparse_flash_attention_v2.py:195-242).
+
+    v_idx: key positions kept for every query, s_idx: diagonal offsets
+    (q_pos - k_pos) kept; any integer dtype, unsorted, shapes that reshape to
+    [batch, heads, nnz]."""
+    if block_size_M != 64 or block_size_N != 64:
+        raise ValueError("only 64x64 blocks are supported")
+    _check_qkv(query, key, value)
+    B, H, N, _ = query.shape
+    v_idx = v_idx.to(torch.int32).reshape((B, H, -1)).sort(dim=-1, descending=False)[0]
+    s_idx = s_idx.to(torch.int32).reshape((B, H, -1)).sort(dim=-1, descending=True)[0]
+    seqlens = torch.full((B,), N, dtype=torch.int32, device=query.device)
+    bc, bo, cc, ci = convert_vertical_slash_indexes(seqlens, v_idx, s_idx, N, block_size_M,
+                                                    block_size_N, zero_fill=False)
+    return vertical_slash_attention_from_index(query, key, value, bc, bo, cc, ci, seqlens)
+
+
+def block_sparse_attention_from_index(query, key, value, block_index):
+    """Block-sparse attention over a prebuilt [batch, heads, rows, max_blocks] int32 block
+    list (counterpart of _triton_block_sparse_attention, block_sparse_flash_attention.py:115-148)."""
+    c = _Call(query, key, value)
+    if block_index.dtype != torch.int32 or not block_index.is_contiguous() or block_index.dim() != 4:
+        raise ValueError("block_index must be a contiguous int32 [batch, heads, rows, max_blocks] tensor")
+    if block_index.shape[0] != c.B or block_index.shape[1] != c.H or block_index.shape[2] < (c.N + 63) // 64:
+        raise ValueError("block_index has the wrong batch/head/row sizes")
+    lib = _lib.load()
+    with torch.cuda.device(c.q.device):
+        st = lib.minf_bs_attn_fwd(c.ref, block_index.data_ptr(), block_index.shape[2],
+                                  block_index.shape[3], _lib.stream_ptr(c.q.device))
+    _lib.check(st, "minf_bs_attn_fwd")
+    return c.result()
+
+
+def _build_block_index(query, key, top_k, block_size_M=64, block_size_N=64, force_diag_first=False):
+    """Top-k key blocks per query block from mean-pooled Q/K
+    (block_sparse_flash_attention.py:151-166).  Pooling, scores and the top-k run in torch for
+    now (fp32); K/V heads are expanded only at pooled (1/64) size."""
+    B, H, N, D = query.shape
+    Hk = key.shape[1]
+    pad = block_size_M - (N & (block_size_M - 1))          # reference :178 (a full block if N%64==0)
+    def pool(x):
+        x = torch.nn.functional.pad(x.float(), [0, 0, 0, pad])
+        return x.reshape(x.shape[0], x.shape[1], -1, block_size_M, D).mean(dim=-2)
+    qp, kp = pool(query), pool(key)
+    if Hk != H:
+        kp = kp.repeat_interleave(H // Hk, dim=1)
+    R = qp.shape[2]
+    p = torch.einsum("bhmk,bhnk->bhmn", qp, kp)
+    ar = torch.arange(R, device=query.device)
+    p = p.masked_fill(ar[:, None] < ar[None, :], float("-inf"))
+    if force_diag_first:
+        p[..., ar, ar] = float("inf")
+        p[..., :, 0] = float("inf")
+    top_k = min(top_k, R)
+    order = torch.argsort(p, dim=-1, descending=True, stable=True)[..., :top_k]
+    return order.to(torch.int32).sort(dim=-1).values.contiguous()
+
+
+def block_sparse_attention(query, key, value, top_k: int, block_size_M: int = 64, block_size_N: int = 64):
+    """Top-k block-sparse attention (block_sparse_flash_attention.py:169-186)."""
+    if block_size_M != 64 or block_size_N != 64:
+        raise ValueError("only 64x64 blocks are supported")
+    _check_qkv(query, key, value)
+    block_index = _build_block_index(query, key, top_k, block_size_M, block_size_N)
+    return block_sparse_attention_from_index(query, key, value, block_index)
+
+
+def streaming_forward(q, k, v, n_init: int, n_local: int):
+    """A-shape attention: n_init sink tokens + a sliding window of n_local
+    (streaming_kernel.py:611-646), in one pass."""
+    c = _Call(q, k, v)
+    lib = _lib.load()
+    with torch.cuda.device(c.q.device):
+        st = lib.minf_ashape_attn_fwd(c.ref, int(n_init), int(n_local), _lib.stream_ptr(c.q.device))
+    _lib.check(st, "minf_ashape_attn_fwd")
+    return c.result()
+
+
+def dense_causal_attention(q, k, v):
+    """Dense causal attention on the same tile engine (comparator for speed-up figures)."""
+    c = _Call(q, k, v)
+    lib = _lib.load()
+    with torch.cuda.device(c.q.device):
+        st = lib.minf_dense_attn_fwd(c.ref, _lib.stream_ptr(c.q.device))
+    _lib.check(st, "minf_dense_attn_fwd")
+    return c.result()
