@@ -213,26 +213,26 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
     const int ld_c = tid & 15;       // 16-byte chunk in the row
     uint4 kreg[8], vreg[8];
 
+    // Rows that do not exist (past seqlen, or padding of a gathered tile) are read from a
+    // clamped, valid address instead of being zeroed: their scores are always masked to
+    // -inf below, so their probabilities are exactly 0 and K/V contents never matter.
     auto issue_loads = [&](const Tile &t) {
+        int tok[8];
+        if (MODE == MODE_VS && t.gathered) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int r = i * 8 + ld_r;
+                tok[i] = p.ci[ridx * p.nnz_v + t.start + min(r, t.nvalid - 1)];
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) tok[i] = t.start + i * 8 + ld_r;
+        }
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            const int r = i * 8 + ld_r;
-            int tok;
-            bool ok;
-            if (MODE == MODE_VS && t.gathered) {
-                ok = r < t.nvalid;
-                tok = ok ? p.ci[ridx * p.nnz_v + t.start + r] : 0;
-            } else {
-                tok = t.start + r;
-                ok = tok < seqlen;
-                if (!ok) tok = 0;
-            }
-            kreg[i] = *reinterpret_cast<const uint4 *>(k_base + tok * k_row + ld_c * 16);
-            vreg[i] = *reinterpret_cast<const uint4 *>(v_base + tok * v_row + ld_c * 16);
-            if (!ok) {
-                kreg[i] = make_uint4(0, 0, 0, 0);
-                vreg[i] = make_uint4(0, 0, 0, 0);
-            }
+            const int tk = max(0, min(tok[i], seqlen - 1));
+            kreg[i] = *reinterpret_cast<const uint4 *>(k_base + tk * k_row + ld_c * 16);
+            vreg[i] = *reinterpret_cast<const uint4 *>(v_base + tk * v_row + ld_c * 16);
         }
     };
     auto store_lds = [&]() {
@@ -291,37 +291,40 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
         }
 
         // ---- mask -----------------------------------------------------------
-        // element (blk, r) of this lane is token 32*blk + 8*(r/4) + 4*g + r%4
+        // element (blk, r) of this lane is tile-local key tk = tkc + 4*g with the compile-time
+        // part tkc = 32*blk + 8*(r/4) + r%4.  keep <=> tk <= hi && (tk > wlo || tk < slim).
         bool need_mask;
         const int wrow_lo = row0 + wave * 32, wrow_hi = wrow_lo + 31;
+        int hi, wlo = -1, slim = 0;      // per-lane bounds on tkc (4*g already subtracted)
         if (MODE == MODE_VS && cur.gathered) {
             need_mask = cur.nvalid < BN;
-        } else if constexpr (MODE == MODE_ASHAPE) {
-            const int c_lo = cur.start, c_hi = cur.start + BN - 1;
-            const bool causal_ok = c_hi <= wrow_lo && c_hi < seqlen;
-            const bool in_window = (wrow_hi - c_lo) < p.n_local;
-            const bool in_sink = c_hi < p.n_init;
-            need_mask = !(causal_ok && (in_window || in_sink));
+            hi = cur.nvalid - 1 - 4 * g;
         } else {
-            need_mask = (cur.start + BN - 1 > wrow_lo) || (cur.start + BN > seqlen);
+            hi = min(qrow, seqlen - 1) - cur.start - 4 * g;
+            if constexpr (MODE == MODE_ASHAPE) {
+                const int c_lo = cur.start, c_hi = cur.start + BN - 1;
+                const bool causal_ok = c_hi <= wrow_lo && c_hi < seqlen;
+                const bool in_window = (wrow_hi - c_lo) < p.n_local;
+                const bool in_sink = c_hi < p.n_init;
+                need_mask = !(causal_ok && (in_window || in_sink));
+                wlo = qrow - cur.start - p.n_local - 4 * g;
+                slim = p.n_init - cur.start - 4 * g;
+            } else {
+                need_mask = (cur.start + BN - 1 > wrow_lo) || (cur.start + BN > seqlen);
+            }
         }
         if (need_mask) {
 #pragma unroll
-            for (int blk = 0; blk < 2; ++blk)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int tk = 32 * blk + 8 * (r >> 2) + 4 * g + (r & 3);
-                    bool keep;
-                    if (MODE == MODE_VS && cur.gathered) {
-                        keep = tk < cur.nvalid;
-                    } else {
-                        const int c = cur.start + tk;
-                        keep = (c <= qrow) && (c < seqlen);
-                        if constexpr (MODE == MODE_ASHAPE)
-                            keep = keep && ((qrow - c) < p.n_local || c < p.n_init);
-                    }
-                    if (!keep) { if (blk == 0) s0[r] = -INFINITY; else s1[r] = -INFINITY; }
+            for (int r = 0; r < 16; ++r) {
+                const int tkc = 8 * (r >> 2) + (r & 3);
+                bool k0 = tkc <= hi, k1 = (tkc + 32) <= hi;
+                if constexpr (MODE == MODE_ASHAPE) {
+                    k0 = k0 & ((tkc > wlo) | (tkc < slim));
+                    k1 = k1 & (((tkc + 32) > wlo) | ((tkc + 32) < slim));
                 }
+                s0[r] = k0 ? s0[r] : -INFINITY;
+                s1[r] = k1 ? s1[r] : -INFINITY;
+            }
         }
 
         // ---- online softmax (exp2 domain) -------------------------------------
