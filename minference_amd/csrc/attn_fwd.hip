@@ -29,6 +29,9 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(short)))) short short4_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
+// native vectors, not HIP's u32x4_t/u32x2_t structs: arrays of those are not promoted to registers
+typedef __attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned u32x4_t;
+typedef __attribute__((__vector_size__(2 * sizeof(unsigned)))) unsigned u32x2_t;
 
 enum { MODE_VS = 0, MODE_BS = 1, MODE_ASHAPE = 2, MODE_DENSE = 3 };
 
@@ -72,7 +75,7 @@ template <> struct Mma<_Float16> {
 };
 
 union Frag {
-    uint4 u;
+    u32x4_t u;
     bf16x8_t b;
     f16x8_t h;
     short4_t s4[2];
@@ -182,7 +185,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
         // row block past the sequence: zeros (16 B per lane-step)
         for (int i = tid; i < BM * 16; i += NTHREADS) {
             int r = row0 + (i >> 4);
-            if (r < p.n) *reinterpret_cast<uint4 *>(o_base + (long long)r * p.os[2] * 2 + (i & 15) * 16) = make_uint4(0, 0, 0, 0);
+            if (r < p.n) *reinterpret_cast<u32x4_t *>(o_base + (long long)r * p.os[2] * 2 + (i & 15) * 16) = u32x4_t{0u, 0u, 0u, 0u};
         }
         return;
     }
@@ -200,8 +203,8 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
         const char *qp = q_base + (long long)(ok ? qrow : row0) * p.qs[2] * 2 + g * 16;
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) {
-            qf[ks].u = *reinterpret_cast<const uint4 *>(qp + ks * 32);
-            if (!ok) qf[ks].u = make_uint4(0, 0, 0, 0);
+            qf[ks].u = *reinterpret_cast<const u32x4_t *>(qp + ks * 32);
+            if (!ok) qf[ks].u = u32x4_t{0u, 0u, 0u, 0u};
         }
     }
 
@@ -211,7 +214,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
     // ---- global -> register staging: thread covers rows i*8 + tid/16, chunk tid%16
     const int ld_r = tid >> 4;       // 0..7
     const int ld_c = tid & 15;       // 16-byte chunk in the row
-    uint4 kreg[8], vreg[8];
+    u32x4_t kreg[8], vreg[8];
 
     // Rows that do not exist (past seqlen, or padding of a gathered tile) are read from a
     // clamped, valid address instead of being zeroed: their scores are always masked to
@@ -231,16 +234,16 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const int tk = max(0, min(tok[i], seqlen - 1));
-            kreg[i] = *reinterpret_cast<const uint4 *>(k_base + tk * k_row + ld_c * 16);
-            vreg[i] = *reinterpret_cast<const uint4 *>(v_base + tk * v_row + ld_c * 16);
+            kreg[i] = *reinterpret_cast<const u32x4_t *>(k_base + tk * k_row + ld_c * 16);
+            vreg[i] = *reinterpret_cast<const u32x4_t *>(v_base + tk * v_row + ld_c * 16);
         }
     };
     auto store_lds = [&]() {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const int r = i * 8 + ld_r;
-            *reinterpret_cast<uint4 *>(lds_k + r * ROW_BYTES + ((ld_c ^ (r & 15)) << 4)) = kreg[i];
-            *reinterpret_cast<uint4 *>(lds_v + r * ROW_BYTES + ((ld_c ^ ((r & 3) << 2)) << 4)) = vreg[i];
+            *reinterpret_cast<u32x4_t *>(lds_k + r * ROW_BYTES + ((ld_c ^ (r & 15)) << 4)) = kreg[i];
+            *reinterpret_cast<u32x4_t *>(lds_v + r * ROW_BYTES + ((ld_c ^ ((r & 3) << 2)) << 4)) = vreg[i];
         }
     };
 
@@ -284,8 +287,8 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
         for (int ks = 0; ks < 8; ++ks) {
             const int x = 2 * ks + g;
             Frag a0, a1;
-            a0.u = *reinterpret_cast<const uint4 *>(lds_k + k_rd_row * ROW_BYTES + ((x ^ (k_rd_row & 15)) << 4));
-            a1.u = *reinterpret_cast<const uint4 *>(lds_k + (32 + k_rd_row) * ROW_BYTES + ((x ^ (k_rd_row & 15)) << 4));
+            a0.u = *reinterpret_cast<const u32x4_t *>(lds_k + k_rd_row * ROW_BYTES + ((x ^ (k_rd_row & 15)) << 4));
+            a1.u = *reinterpret_cast<const u32x4_t *>(lds_k + (32 + k_rd_row) * ROW_BYTES + ((x ^ (k_rd_row & 15)) << 4));
             s0 = Mma<T>::mfma(frag_as<T>(a0), frag_as<T>(qf[ks]), s0);
             s1 = Mma<T>::mfma(frag_as<T>(a1), frag_as<T>(qf[ks]), s1);
         }
@@ -387,10 +390,10 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
 #pragma unroll
             for (int rq = 0; rq < 4; ++rq) {
                 // d = 32*db + 8*rq + 4*g + 0..3
-                union { T e[4]; uint2 u; } out4;
+                union { T e[4]; u32x2_t u; } out4;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) out4.e[e] = live ? (T)(oacc[db][rq * 4 + e] * inv) : (T)0.f;
-                *reinterpret_cast<uint2 *>(orow + (32 * db + 8 * rq + 4 * g) * 2) = out4.u;
+                *reinterpret_cast<u32x2_t *>(orow + (32 * db + 8 * rq + 4 * g) * 2) = out4.u;
             }
     }
 }
