@@ -20,6 +20,7 @@
  */
 #ifndef MINF_HIP_H
 #define MINF_HIP_H
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -136,6 +137,43 @@ int minf_ashape_attn_fwd(const minf_qkvo *t, int n_init, int n_local, void *stre
  * minference/modules/minference_forward.py:666).
  */
 int minf_dense_attn_fwd(const minf_qkvo *t, void *stream);
+
+/*
+ * Online vertical/slash pattern estimation.  Replaces the torch op chain of
+ * vertical_and_slash_kernel (reference
+ * minference/modules/minference_forward.py:599-610) and sum_all_diagonal_matrix
+ * (:110-116), batched over heads:
+ *   P = softmax(q[:, :, -last_q:] . k^T * sm_scale) with the trailing
+ *   last_q x last_q corner causally masked (fp32);
+ *   vertical[b,h,c] = sum_i P[i,c];  slash[b,h,j] = sum_i P[i, i+j+1-last_q]
+ *   (slash[j] is the mass on the diagonal with offset n-1-j);
+ *   then vertical[..., :force_vertical] = +inf and slash[..., n-force_slash:] = +inf
+ *   (the reference forces 30 and 100; pass 0 to get the raw sums).
+ * q [batch, heads_q, n, 128], k [batch, heads_kv, n, 128] as base pointer +
+ * element strides {batch, head, token}; last_q <= 64 (clamped to n).
+ * vertical, slash: [batch, heads_q, n] fp32, contiguous.
+ * workspace: at least minf_vs_estimate_workspace_bytes() bytes, 16-byte aligned.
+ */
+size_t minf_vs_estimate_workspace_bytes(int batch, int heads_q, int n);
+int minf_vs_estimate(const void *q, const void *k, const int64_t *q_stride,
+                     const int64_t *k_stride, int batch, int heads_q, int heads_kv, int n,
+                     int head_dim, int dtype, float sm_scale, int last_q, int force_vertical,
+                     int force_slash, float *vertical, float *slash, void *workspace,
+                     size_t workspace_bytes, void *stream);
+
+/*
+ * Indices of the k largest entries of each fp32 row, written in ASCENDING
+ * INDEX order (ties at the k-th value: lowest index first).  Replaces
+ * torch.topk(...).indices followed by the sort in the op wrapper (reference
+ * minference/modules/minference_forward.py:607,612 and
+ * minference/ops/pit_sparse_flash_attention_v2.py:218-219).
+ * scores [rows, n] with row_stride elements between rows; out [rows, min(k,n)]
+ * with out_stride.  reverse_base < 0: out = index; otherwise out =
+ * reverse_base - index (slash: reverse_base = n-1 turns ascending j into
+ * descending diagonal offsets, the order the index builder wants).
+ */
+int minf_topk_indices(const float *scores, int rows, int n, int64_t row_stride, int k,
+                      int32_t *out, int64_t out_stride, int reverse_base, void *stream);
 
 #ifdef __cplusplus
 }

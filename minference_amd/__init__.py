@@ -12,7 +12,13 @@ from .ops import (block_sparse_attention, block_sparse_attention_from_index, den
                   streaming_forward, vertical_slash_attention_from_index,
                   vertical_slash_sparse_attention)
 
+from .estimate import estimate_vertical_slash, topk_indices, vertical_slash_scores
+from .prefill import (load_best_pattern, minference_prefill_forward, minference_prefill_kernel,
+                      vertical_slash_prefill)
+
 __all__ = [
+    "estimate_vertical_slash", "vertical_slash_scores", "topk_indices", "vertical_slash_prefill",
+    "minference_prefill_forward", "minference_prefill_kernel", "load_best_pattern",
     "vertical_slash_sparse_attention", "block_sparse_attention", "streaming_forward",
     "convert_vertical_slash_indexes", "vertical_slash_attention_from_index",
     "block_sparse_attention_from_index", "dense_causal_attention",

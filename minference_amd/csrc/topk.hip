@@ -1,0 +1,124 @@
+// Top-k index selection over fp32 score rows for gfx950 (vertical / slash
+// candidates: k = 1000 / 6096 of up to ~10^6 entries per head).
+//
+// One 1024-thread workgroup per row:
+//   1. MSB-first radix select (4 x 8 bits, LDS histogram) finds the exact value
+//      T of the k-th largest entry and how many entries equal to T are needed;
+//   2. every wavefront counts, over its contiguous slice, entries > T and == T;
+//   3. the slices are scanned and the selected indices are written in
+//      ASCENDING INDEX order with ballot prefix counts (entries > T always,
+//      entries == T lowest index first until k are out).
+// Ties are therefore resolved towards the lowest index (torch.topk, which the
+// reference uses at minference/modules/minference_forward.py:607,612, leaves the
+// tie order unspecified), and the output needs no sort before the index
+// builder.  With reverse_base >= 0 the value written is reverse_base - index
+// (slash: diagonal offset = N-1-j, so ascending j gives descending offsets).
+#include "minf_common.h"
+
+namespace {
+
+constexpr int TK_THREADS = 1024;
+constexpr int TK_WAVES = TK_THREADS / 64;
+
+__device__ __forceinline__ unsigned order_key(float x) {
+    unsigned u = __float_as_uint(x);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);   // monotone for all finite/inf floats
+}
+
+__global__ __launch_bounds__(TK_THREADS) void topk_kernel(const float *__restrict__ scores,
+                                                           long long row_stride, int n, int k,
+                                                           int32_t *__restrict__ out,
+                                                           long long out_stride, int reverse_base) {
+    __shared__ unsigned hist[256];
+    __shared__ unsigned sh_prefix, sh_need;
+    __shared__ int wave_gt[TK_WAVES], wave_eq[TK_WAVES];
+
+    const float *x = scores + (long long)blockIdx.x * row_stride;
+    int32_t *o = out + (long long)blockIdx.x * out_stride;
+    const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+    if (k >= n) {                    // everything is selected
+        for (int i = tid; i < n; i += TK_THREADS) o[i] = reverse_base >= 0 ? reverse_base - i : i;
+        return;
+    }
+
+    // ---- 1. radix select --------------------------------------------------
+    unsigned prefix = 0, mask = 0;
+    unsigned need = (unsigned)k;     // rank (from the top) inside the current prefix bucket
+    for (int shift = 24; shift >= 0; shift -= 8) {
+        if (tid < 256) hist[tid] = 0;
+        __syncthreads();
+        for (int i = tid; i < n; i += TK_THREADS) {
+            const unsigned u = order_key(x[i]);
+            if ((u & mask) == prefix) atomicAdd(&hist[(u >> shift) & 255u], 1u);
+        }
+        __syncthreads();
+        if (tid == 0) {
+            unsigned cum = 0;
+            int b = 255;
+            for (; b > 0; --b) {
+                if (cum + hist[b] >= need) break;
+                cum += hist[b];
+            }
+            sh_prefix = prefix | ((unsigned)b << shift);
+            sh_need = need - cum;
+        }
+        __syncthreads();
+        prefix = sh_prefix;
+        need = sh_need;
+        mask |= 255u << shift;
+    }
+    const unsigned T = prefix;       // key of the k-th largest; `need` entries equal to T are taken
+
+    // ---- 2. per-wave counts over contiguous slices --------------------------
+    const int per_wave = ((n + TK_WAVES * 64 - 1) / (TK_WAVES * 64)) * 64;
+    const int begin = wave * per_wave;
+    const int end = min(n, begin + per_wave);
+    int cgt = 0, ceq = 0;
+    for (int i = begin + lane; i < end; i += 64) {
+        const unsigned u = order_key(x[i]);
+        cgt += u > T;
+        ceq += u == T;
+    }
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) {
+        cgt += __shfl_xor(cgt, d);
+        ceq += __shfl_xor(ceq, d);
+    }
+    if (lane == 0) { wave_gt[wave] = cgt; wave_eq[wave] = ceq; }
+    __syncthreads();
+    int gt_before = 0, eq_before = 0;
+    for (int wv = 0; wv < wave; ++wv) { gt_before += wave_gt[wv]; eq_before += wave_eq[wv]; }
+
+    // ---- 3. ordered emit ---------------------------------------------------
+    const int r = (int)need;
+    for (int base = begin; base < end; base += 64) {
+        const int i = base + lane;
+        unsigned u = 0;
+        bool gt = false, eq = false;
+        if (i < end) { u = order_key(x[i]); gt = u > T; eq = u == T; }
+        const uint64_t mg = __ballot(gt), me = __ballot(eq);
+        const uint64_t lt = minf_lanemask_lt();
+        const int g_here = gt_before + __builtin_popcountll(mg & lt);
+        const int e_here = eq_before + __builtin_popcountll(me & lt);
+        const bool take = gt || (eq && e_here < r);
+        if (take) {
+            const int pos = g_here + min(e_here, r);
+            o[pos] = reverse_base >= 0 ? reverse_base - i : i;
+        }
+        gt_before += __builtin_popcountll(mg);
+        eq_before += __builtin_popcountll(me);
+    }
+}
+
+}  // namespace
+
+extern "C" int minf_topk_indices(const float *scores, int rows, int n, int64_t row_stride, int k,
+                                 int32_t *out, int64_t out_stride, int reverse_base, void *stream) {
+    if (!scores || !out || rows < 0 || n <= 0 || k <= 0) return MINF_ERR_INVALID_ARG;
+    if (row_stride < n || out_stride < (k < n ? k : n)) return MINF_ERR_INVALID_ARG;
+    if (rows == 0) return MINF_OK;
+    hipLaunchKernelGGL(topk_kernel, dim3((unsigned)rows), dim3(TK_THREADS), 0, (hipStream_t)stream,
+                       scores, (long long)row_stride, n, k, out, (long long)out_stride, reverse_base);
+    return minf_launch_status();
+}

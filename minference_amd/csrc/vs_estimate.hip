@@ -1,0 +1,348 @@
+// Online vertical/slash pattern estimation for gfx950.
+//
+// For every (batch, query head): P = softmax(Q[-last_q:] . K^T / sqrt(d)) with the
+// trailing last_q x last_q corner causally masked, then
+//   vertical[c] = sum_i P[i, c]                      (column sums)
+//   slash[j]    = sum_i P[i, i + j + 1 - last_q]     (diagonal sums; j <-> offset N-1-j)
+// (reference minference/modules/minference_forward.py:599-614 and :110-116).
+//
+// Two sweeps over K, both on v_mfma_f32_32x32x16 with K and Q fragments read
+// straight from global memory in operand layout (no LDS staging; the same
+// registers serve as A or B operand, so swapping the operands transposes the
+// score tile for free):
+//   stats  : S^T = K.Q^T  -> lane <-> query row: running max / sum-of-exp in
+//            registers, one (max, sum) pair per row per 1024-key chunk;
+//   reduce : combine the chunk pairs into M_i = max_i + log2(sum_i);
+//   scores : S = Q.K^T    -> lane <-> key: p = exp2(s - M_row); column sums are
+//            in-lane adds (+ one cross-half shuffle), diagonal sums go through
+//            LDS float atomics into a per-chunk window that is written out whole;
+//   finalize: stitch the chunk windows together (each diagonal gets at most two
+//            pieces, added in a fixed order) and apply the forced +inf entries.
+// All arithmetic is fp32 on 16-bit inputs (the reference rounds q.k to bf16
+// before its fp32 softmax).
+#include "minf_common.h"
+#include <math.h>
+
+namespace {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
+typedef __attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned u32x4_t;
+
+constexpr int LQ = 64;          // query rows held per head (last_q <= LQ)
+constexpr int KC = 1024;        // keys per workgroup
+constexpr int EST_THREADS = 256;
+constexpr int WIN = KC + LQ;    // diagonal window of one chunk
+constexpr int HD = 128;
+
+struct EstParams {
+    const char *q, *k;
+    long long qs[3], ks[3];     // element strides batch, head, token
+    int batch, hq, hk, n, last_q;
+    float scale_log2;
+    int nchunks;
+    float *stats;               // [B, Hq, nchunks, LQ, 2]
+    float *rowstat;             // [B, Hq, LQ]
+    float *win;                 // [B, Hq, nchunks, WIN]
+    float *vertical, *slash;    // [B, Hq, N]
+    int force_v, force_s;
+    long long total_wg;
+};
+
+union Frag {
+    u32x4_t u;
+    bf16x8_t b;
+    f16x8_t h;
+};
+
+template <typename T> __device__ __forceinline__ f32x16_t mma(const Frag &a, const Frag &b, f32x16_t c);
+template <> __device__ __forceinline__ f32x16_t mma<__bf16>(const Frag &a, const Frag &b, f32x16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.b, b.b, c, 0, 0, 0);
+}
+template <> __device__ __forceinline__ f32x16_t mma<_Float16>(const Frag &a, const Frag &b, f32x16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a.h, b.h, c, 0, 0, 0);
+}
+
+struct WgId { int b, h, hkv, chunk; bool valid; };
+
+// XCD-aware order: (batch, kv head, chunk, query head in group) contiguous per XCD
+__device__ __forceinline__ WgId decode_wg(const EstParams &p) {
+    WgId w;
+    const long long per_xcd = (p.total_wg + 7) >> 3;
+    const long long logical = (long long)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    w.valid = logical < p.total_wg;
+    const int group = p.hq / p.hk;
+    long long rest = logical;
+    const int hin = (int)(rest % group); rest /= group;
+    w.chunk = (int)(rest % p.nchunks); rest /= p.nchunks;
+    w.hkv = (int)(rest % p.hk);
+    w.b = (int)(rest / p.hk);
+    w.h = w.hkv * group + hin;
+    return w;
+}
+
+// Q fragments of one head: rows N-last_q+i, i = 32*blk + lane%32, d = 16*ks + 8*(lane/32) + 0..7
+__device__ __forceinline__ void load_q(const EstParams &p, const WgId &w, int lane, Frag (&qf)[2][8]) {
+    const int l32 = lane & 31, g = lane >> 5;
+    const char *qb = p.q + ((long long)w.b * p.qs[0] + (long long)w.h * p.qs[1]) * 2;
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk) {
+        const int i = 32 * blk + l32;
+        const int row = min(max(p.n - p.last_q + i, 0), p.n - 1);
+        const char *rp = qb + (long long)row * p.qs[2] * 2 + g * 16;
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) qf[blk][ks].u = *reinterpret_cast<const u32x4_t *>(rp + ks * 32);
+    }
+}
+
+// K fragments of one 32-key block starting at key c0 (rows clamped to n-1)
+__device__ __forceinline__ void load_k(const EstParams &p, const char *kb, int c0, int lane, Frag (&kf)[8]) {
+    const int l32 = lane & 31, g = lane >> 5;
+    const int row = min(c0 + l32, p.n - 1);
+    const char *rp = kb + (long long)row * p.ks[2] * 2 + g * 16;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) kf[ks].u = *reinterpret_cast<const u32x4_t *>(rp + ks * 32);
+}
+
+// ---------------------------------------------------------------- stats sweep
+template <typename T>
+__global__ __launch_bounds__(EST_THREADS) void est_stats_kernel(const EstParams p) {
+    __shared__ float lds_m[4][LQ], lds_l[4][LQ];
+    const WgId w = decode_wg(p);
+    if (!w.valid) return;
+    const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, g = lane >> 5;
+    const char *kb = p.k + ((long long)w.b * p.ks[0] + (long long)w.hkv * p.ks[1]) * 2;
+
+    Frag qf[2][8];
+    load_q(p, w, lane, qf);
+
+    // lane <-> query rows i = l32 and 32 + l32; regs <-> keys 8*(r/4) + 4*g + r%4 of the block
+    float m_run[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.f, 0.f};
+    const int key_begin = w.chunk * KC + wave * (KC / 4);
+    const int qpos0 = p.n - p.last_q;          // absolute position of query row 0
+    Frag kf[8];
+    for (int blk = 0; blk < KC / 4 / 32; ++blk) {
+        const int c0 = key_begin + blk * 32;
+        if (c0 >= p.n) break;
+        load_k(p, kb, c0, lane, kf);
+        f32x16_t st[2];
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) st[nb][r] = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks) st[nb] = mma<T>(kf[ks], qf[nb][ks], st[nb]);
+        }
+        const bool edge = c0 + 31 > qpos0 || c0 + 32 > p.n;
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) {
+            const int i = 32 * nb + l32;
+            // key c is visible to row i iff c <= qpos0 + i, c < n, i < last_q
+            const int hi = (i < p.last_q ? min(qpos0 + i, p.n - 1) : -1) - c0 - 4 * g;
+            float mx = -INFINITY;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int tkc = 8 * (r >> 2) + (r & 3);
+                float s = st[nb][r] * p.scale_log2;
+                if (edge) s = (tkc <= hi) ? s : -INFINITY;
+                st[nb][r] = s;
+                mx = fmaxf(mx, s);
+            }
+            const float m_new = fmaxf(m_run[nb], mx);
+            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+            float sum = 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sum += __builtin_amdgcn_exp2f(st[nb][r] - m_use);
+            l_run[nb] = l_run[nb] * __builtin_amdgcn_exp2f(m_run[nb] - m_use) + sum;
+            m_run[nb] = m_new;
+        }
+    }
+    // merge the two lane halves, then the 4 waves
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) {
+        const float mo = __shfl_xor(m_run[nb], 32), lo = __shfl_xor(l_run[nb], 32);
+        const float m_new = fmaxf(m_run[nb], mo);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        l_run[nb] = l_run[nb] * __builtin_amdgcn_exp2f(m_run[nb] - m_use) + lo * __builtin_amdgcn_exp2f(mo - m_use);
+        m_run[nb] = m_new;
+        if (g == 0) {
+            lds_m[wave][32 * nb + l32] = m_run[nb];
+            lds_l[wave][32 * nb + l32] = l_run[nb];
+        }
+    }
+    __syncthreads();
+    if (tid < LQ) {
+        float m = lds_m[0][tid], l = lds_l[0][tid];
+#pragma unroll
+        for (int wv = 1; wv < 4; ++wv) {
+            const float mo = lds_m[wv][tid], lo = lds_l[wv][tid];
+            const float m_new = fmaxf(m, mo);
+            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+            l = l * __builtin_amdgcn_exp2f(m - m_use) + lo * __builtin_amdgcn_exp2f(mo - m_use);
+            m = m_new;
+        }
+        float *dst = p.stats + ((((long long)w.b * p.hq + w.h) * p.nchunks + w.chunk) * LQ + tid) * 2;
+        dst[0] = m;
+        dst[1] = l;
+    }
+}
+
+// ------------------------------------------------------------- chunk reduction
+__global__ __launch_bounds__(LQ) void est_reduce_kernel(const EstParams p) {
+    const long long bh = blockIdx.x;
+    const int i = (int)threadIdx.x;
+    const float *src = p.stats + (bh * p.nchunks * LQ + i) * 2;
+    float m = -INFINITY, l = 0.f;
+    for (int c = 0; c < p.nchunks; ++c) {
+        const float mo = src[(long long)c * LQ * 2], lo = src[(long long)c * LQ * 2 + 1];
+        const float m_new = fmaxf(m, mo);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        l = l * __builtin_amdgcn_exp2f(m - m_use) + lo * __builtin_amdgcn_exp2f(mo - m_use);
+        m = m_new;
+    }
+    // rows that do not exist (i >= last_q) get +inf so that every probability is 0
+    p.rowstat[bh * LQ + i] = (i < p.last_q && l > 0.f) ? m + __builtin_amdgcn_logf(l) : INFINITY;
+}
+
+// --------------------------------------------------------------- scores sweep
+template <typename T>
+__global__ __launch_bounds__(EST_THREADS) void est_scores_kernel(const EstParams p) {
+    __shared__ float lds_win[WIN];
+    const WgId w = decode_wg(p);
+    if (!w.valid) return;
+    const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, g = lane >> 5;
+    const char *kb = p.k + ((long long)w.b * p.ks[0] + (long long)w.hkv * p.ks[1]) * 2;
+    const long long bh = (long long)w.b * p.hq + w.h;
+
+    for (int i = tid; i < WIN; i += EST_THREADS) lds_win[i] = 0.f;
+
+    Frag qf[2][8];
+    load_q(p, w, lane, qf);
+    // lane <-> key; reg r of block mb <-> query row i = 32*mb + 8*(r/4) + 4*g + r%4
+    float mrow[2][16];
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+            mrow[mb][r] = p.rowstat[bh * LQ + 32 * mb + 8 * (r >> 2) + 4 * g + (r & 3)];
+    __syncthreads();
+
+    const int chunk0 = w.chunk * KC;
+    const int key_begin = chunk0 + wave * (KC / 4);
+    const int qpos0 = p.n - p.last_q;
+    float *vout = p.vertical + bh * p.n;
+    Frag kf[8];
+    for (int blk = 0; blk < KC / 4 / 32; ++blk) {
+        const int c0 = key_begin + blk * 32;
+        if (c0 >= p.n) break;
+        load_k(p, kb, c0, lane, kf);
+        const int c = c0 + l32;                 // this lane's key
+        const bool edge = c0 + 31 > qpos0 || c0 + 32 > p.n;
+        float colsum = 0.f;
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb) {
+            f32x16_t s;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s[r] = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks) s = mma<T>(qf[mb][ks], kf[ks], s);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int i = 32 * mb + 8 * (r >> 2) + 4 * g + (r & 3);
+                float pr = __builtin_amdgcn_exp2f(fmaf(s[r], p.scale_log2, -mrow[mb][r]));
+                if (edge) pr = (c <= qpos0 + i && c < p.n) ? pr : 0.f;
+                colsum += pr;
+                // diagonal index j = c + (last_q - 1 - i); window position j - chunk0
+                // (rows i >= last_q carry pr == 0; their position is clamped into the window)
+                atomicAdd(&lds_win[max(c - chunk0 + (p.last_q - 1 - i), 0)], pr);
+            }
+        }
+        colsum += __shfl_xor(colsum, 32);
+        if (g == 0 && c < p.n) vout[c] = colsum;
+    }
+    __syncthreads();
+    float *wout = p.win + (bh * p.nchunks + w.chunk) * WIN;
+    for (int i = tid; i < WIN; i += EST_THREADS) wout[i] = lds_win[i];
+}
+
+// ------------------------------------------------------------------- finalize
+__global__ __launch_bounds__(256) void est_finalize_kernel(const EstParams p) {
+    const long long bh = blockIdx.y;
+    const int j = (int)(blockIdx.x * 256 + threadIdx.x);
+    if (j >= p.n) return;
+    const int c = j / KC, off = j - c * KC;
+    const float *wbase = p.win + bh * p.nchunks * WIN;
+    // diagonal j lives at window position `off` of chunk c and, when off < LQ, also at
+    // position KC + off of chunk c-1 (keys of the previous chunk seen by later rows)
+    float v = wbase[(long long)c * WIN + off];
+    if (c > 0 && off < LQ) v = wbase[(long long)(c - 1) * WIN + KC + off] + v;
+    if (p.force_s > 0 && j >= p.n - p.force_s) v = INFINITY;
+    p.slash[bh * p.n + j] = v;
+    if (j < p.force_v) p.vertical[bh * p.n + j] = INFINITY;
+}
+
+int fill(EstParams &p, const void *q, const void *k, const int64_t *q_stride, const int64_t *k_stride,
+         int batch, int heads_q, int heads_kv, int n, int head_dim, int dtype, float sm_scale,
+         int last_q, int force_v, int force_s, float *vertical, float *slash, void *ws, size_t ws_bytes) {
+    if (!q || !k || !vertical || !slash || !ws) return MINF_ERR_INVALID_ARG;
+    if (batch < 0 || heads_q <= 0 || heads_kv <= 0 || n <= 0 || heads_q % heads_kv) return MINF_ERR_INVALID_ARG;
+    if (head_dim != HD || (dtype != MINF_BF16 && dtype != MINF_F16)) return MINF_ERR_UNSUPPORTED;
+    if (last_q < 1 || last_q > LQ || force_v < 0 || force_s < 0) return MINF_ERR_INVALID_ARG;
+    if (((uintptr_t)q & 15) || ((uintptr_t)k & 15)) return MINF_ERR_ALIGNMENT;
+    for (int j = 0; j < 3; ++j)
+        if ((q_stride[j] & 7) || (k_stride[j] & 7)) return MINF_ERR_ALIGNMENT;
+    p.q = (const char *)q; p.k = (const char *)k;
+    for (int j = 0; j < 3; ++j) { p.qs[j] = q_stride[j]; p.ks[j] = k_stride[j]; }
+    p.batch = batch; p.hq = heads_q; p.hk = heads_kv; p.n = n;
+    p.last_q = last_q < n ? last_q : n;
+    p.scale_log2 = sm_scale * 1.4426950408889634f;
+    p.nchunks = (n + KC - 1) / KC;
+    const long long bh = (long long)batch * heads_q;
+    const size_t stats_b = (size_t)bh * p.nchunks * LQ * 2 * sizeof(float);
+    const size_t row_b = (size_t)bh * LQ * sizeof(float);
+    const size_t win_b = (size_t)bh * p.nchunks * WIN * sizeof(float);
+    if (ws_bytes < stats_b + row_b + win_b) return MINF_ERR_WORKSPACE;
+    if ((uintptr_t)ws & 15) return MINF_ERR_ALIGNMENT;
+    p.stats = (float *)ws;
+    p.rowstat = (float *)((char *)ws + stats_b);
+    p.win = (float *)((char *)ws + stats_b + row_b);
+    p.vertical = vertical; p.slash = slash;
+    p.force_v = force_v; p.force_s = force_s;
+    p.total_wg = bh * p.nchunks;
+    return MINF_OK;
+}
+
+}  // namespace
+
+extern "C" size_t minf_vs_estimate_workspace_bytes(int batch, int heads_q, int n) {
+    if (batch <= 0 || heads_q <= 0 || n <= 0) return 0;
+    const size_t bh = (size_t)batch * heads_q;
+    const size_t nchunks = ((size_t)n + KC - 1) / KC;
+    return bh * nchunks * LQ * 2 * sizeof(float) + bh * LQ * sizeof(float) + bh * nchunks * WIN * sizeof(float);
+}
+
+extern "C" int minf_vs_estimate(const void *q, const void *k, const int64_t *q_stride,
+                                const int64_t *k_stride, int batch, int heads_q, int heads_kv, int n,
+                                int head_dim, int dtype, float sm_scale, int last_q, int force_vertical,
+                                int force_slash, float *vertical, float *slash, void *workspace,
+                                size_t workspace_bytes, void *stream) {
+    EstParams p;
+    if (batch == 0) return MINF_OK;
+    int st = fill(p, q, k, q_stride, k_stride, batch, heads_q, heads_kv, n, head_dim, dtype, sm_scale,
+                  last_q, force_vertical, force_slash, vertical, slash, workspace, workspace_bytes);
+    if (st) return st;
+    const long long grid = ((p.total_wg + 7) >> 3) * 8;
+    if (grid > 0x7fffffffLL) return MINF_ERR_UNSUPPORTED;
+    hipStream_t s = (hipStream_t)stream;
+    const long long bh = (long long)batch * heads_q;
+    if (dtype == MINF_BF16) hipLaunchKernelGGL(est_stats_kernel<__bf16>, dim3((unsigned)grid), dim3(EST_THREADS), 0, s, p);
+    else hipLaunchKernelGGL(est_stats_kernel<_Float16>, dim3((unsigned)grid), dim3(EST_THREADS), 0, s, p);
+    hipLaunchKernelGGL(est_reduce_kernel, dim3((unsigned)bh), dim3(LQ), 0, s, p);
+    if (dtype == MINF_BF16) hipLaunchKernelGGL(est_scores_kernel<__bf16>, dim3((unsigned)grid), dim3(EST_THREADS), 0, s, p);
+    else hipLaunchKernelGGL(est_scores_kernel<_Float16>, dim3((unsigned)grid), dim3(EST_THREADS), 0, s, p);
+    hipLaunchKernelGGL(est_finalize_kernel, dim3((unsigned)((n + 255) / 256), (unsigned)bh), dim3(256), 0, s, p);
+    return minf_launch_status();
+}

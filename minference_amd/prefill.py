@@ -1,0 +1,102 @@
+"""Per-head pattern dispatch for one attention layer -- host side.
+
+Counterpart of ``minference_prefill_kernel`` / ``minference_prefill_forward``
+(reference minference/modules/minference_forward.py:594-674) with the same
+``prefill_kwargs`` dictionary: ``layer_idx`` and ``attn_forward_config`` with
+``best_pattern`` (list over layers of ``{"<head>": [type, vertical_size,
+slash_size, score]}``), ``starting_layer`` and ``minference_ratio``.  Heads are
+grouped by (pattern, sizes) and every group is one batched launch sequence
+instead of the reference's Python loop over heads.  K/V may have fewer heads
+than Q (no repeat_kv needed).
+"""
+from __future__ import annotations
+
+import json
+
+import torch
+
+from .estimate import estimate_vertical_slash
+from .index import convert_vertical_slash_indexes
+from .ops import (block_sparse_attention, dense_causal_attention, streaming_forward,
+                  vertical_slash_attention_from_index)
+
+DEFAULT_PATTERN = ("vertical_and_slash", 1000, 6096, 1)   # minference_forward.py:621
+
+
+def vertical_slash_prefill(q, k, v, vertical_size=1000, slash_size=6096):
+    """estimate -> top-k -> index build -> mixed sparse attention for all heads of ``q``
+    (``vertical_and_slash_kernel``, minference_forward.py:599-614)."""
+    B, H, N, _ = q.shape
+    v_idx, s_idx = estimate_vertical_slash(q, k, vertical_size, slash_size)
+    seqlens = torch.full((B,), N, dtype=torch.int32, device=q.device)
+    bc, bo, cc, ci = convert_vertical_slash_indexes(seqlens, v_idx, s_idx, N, 64, 64, zero_fill=False)
+    return vertical_slash_attention_from_index(q, k, v, bc, bo, cc, ci, seqlens)
+
+
+def load_best_pattern(path):
+    """Read a per-model pattern file (same JSON format as minference/configs/*.json)."""
+    with open(path) as f:
+        return json.load(f)
+
+
+def _head_plan(config, layer_idx, num_heads):
+    """-> {(type, vertical_size, slash_size): [head ids]} following :621-625."""
+    best = config.get("best_pattern")
+    layer = best[layer_idx] if best is not None else {}
+    plan = {}
+    for h in range(num_heads):
+        ty, vs, ss, _ = layer.get(str(h), DEFAULT_PATTERN)
+        if "minference_ratio" in config:
+            ratio = config.get("minference_ratio", 1)
+            vs, ss = int(vs * ratio), int(ss * ratio)
+        plan.setdefault((ty, int(vs), int(ss)), []).append(h)
+    return plan
+
+
+def _kv_for_heads(k, heads, group):
+    """K/V heads feeding the query heads ``heads`` -> (tensor, heads_kv) so that the query
+    subset [len(heads)] maps onto it with the usual h // (Hq/Hk) rule."""
+    if group == 1:
+        return k[:, heads]
+    kv = sorted({h // group for h in heads})
+    full = all(h // group in kv for h in heads) and len(heads) == len(kv) * group and \
+        heads == [g * group + i for g in kv for i in range(group)]
+    if full:
+        return k[:, kv]
+    return k[:, [h // group for h in heads]]          # one kv head per query head
+
+
+def minference_prefill_kernel(q, k, v, pattern, vertical_size, slash_size):
+    """One pattern for all heads of q (minference_forward.py:626-631; for ``stream_llm`` the
+    two sizes are n_init and n_local, as in the reference)."""
+    if pattern == "stream_llm":
+        return streaming_forward(q, k, v, vertical_size, slash_size)
+    if pattern == "vertical_and_slash":
+        return vertical_slash_prefill(q, k, v, vertical_size, slash_size)
+    if pattern == "block_sparse":
+        return block_sparse_attention(q, k, v, 100)     # top_k fixed at 100 (:616-618)
+    raise KeyError(pattern)
+
+
+def minference_prefill_forward(query_states, key_states, value_states, prefill_kwargs):
+    """Sparse prefill attention of one layer: [B,Hq,N,D] x [B,Hk,N,D] -> [B,Hq,N,D]."""
+    config = prefill_kwargs["attn_forward_config"]
+    layer_idx = prefill_kwargs["layer_idx"]
+    starting_layer = config.get("starting_layer", 0)
+    if config.get("is_search", False):
+        raise NotImplementedError("offline pattern search is not part of this package")
+    B, H, N, D = query_states.shape
+    group = H // key_states.shape[1]
+    if layer_idx < starting_layer:
+        return dense_causal_attention(query_states, key_states, value_states)
+    plan = _head_plan(config, layer_idx, H)
+    if len(plan) == 1:
+        (ty, vs, ss), _ = next(iter(plan.items()))
+        return minference_prefill_kernel(query_states, key_states, value_states, ty, vs, ss)
+    output = torch.empty_like(query_states)
+    for (ty, vs, ss), heads in plan.items():
+        qh = query_states[:, heads]
+        kh = _kv_for_heads(key_states, heads, group)
+        vh = _kv_for_heads(value_states, heads, group)
+        output[:, heads] = minference_prefill_kernel(qh, kh, vh, ty, vs, ss)
+    return output

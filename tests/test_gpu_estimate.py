@@ -1,0 +1,74 @@
+"""GPU parity of the estimation kernels and the top-k selection against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+from tests import gen
+
+pytestmark = pytest.mark.gpu
+
+
+def expand(x, hq):
+    return x.repeat_interleave(hq // x.shape[1], dim=1)
+
+
+@pytest.mark.parametrize("n,hq,hk,dtype", [
+    (64, 1, 1, torch.bfloat16), (100, 2, 1, torch.bfloat16), (1024, 4, 2, torch.bfloat16),
+    (3000, 2, 2, torch.float16), (5000, 4, 1, torch.bfloat16), (40, 1, 1, torch.bfloat16),
+])
+def test_scores_vs_oracle(gpu, n, hq, hk, dtype):
+    from minference_amd.estimate import vertical_slash_scores
+    print(f"case est n={n} hq={hq} hk={hk} {dtype}", flush=True)
+    q, k, _ = gen.qkv(1, hq, hk, n, 128, seed=n, scale=1.0)
+    q, k = q.to(dtype), k.to(dtype)
+    vert, slash = vertical_slash_scores(q.to(gpu), k.to(gpu), force_vertical=0, force_slash=0)
+    rv, rs = O.estimate_scores(q, expand(k, hq))
+    vert, slash = vert.cpu(), slash.cpu()
+    lq = min(64, n)
+    assert torch.allclose(vert.sum(-1), torch.full((1, hq), float(lq)), atol=1e-3)
+    assert torch.allclose(slash.sum(-1), torch.full((1, hq), float(lq)), atol=1e-3)
+    # fp32 arithmetic on identical 16-bit inputs: relative 1e-3 on the score vectors
+    assert torch.allclose(vert, rv, rtol=1e-3, atol=1e-6), (vert - rv).abs().max()
+    assert torch.allclose(slash, rs, rtol=1e-3, atol=1e-6), (slash - rs).abs().max()
+
+
+def test_forcing(gpu):
+    from minference_amd.estimate import vertical_slash_scores
+    q, k, _ = gen.qkv(1, 2, 2, 500, 128, seed=9, scale=1.0)
+    vert, slash = vertical_slash_scores(q.bfloat16().to(gpu), k.bfloat16().to(gpu))
+    assert torch.isinf(vert[..., :30]).all() and torch.isfinite(vert[..., 30:]).all()
+    assert torch.isinf(slash[..., -100:]).all() and torch.isfinite(slash[..., :-100]).all()
+
+
+@pytest.mark.parametrize("n,k", [(1000, 10), (5000, 1000), (131072, 6096), (70001, 1000), (300, 300), (64, 100)])
+def test_topk_exact_vs_oracle(gpu, n, k):
+    from minference_amd.estimate import topk_indices
+    g = torch.Generator().manual_seed(n + k)
+    x = torch.rand(3, n, generator=g)
+    x[0, : min(30, n)] = torch.inf
+    x[1, -min(100, n):] = torch.inf
+    x[2] = (x[2] * 50).floor() / 50             # many ties
+    got = topk_indices(x.to(gpu), k).cpu()
+    ref = O.topk_lowest_index(x, min(k, n)).to(torch.int32)
+    assert torch.equal(got, ref)
+    got_r = topk_indices(x.to(gpu), k, reverse_base=n - 1).cpu()
+    assert torch.equal(got_r, (n - 1) - ref)
+
+
+def test_estimate_sets_vs_oracle(gpu):
+    from minference_amd.estimate import estimate_vertical_slash
+    n = 4096
+    q, k, _ = gen.qkv(1, 4, 2, n, 128, seed=77, scale=1.0)
+    q, k = q.bfloat16(), k.bfloat16()
+    v_idx, s_idx = estimate_vertical_slash(q.to(gpu), k.to(gpu), 200, 600)
+    rv, rs, vs, ss = O.estimate_vs(q, expand(k, 4), 200, 600)
+    v_idx, s_idx = v_idx.cpu(), s_idx.cpu()
+    assert v_idx.dtype == torch.int32 and v_idx.shape == (1, 4, 200) and s_idx.shape == (1, 4, 600)
+    for h in range(4):
+        a, b = set(v_idx[0, h].tolist()), set(rv[0, h].tolist())
+        c, d = set(s_idx[0, h].tolist()), set(rs[0, h].tolist())
+        # identical up to near-ties at the k-th score: recall >= 0.99
+        assert len(a & b) >= 0.99 * 200 and len(c & d) >= 0.99 * 600
+        assert set(range(30)) <= a and set(range(100)) <= c
+        assert (np.diff(v_idx[0, h].numpy()) > 0).all() and (np.diff(s_idx[0, h].numpy()) < 0).all()
