@@ -9,7 +9,7 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libminf_hip.so")
+LIB_PATH = os.environ.get("MINF_HIP_LIB", os.path.join(_HERE, "libminf_hip.so"))
 _lib = None
 
 c_int = ctypes.c_int

@@ -24,6 +24,7 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-fno-honor-nans",      # fmax/fmin without NaN canonicalisation (infinities are still honoured)
     "-Wno-unused-command-line-argument", "-Wno-ignored-optimization-argument",
 ]
 

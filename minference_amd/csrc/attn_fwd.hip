@@ -19,9 +19,12 @@
 // LDS: K and V tiles are [64 tokens][128] 16-bit, 256 B per row, no padding;
 // 16-byte chunks are XOR-swizzled (K: chunk ^ row%16, V: chunk ^ 4*(row%4)) so
 // that ds_read_b128 of 16 rows and the 4-row transpose reads hit distinct banks.
-// Global->LDS goes through registers, prefetched one tile ahead.
+// Global->LDS goes through registers in half tiles (32 keys), prefetched a tile ahead, and the
+// main loop is software-pipelined over half tiles: the QK^T MFMAs of half tile h+1 are issued
+// next to the softmax VALU work of half tile h (see the schedule above the loop).
 #include "minf_common.h"
 #include <math.h>
+#include <type_traits>
 
 namespace {
 
@@ -38,8 +41,15 @@ enum { MODE_VS = 0, MODE_BS = 1, MODE_ASHAPE = 2, MODE_DENSE = 3 };
 constexpr int BM = 64;        // query rows per workgroup
 constexpr int BN = 64;        // keys per tile
 constexpr int HD = 128;       // head_dim
-constexpr int NTHREADS = 128; // 2 wavefronts
+constexpr int NTHREADS = 256; // 4 wavefronts: 2 row halves x 2 key halves
 constexpr int ROW_BYTES = HD * 2;
+// LDS row pitches: +16 B (K) makes ds_read_b128 of 16 consecutive rows hit 64 distinct banks,
+// +64 B (V) does the same for the 4-row x 64-byte transpose reads; with plain padding every LDS
+// address is one per-lane base plus an immediate offset.
+constexpr int K_PITCH = ROW_BYTES + 16;
+constexpr int V_PITCH = ROW_BYTES + 64;
+constexpr int LDS_K_BYTES = BN * K_PITCH;
+constexpr int LDS_V_BYTES = BN * V_PITCH;
 
 struct AttnParams {
     const char *q, *k, *v;
@@ -59,6 +69,17 @@ struct AttnParams {
     int n_init, n_local;
     long long total_wg;
 };
+
+// The index tensors are read-only for the whole launch.  Their wave-uniform entries (counts,
+// block offsets, block ids) are read through constant-address-space pointers so that they become
+// scalar loads: a vector load whose result is needed at once would make the wave wait for every
+// K/V prefetch issued before it.  The gathered column ids stay vector loads (one per lane).
+typedef const __attribute__((address_space(4))) int *cint_ptr;
+struct IdxPtrs {
+    cint_ptr bc, bo, cc, bidx;
+    const int *ci;
+};
+__device__ __forceinline__ cint_ptr as_const(const int *p) { return (cint_ptr)(unsigned long long)p; }
 
 template <typename T> struct Mma;
 template <> struct Mma<__bf16> {
@@ -95,6 +116,31 @@ template <> __device__ __forceinline__ void cvt8<_Float16>(const float *x, Frag 
     for (int j = 0; j < 8; ++j) f.h[j] = (_Float16)x[j];
 }
 
+// sum of the 8 (rounded) values of a fragment, via the 2-way dot-product instructions
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
+typedef __attribute__((__vector_size__(2 * sizeof(_Float16)))) _Float16 f16x2_t;
+template <typename T> __device__ __forceinline__ float pair_sum(const Frag &f);
+template <> __device__ __forceinline__ float pair_sum<__bf16>(const Frag &f) {
+    const bf16x2_t one = {(__bf16)1.0f, (__bf16)1.0f};
+    float acc = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        bf16x2_t pr = {f.b[2 * j], f.b[2 * j + 1]};
+        acc = __builtin_amdgcn_fdot2_f32_bf16(pr, one, acc, false);
+    }
+    return acc;
+}
+template <> __device__ __forceinline__ float pair_sum<_Float16>(const Frag &f) {
+    const f16x2_t one = {(_Float16)1.0f, (_Float16)1.0f};
+    float acc = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        f16x2_t pr = {f.h[2 * j], f.h[2 * j + 1]};
+        acc = __builtin_amdgcn_fdot2(pr, one, acc, false);
+    }
+    return acc;
+}
+
 // One tile of keys: either 64 consecutive tokens from `start`, or 64 gathered
 // token ids read from `gather` (entries >= nvalid are padding).
 struct Tile {
@@ -104,10 +150,10 @@ struct Tile {
 };
 
 template <int MODE>
-__device__ __forceinline__ int tile_count(const AttnParams &p, long long ridx, int m, int &nblk) {
+__device__ __forceinline__ int tile_count(const AttnParams &p, const IdxPtrs &ix, long long ridx, int m, int &nblk) {
     if constexpr (MODE == MODE_VS) {
-        nblk = p.bc[ridx];
-        return nblk + ((p.cc[ridx] + BN - 1) >> 6);
+        nblk = ix.bc[ridx];
+        return nblk + ((ix.cc[ridx] + BN - 1) >> 6);
     } else if constexpr (MODE == MODE_BS) {
         nblk = min(m + 1, p.max_blocks);
         return nblk;
@@ -125,20 +171,20 @@ __device__ __forceinline__ int tile_count(const AttnParams &p, long long ridx, i
 }
 
 template <int MODE>
-__device__ __forceinline__ Tile tile_at(const AttnParams &p, long long ridx, int m, int nblk, int it) {
+__device__ __forceinline__ Tile tile_at(const AttnParams &p, const IdxPtrs &ix, long long ridx, int m, int nblk, int it) {
     Tile t;
     t.gathered = 0;
     t.nvalid = BN;
     if constexpr (MODE == MODE_VS) {
         if (it < nblk) {
-            t.start = p.bo[ridx * p.nnz_s + it];
+            t.start = ix.bo[ridx * p.nnz_s + it];
         } else {
             t.gathered = 1;
             t.start = (it - nblk) * BN;
-            t.nvalid = min(BN, p.cc[ridx] - t.start);
+            t.nvalid = min(BN, ix.cc[ridx] - t.start);
         }
     } else if constexpr (MODE == MODE_BS) {
-        t.start = p.bidx[((ridx / p.rows) * p.bidx_rows + m) * p.max_blocks + it] * BN;
+        t.start = ix.bidx[((ridx / p.rows) * p.bidx_rows + m) * p.max_blocks + it] * BN;
     } else if constexpr (MODE == MODE_ASHAPE) {
         int lo_key = m * BM - p.n_local + 1;
         int t_lo = lo_key > 0 ? (lo_key >> 6) : 0;
@@ -151,8 +197,14 @@ __device__ __forceinline__ Tile tile_at(const AttnParams &p, long long ridx, int
 
 template <typename T, int MODE>
 __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams p) {
-    __shared__ __attribute__((aligned(16))) char lds_k[BN * ROW_BYTES];
-    __shared__ __attribute__((aligned(16))) char lds_v[BN * ROW_BYTES];
+    IdxPtrs ix;
+    ix.bc = as_const(p.bc); ix.bo = as_const(p.bo); ix.cc = as_const(p.cc); ix.bidx = as_const(p.bidx);
+    ix.ci = p.ci;
+    // K tile, V tile, and 1 KB for the (max, sum) pairs of the final merge; the O partials of
+    // the merge reuse the K/V space.
+    __shared__ __attribute__((aligned(16))) char lds[LDS_K_BYTES + LDS_V_BYTES];
+    char *const lds_k = lds;
+    char *const lds_v = lds + LDS_K_BYTES;
 
     // ---- which (batch, head, row block): XCD-aware remap --------------------
     // Consecutive workgroup ids are dealt round-robin to the 8 XCDs; give each
@@ -173,12 +225,14 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
     const int tid = (int)threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
+    const int rw = wave & 1;          // which 32 query rows of the block
+    const int kw = wave >> 1;         // which 32 keys of every tile
     const int l32 = lane & 31;
     const int g = lane >> 5;
 
     const int seqlen = p.seqlens ? min(p.seqlens[b], p.n) : p.n;
     const int row0 = m * BM;
-    const int qrow = row0 + wave * 32 + l32;          // this lane's query row
+    const int qrow = row0 + rw * 32 + l32;          // this lane's query row
     char *o_base = p.o + ((long long)b * p.os[0] + (long long)h * p.os[1]) * 2;
 
     if (row0 >= seqlen) {
@@ -209,174 +263,297 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
     }
 
     int nblk = 0;
-    const int ntiles = tile_count<MODE>(p, ridx, m, nblk);
+    const int ntiles = tile_count<MODE>(p, ix, ridx, m, nblk);
 
-    // ---- global -> register staging: thread covers rows i*8 + tid/16, chunk tid%16
-    const int ld_r = tid >> 4;       // 0..7
-    const int ld_c = tid & 15;       // 16-byte chunk in the row
-    u32x4_t kreg[8], vreg[8];
-
+    // ---- global -> register -> LDS staging ---------------------------------------
+    // A thread covers rows 16*i + tid/16 (i = 0..3) of a tile, 16-byte chunk tid%16.
     // Rows that do not exist (past seqlen, or padding of a gathered tile) are read from a
     // clamped, valid address instead of being zeroed: their scores are always masked to
     // -inf below, so their probabilities are exactly 0 and K/V contents never matter.
-    auto issue_loads = [&](const Tile &t) {
-        int tok[8];
+    const int ld_r = tid >> 4;       // 0..15
+    const int ld_c = tid & 15;       // 16-byte chunk in the row
+    u32x4_t kreg[4], vreg[4];        // in flight: next K tile, next V tile
+
+    // byte offset of this thread's first row inside a contiguous tile (rows 16 apart add a
+    // wave-uniform 16*pitch, so one 32-bit lane offset serves all four loads)
+    const unsigned koff = (unsigned)(ld_r * k_row + ld_c * 16);
+    const unsigned voff = (unsigned)(ld_r * v_row + ld_c * 16);
+    const bool small_pitch = k_row * 64 < (1ll << 31) && v_row * 64 < (1ll << 31);
+    // token ids of this thread's 4 rows of a gathered (column) tile
+    auto gather_ids = [&](const Tile &t, int (&tok)[4]) {
         if (MODE == MODE_VS && t.gathered) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const int r = i * 8 + ld_r;
-                tok[i] = p.ci[ridx * p.nnz_v + t.start + min(r, t.nvalid - 1)];
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) tok[i] = t.start + i * 8 + ld_r;
-        }
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int tk = max(0, min(tok[i], seqlen - 1));
-            kreg[i] = *reinterpret_cast<const u32x4_t *>(k_base + tk * k_row + ld_c * 16);
-            vreg[i] = *reinterpret_cast<const u32x4_t *>(v_base + tk * v_row + ld_c * 16);
+            for (int i = 0; i < 4; ++i)
+                tok[i] = ix.ci[ridx * p.nnz_v + t.start + min(i * 16 + ld_r, t.nvalid - 1)];
         }
     };
-    auto store_lds = [&]() {
+    auto load_tile = [&](const Tile &t, const char *base, long long rowstride, const unsigned off,
+                         const int (&gtok)[4], u32x4_t (&dst)[4]) {
+        const bool gathered = MODE == MODE_VS && t.gathered;
+        if (!gathered && small_pitch && t.start >= 0 && t.start + BN <= seqlen) {
+            // common case: one wave-uniform base, loop-invariant per-thread offsets
+            const char *tb = base + (long long)t.start * rowstride;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int r = i * 8 + ld_r;
-            *reinterpret_cast<u32x4_t *>(lds_k + r * ROW_BYTES + ((ld_c ^ (r & 15)) << 4)) = kreg[i];
-            *reinterpret_cast<u32x4_t *>(lds_v + r * ROW_BYTES + ((ld_c ^ ((r & 3) << 2)) << 4)) = vreg[i];
+            for (int i = 0; i < 4; ++i)
+                dst[i] = *reinterpret_cast<const u32x4_t *>(tb + (long long)i * 16 * rowstride + off);
+            return;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int tok = gathered ? gtok[i] : t.start + i * 16 + ld_r;
+            const int tk = max(0, min(tok, seqlen - 1));
+            dst[i] = *reinterpret_cast<const u32x4_t *>(base + tk * rowstride + ld_c * 16);
+        }
+    };
+    char *const lds_k_st = lds_k + ld_r * K_PITCH + ld_c * 16;
+    char *const lds_v_st = lds_v + ld_r * V_PITCH + ld_c * 16;
+    auto store_k = [&](const u32x4_t (&src)[4]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            *reinterpret_cast<u32x4_t *>(lds_k_st + i * 16 * K_PITCH) = src[i];
+        }
+    };
+    auto store_v = [&](const u32x4_t (&src)[4]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            *reinterpret_cast<u32x4_t *>(lds_v_st + i * 16 * V_PITCH) = src[i];
         }
     };
 
-    // ---- accumulators -------------------------------------------------------
+    // ---- accumulators (this wave's share: its 32 rows x its 32 keys of every tile) -----
     f32x16_t oacc[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int r = 0; r < 16; ++r) oacc[i][r] = 0.f;
-    float m_i = -INFINITY;   // running max (log2 domain, scaled)
+    float m_i = -INFINITY;   // reference max of the row (log2 domain, scaled); lags the true max by <= 8
     float l_i = 0.f;         // this lane's share of the running sum
 
-    // LDS read addresses that do not depend on the tile
-    // K: row = 32*blk + l32, logical chunk 2*ks + g
-    const int k_rd_row = l32;
     // V transpose read: row = T0 + (lane%16)/4, col = 32*db + 16*((lane/16)%2) + 4*(lane%4)
     const int v_rd_rsub = (lane & 15) >> 2;
-    const int v_rd_chunk = (((lane >> 4) & 1) << 1) + ((lane & 3) >> 1);   // + 4*db
-    const int v_rd_byte = (lane & 1) << 3;
+    const int v_rd_col = (((lane >> 4) & 1) << 4) + ((lane & 3) << 2);      // + 32*db
+    const int wrow_lo = row0 + rw * 32, wrow_hi = wrow_lo + 31;
 
-    Tile cur, nxt;
-    if (ntiles > 0) {
-        cur = tile_at<MODE>(p, ridx, m, nblk, 0);
-        issue_loads(cur);
-    }
-
-    for (int it = 0; it < ntiles; ++it) {
-        __syncthreads();            // previous tile fully consumed
-        store_lds();
-        __syncthreads();
-        if (it + 1 < ntiles) {
-            nxt = tile_at<MODE>(p, ridx, m, nblk, it + 1);
-            issue_loads(nxt);
-        }
-
-        // ---- S^T = K . Q^T --------------------------------------------------
-        f32x16_t s0, s1;
+    const char *const lds_k_rd = lds_k + (32 * kw + l32) * K_PITCH + g * 16;
+    const char *const lds_v_rd = lds_v + (32 * kw + 4 * g + v_rd_rsub) * V_PITCH + v_rd_col * 2;
+    // S^T of this wave: keys 32*kw + (0..31) of the tile in LDS x its 32 query rows
+    auto qk_tile = [&]() {
+        f32x16_t s;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) { s0[r] = 0.f; s1[r] = 0.f; }
+        for (int r = 0; r < 16; ++r) s[r] = 0.f;
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) {
-            const int x = 2 * ks + g;
-            Frag a0, a1;
-            a0.u = *reinterpret_cast<const u32x4_t *>(lds_k + k_rd_row * ROW_BYTES + ((x ^ (k_rd_row & 15)) << 4));
-            a1.u = *reinterpret_cast<const u32x4_t *>(lds_k + (32 + k_rd_row) * ROW_BYTES + ((x ^ (k_rd_row & 15)) << 4));
-            s0 = Mma<T>::mfma(frag_as<T>(a0), frag_as<T>(qf[ks]), s0);
-            s1 = Mma<T>::mfma(frag_as<T>(a1), frag_as<T>(qf[ks]), s1);
+            Frag a;
+            a.u = *reinterpret_cast<const u32x4_t *>(lds_k_rd + ks * 32);
+            s = Mma<T>::mfma(frag_as<T>(a), frag_as<T>(qf[ks]), s);
         }
+        return s;
+    };
 
-        // ---- mask -----------------------------------------------------------
-        // element (blk, r) of this lane is tile-local key tk = tkc + 4*g with the compile-time
-        // part tkc = 32*blk + 8*(r/4) + r%4.  keep <=> tk <= hi && (tk > wlo || tk < slim).
-        bool need_mask;
-        const int wrow_lo = row0 + wave * 32, wrow_hi = wrow_lo + 31;
-        int hi, wlo = -1, slim = 0;      // per-lane bounds on tkc (4*g already subtracted)
-        if (MODE == MODE_VS && cur.gathered) {
-            need_mask = cur.nvalid < BN;
-            hi = cur.nvalid - 1 - 4 * g;
-        } else {
-            hi = min(qrow, seqlen - 1) - cur.start - 4 * g;
-            if constexpr (MODE == MODE_ASHAPE) {
-                const int c_lo = cur.start, c_hi = cur.start + BN - 1;
-                const bool causal_ok = c_hi <= wrow_lo && c_hi < seqlen;
-                const bool in_window = (wrow_hi - c_lo) < p.n_local;
-                const bool in_sink = c_hi < p.n_init;
-                need_mask = !(causal_ok && (in_window || in_sink));
-                wlo = qrow - cur.start - p.n_local - 4 * g;
-                slim = p.n_init - cur.start - 4 * g;
-            } else {
-                need_mask = (cur.start + BN - 1 > wrow_lo) || (cur.start + BN > seqlen);
-            }
+    // does this wave have to mask anything in its keys [32*kw, 32*kw+32) of tile t ?
+    auto needs_mask = [&](const Tile &t) {
+        if (MODE == MODE_VS && t.gathered) return t.nvalid < 32 * kw + 32;
+        const int c_lo = t.start + 32 * kw, c_hi = c_lo + 31;
+        if constexpr (MODE == MODE_ASHAPE) {
+            const bool causal_ok = c_hi <= wrow_lo && c_hi < seqlen;
+            const bool in_window = (wrow_hi - c_lo) < p.n_local;
+            const bool in_sink = c_hi < p.n_init;
+            return !(causal_ok && (in_window || in_sink));
         }
-        if (need_mask) {
+        return (c_hi > wrow_lo) || (c_hi >= seqlen);
+    };
+
+    // online softmax of this wave's 32x32 score block (exp2 domain); s -> probabilities, packed
+    // into the B-operand fragments of the two PV k-steps; alpha = factor for the O accumulators.
+    // Element r of this lane is tile-local key 32*kw + 4*g + tkc, tkc = 8*(r/4) + r%4.
+    // keep <=> tkc <= hi && (tkc > wlo || tkc < slim).
+    auto softmax_tile = [&](f32x16_t &s, const Tile &t, auto masked, Frag (&pf)[2], float &alpha, bool &rescale) {
+        if constexpr (decltype(masked)::value) {
+            int hi, wlo = -1, slim = 0;
+            const int sh = 4 * g + 32 * kw;
+            if (MODE == MODE_VS && t.gathered) {
+                hi = t.nvalid - 1 - sh;
+            } else {
+                hi = min(qrow, seqlen - 1) - t.start - sh;
+                if constexpr (MODE == MODE_ASHAPE) {
+                    wlo = qrow - t.start - p.n_local - sh;
+                    slim = p.n_init - t.start - sh;
+                }
+            }
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int tkc = 8 * (r >> 2) + (r & 3);
-                bool k0 = tkc <= hi, k1 = (tkc + 32) <= hi;
-                if constexpr (MODE == MODE_ASHAPE) {
-                    k0 = k0 & ((tkc > wlo) | (tkc < slim));
-                    k1 = k1 & (((tkc + 32) > wlo) | ((tkc + 32) < slim));
-                }
-                s0[r] = k0 ? s0[r] : -INFINITY;
-                s1[r] = k1 ? s1[r] : -INFINITY;
+                bool kp = tkc <= hi;
+                if constexpr (MODE == MODE_ASHAPE) kp = kp & ((tkc > wlo) | (tkc < slim));
+                s[r] = kp ? s[r] : -INFINITY;
             }
         }
-
-        // ---- online softmax (exp2 domain) -------------------------------------
-        float mx = s0[0];
+        float mx = fmaxf(s[0], s[1]);
 #pragma unroll
-        for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s0[r]);
-#pragma unroll
-        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s1[r]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = fmaxf(m_i, mx * p.scale_log2);
-        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = __builtin_amdgcn_exp2f(m_i - m_use);
-        m_i = m_new;
-        float psum = 0.f;
-        float pv[32];
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            pv[r] = __builtin_amdgcn_exp2f(fmaf(s0[r], p.scale_log2, -m_use));
-            pv[16 + r] = __builtin_amdgcn_exp2f(fmaf(s1[r], p.scale_log2, -m_use));
+        for (int r = 2; r < 16; ++r) mx = fmaxf(mx, s[r]);
+        {
+            // max over the two lane halves (lanes l and l^32 hold the same query row)
+            const unsigned u = __float_as_uint(mx);
+            auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+            mx = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
         }
+        // lazy reference max: only move it when the row max grew by more than 2^8
+        const float cand = mx * p.scale_log2;
+        const bool grow = cand > m_i + 8.0f;
+        const float m_next = grow ? cand : m_i;
+        alpha = grow ? __builtin_amdgcn_exp2f(m_i - m_next) : 1.0f;
+        rescale = __any(grow);
+        m_i = m_next;
+        const float m_sub = (m_next == -INFINITY) ? 0.f : m_next;
+        float pr[16];
 #pragma unroll
-        for (int r = 0; r < 32; ++r) psum += pv[r];
-        l_i = l_i * alpha + psum;
-        if (__any(alpha != 1.0f)) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
-        }
+        for (int r = 0; r < 16; ++r) pr[r] = __builtin_amdgcn_exp2f(fmaf(s[r], p.scale_log2, -m_sub));
+        cvt8<T>(&pr[0], pf[0]);
+        cvt8<T>(&pr[8], pf[1]);
+        // row sum of the ROUNDED probabilities (what the PV product really uses)
+        l_i = l_i * alpha + pair_sum<T>(pf[0]) + pair_sum<T>(pf[1]);
+    };
 
-        // ---- O^T += V^T . P^T -------------------------------------------------
+    auto pv_tile = [&](const Frag (&pf)[2]) {
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            Frag pf;
-            cvt8<T>(&pv[8 * s], pf);     // slots j <-> regs 8*(s%2)+j of block s/2 == pv[8*s + j]
+        for (int s2 = 0; s2 < 2; ++s2) {
 #pragma unroll
             for (int db = 0; db < 4; ++db) {
                 Frag vf;
 #pragma unroll
                 for (int jj = 0; jj < 2; ++jj) {
-                    const int row = 16 * s + 8 * jj + 4 * g + v_rd_rsub;
-                    const int chunk = (4 * db + v_rd_chunk) ^ ((row & 3) << 2);
                     vf.s4[jj] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                        (__attribute__((address_space(3))) short4_t *)(lds_v + row * ROW_BYTES + (chunk << 4) + v_rd_byte));
+                        (__attribute__((address_space(3))) short4_t *)(lds_v_rd + (16 * s2 + 8 * jj) * V_PITCH + db * 64));
                 }
-                oacc[db] = Mma<T>::mfma(frag_as<T>(vf), frag_as<T>(pf), oacc[db]);
+                oacc[db] = Mma<T>::mfma(frag_as<T>(vf), frag_as<T>(pf[s2]), oacc[db]);
             }
         }
-        cur = nxt;
+    };
+    auto rescale_o = [&](float alpha) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
+    };
+    // Ask the scheduler to spread the 8 QK MFMAs of a phase between the softmax VALU work of the
+    // same basic block: (1 LDS read, 1 MFMA, 10 VALU) x 8.
+    auto interleave_hint = [&]() {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 10, 0);
+        }
+    };
+
+    // ---- software pipeline over tiles ----------------------------------------------
+    // Iteration `it` (t0 = tile it, t1 = it+1, ...; indices clamped to the last tile):
+    //   A : S_next = QK(t1) [Kbuf = K(t1)]  ||  softmax(S_cur = scores of t0)
+    //   barrier; store K(t2) -> Kbuf; load kreg <- K(t3)
+    //   B : O += P.V(t0)   [Vbuf = V(t0)]
+    //   barrier; store V(t1) -> Vbuf; load vreg <- V(t2)
+    // The QK MFMAs of the next tile share a basic block with the softmax VALU work of the
+    // current one; every LDS region is overwritten only after the barrier that follows its
+    // last read and read only after the barrier that follows its write.
+    if (ntiles > 0) {
+        const int last = ntiles - 1;
+        Tile t0 = tile_at<MODE>(p, ix, ridx, m, nblk, 0);
+        Tile t1 = tile_at<MODE>(p, ix, ridx, m, nblk, min(1, last));
+        Tile t2 = tile_at<MODE>(p, ix, ridx, m, nblk, min(2, last));
+        Tile t3 = tile_at<MODE>(p, ix, ridx, m, nblk, min(3, last));
+        // (global loads are issued in the same order as inside the loop -- gather ids, K, V -- so
+        // that the outstanding-load counters the waits are derived from agree on every path)
+        Tile t4 = tile_at<MODE>(p, ix, ridx, m, nblk, min(4, last));
+        int tokK[4] = {0, 0, 0, 0}, tokV[4] = {0, 0, 0, 0}, tokN[4] = {0, 0, 0, 0};
+        gather_ids(t0, tokK);
+        load_tile(t0, k_base, k_row, koff, tokK, kreg);
+        load_tile(t0, v_base, v_row, voff, tokK, vreg);
+        store_k(kreg);
+        store_v(vreg);
+        gather_ids(t1, tokV);
+        load_tile(t1, k_base, k_row, koff, tokV, kreg);
+        __syncthreads();
+        f32x16_t s_a = qk_tile();
+        __syncthreads();
+        store_k(kreg);
+        gather_ids(t2, tokK);
+        gather_ids(t3, tokN);
+        load_tile(t2, k_base, k_row, koff, tokK, kreg);
+        load_tile(t1, v_base, v_row, voff, tokV, vreg);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) tokV[i] = tokK[i];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) tokK[i] = tokN[i];
+        __syncthreads();
+
+        // One pipeline step; the score registers ping-pong between two steps (no copies).
+        // On entry: Kbuf = K(t1), Vbuf = V(t0), kreg = K(t2) and vreg = V(t1) in flight;
+        // tokK / tokV = gathered token ids of t3 / t2 (if those are column tiles).
+        auto step = [&](f32x16_t &s_cur, f32x16_t &s_nxt, int it) {
+            Frag pf[2];
+            float alpha;
+            bool rescale;
+            gather_ids(t4, tokN);          // needed one step from now: stays older than the K/V loads below
+            if (needs_mask(t0)) {
+                s_nxt = qk_tile();
+                softmax_tile(s_cur, t0, std::true_type{}, pf, alpha, rescale);
+                interleave_hint();
+            } else {
+                s_nxt = qk_tile();
+                softmax_tile(s_cur, t0, std::false_type{}, pf, alpha, rescale);
+                interleave_hint();
+            }
+            __syncthreads();
+            store_k(kreg);
+            load_tile(t3, k_base, k_row, koff, tokK, kreg);
+            if (rescale) rescale_o(alpha);
+            pv_tile(pf);
+            __syncthreads();
+            store_v(vreg);
+            load_tile(t2, v_base, v_row, voff, tokV, vreg);
+            t0 = t1;
+            t1 = t2;
+            t2 = t3;
+            t3 = t4;
+            t4 = tile_at<MODE>(p, ix, ridx, m, nblk, min(it + 5, last));
+#pragma unroll
+            for (int i = 0; i < 4; ++i) tokV[i] = tokK[i];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) tokK[i] = tokN[i];
+        };
+        f32x16_t s_b;
+        for (int it = 0;;) {
+            step(s_a, s_b, it);
+            if (++it >= ntiles) break;
+            step(s_b, s_a, it);
+            if (++it >= ntiles) break;
+        }
+    }
+
+    // ---- merge the two key halves: waves kw=1 hand (m, l, O) to waves kw=0 through LDS ----
+    __syncthreads();
+    float *xo = reinterpret_cast<float *>(lds) + rw * (64 * 64);        // [reg 0..63][lane]
+    float *xml = reinterpret_cast<float *>(lds + 2 * 64 * 64 * 4) + rw * 128;   // [m|l][lane]
+    if (kw == 1) {
+#pragma unroll
+        for (int db = 0; db < 4; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) xo[(db * 16 + r) * 64 + lane] = oacc[db][r];
+        xml[lane] = m_i;
+        xml[64 + lane] = l_i;
+    }
+    __syncthreads();
+    if (kw == 1) return;
+    {
+        const float m1 = xml[lane], l1 = xml[64 + lane];
+        const float mm = fmaxf(m_i, m1);
+        const float mu = (mm == -INFINITY) ? 0.f : mm;
+        const float a0 = __builtin_amdgcn_exp2f(m_i - mu), a1 = __builtin_amdgcn_exp2f(m1 - mu);
+        l_i = l_i * a0 + l1 * a1;
+#pragma unroll
+        for (int db = 0; db < 4; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[db][r] = oacc[db][r] * a0 + xo[(db * 16 + r) * 64 + lane] * a1;
     }
 
     // ---- epilogue: O = O^T / l, store ------------------------------------------
