@@ -43,13 +43,8 @@ constexpr int BN = 64;        // keys per tile
 constexpr int HD = 128;       // head_dim
 constexpr int NTHREADS = 256; // 4 wavefronts: 2 row halves x 2 key halves
 constexpr int ROW_BYTES = HD * 2;
-// LDS row pitches: +16 B (K) makes ds_read_b128 of 16 consecutive rows hit 64 distinct banks,
-// +64 B (V) does the same for the 4-row x 64-byte transpose reads; with plain padding every LDS
-// address is one per-lane base plus an immediate offset.
-constexpr int K_PITCH = ROW_BYTES + 16;
-constexpr int V_PITCH = ROW_BYTES + 64;
-constexpr int LDS_K_BYTES = BN * K_PITCH;
-constexpr int LDS_V_BYTES = BN * V_PITCH;
+constexpr int TILE_BYTES = BN * ROW_BYTES;          // 16 KB, rows unpadded, 16-byte chunks XOR-swizzled
+constexpr int LDS_BYTES = 4 * TILE_BYTES + 1024;    // K x2, V x2 (double buffered) [+ merge scratch]
 
 struct AttnParams {
     const char *q, *k, *v;
@@ -202,9 +197,13 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
     ix.ci = p.ci;
     // K tile, V tile, and 1 KB for the (max, sum) pairs of the final merge; the O partials of
     // the merge reuse the K/V space.
-    __shared__ __attribute__((aligned(16))) char lds[LDS_K_BYTES + LDS_V_BYTES];
-    char *const lds_k = lds;
-    char *const lds_v = lds + LDS_K_BYTES;
+    // K and V double buffers as four separate LDS objects: the compiler only lets an LDS read
+    // run ahead of an in-flight global->LDS copy when it can prove they touch different objects.
+    __shared__ __attribute__((aligned(16))) char lds_k0[TILE_BYTES];
+    __shared__ __attribute__((aligned(16))) char lds_k1[TILE_BYTES];
+    __shared__ __attribute__((aligned(16))) char lds_v0[TILE_BYTES];
+    __shared__ __attribute__((aligned(16))) char lds_v1[TILE_BYTES];
+    __shared__ float lds_ml[256];
 
     // ---- which (batch, head, row block): XCD-aware remap --------------------
     // Consecutive workgroup ids are dealt round-robin to the 8 XCDs; give each
@@ -265,58 +264,39 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
     int nblk = 0;
     const int ntiles = tile_count<MODE>(p, ix, ridx, m, nblk);
 
-    // ---- global -> register -> LDS staging ---------------------------------------
-    // A thread covers rows 16*i + tid/16 (i = 0..3) of a tile, 16-byte chunk tid%16.
+    // ---- global -> LDS copies without a register round trip --------------------------------
+    // global_load_lds_dwordx4: every lane fetches 16 bytes from its own global address and the
+    // wave's 64 x 16 B land CONTIGUOUSLY in LDS at a wave-uniform base (lane i -> base + 16*i).
+    // One instruction therefore fills 4 tile rows (16 lanes x 16 B each); wave w owns rows
+    // 16*w .. 16*w+15 of every tile (4 instructions per matrix).  Bank-conflict-free reads need
+    // the 16-byte chunks of a row permuted (K: chunk ^ row%16, V: chunk ^ 4*(row%4)); with DMA
+    // the permutation is applied on the global side: lane (row, c') loads global chunk c'^swz(row).
     // Rows that do not exist (past seqlen, or padding of a gathered tile) are read from a
-    // clamped, valid address instead of being zeroed: their scores are always masked to
-    // -inf below, so their probabilities are exactly 0 and K/V contents never matter.
-    const int ld_r = tid >> 4;       // 0..15
-    const int ld_c = tid & 15;       // 16-byte chunk in the row
-    u32x4_t kreg[4], vreg[4];        // in flight: next K tile, next V tile
-
-    // byte offset of this thread's first row inside a contiguous tile (rows 16 apart add a
-    // wave-uniform 16*pitch, so one 32-bit lane offset serves all four loads)
-    const unsigned koff = (unsigned)(ld_r * k_row + ld_c * 16);
-    const unsigned voff = (unsigned)(ld_r * v_row + ld_c * 16);
-    const bool small_pitch = k_row * 64 < (1ll << 31) && v_row * 64 < (1ll << 31);
-    // token ids of this thread's 4 rows of a gathered (column) tile
+    // clamped, valid address: their scores are always masked to -inf, so their probabilities are
+    // exactly 0 and the K/V contents never matter.
+    const int cp_r = lane >> 4;                  // row inside the 4-row group
+    const int cp_c = lane & 15;                  // LDS chunk
+    // token ids of this lane's 4 rows of a gathered (column) tile
     auto gather_ids = [&](const Tile &t, int (&tok)[4]) {
         if (MODE == MODE_VS && t.gathered) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                tok[i] = ix.ci[ridx * p.nnz_v + t.start + min(i * 16 + ld_r, t.nvalid - 1)];
+            for (int j = 0; j < 4; ++j)
+                tok[j] = ix.ci[ridx * p.nnz_v + t.start + min(16 * wave + 4 * j + cp_r, t.nvalid - 1)];
         }
     };
-    auto load_tile = [&](const Tile &t, const char *base, long long rowstride, const unsigned off,
-                         const int (&gtok)[4], u32x4_t (&dst)[4]) {
+    auto copy_tile = [&](const Tile &t, const char *base, long long rowstride, bool is_v, const int (&gtok)[4],
+                         char *ldsbuf) {
         const bool gathered = MODE == MODE_VS && t.gathered;
-        if (!gathered && small_pitch && t.start >= 0 && t.start + BN <= seqlen) {
-            // common case: one wave-uniform base, loop-invariant per-thread offsets
-            const char *tb = base + (long long)t.start * rowstride;
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                dst[i] = *reinterpret_cast<const u32x4_t *>(tb + (long long)i * 16 * rowstride + off);
-            return;
-        }
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int tok = gathered ? gtok[i] : t.start + i * 16 + ld_r;
+        for (int j = 0; j < 4; ++j) {
+            const int r = 16 * wave + 4 * j + cp_r;          // tile row
+            const int tok = gathered ? gtok[j] : t.start + r;
             const int tk = max(0, min(tok, seqlen - 1));
-            dst[i] = *reinterpret_cast<const u32x4_t *>(base + tk * rowstride + ld_c * 16);
-        }
-    };
-    char *const lds_k_st = lds_k + ld_r * K_PITCH + ld_c * 16;
-    char *const lds_v_st = lds_v + ld_r * V_PITCH + ld_c * 16;
-    auto store_k = [&](const u32x4_t (&src)[4]) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            *reinterpret_cast<u32x4_t *>(lds_k_st + i * 16 * K_PITCH) = src[i];
-        }
-    };
-    auto store_v = [&](const u32x4_t (&src)[4]) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            *reinterpret_cast<u32x4_t *>(lds_v_st + i * 16 * V_PITCH) = src[i];
+            const int c = is_v ? (cp_c ^ ((r & 3) << 2)) : (cp_c ^ (r & 15));
+            const char *gp = base + tk * rowstride + c * 16;
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
+                                             (__attribute__((address_space(3))) void *)(ldsbuf + (16 * wave + 4 * j) * ROW_BYTES),
+                                             16, 0, 0);
         }
     };
 
@@ -331,20 +311,28 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
 
     // V transpose read: row = T0 + (lane%16)/4, col = 32*db + 16*((lane/16)%2) + 4*(lane%4)
     const int v_rd_rsub = (lane & 15) >> 2;
-    const int v_rd_col = (((lane >> 4) & 1) << 4) + ((lane & 3) << 2);      // + 32*db
     const int wrow_lo = row0 + rw * 32, wrow_hi = wrow_lo + 31;
 
-    const char *const lds_k_rd = lds_k + (32 * kw + l32) * K_PITCH + g * 16;
-    const char *const lds_v_rd = lds_v + (32 * kw + 4 * g + v_rd_rsub) * V_PITCH + v_rd_col * 2;
+    // K read: row 32*kw + l32, logical chunk 2*ks + g -> physical chunk ^ (row % 16)
+    int k_rd_off[8];
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) k_rd_off[ks] = (32 * kw + l32) * ROW_BYTES + (((2 * ks + g) ^ (l32 & 15)) << 4);
+    // V transpose read: row 32*kw + 16*s2 + 8*jj + 4*g + rsub (row % 4 == rsub), logical chunk
+    // 4*db + vc -> physical 4*(db ^ rsub) + vc
+    const int v_rd_vc = (((lane >> 4) & 1) << 1) + ((lane & 3) >> 1);
+    int v_rd_off[4];
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+        v_rd_off[db] = (32 * kw + 4 * g + v_rd_rsub) * ROW_BYTES + ((((db ^ v_rd_rsub) << 2) + v_rd_vc) << 4) + ((lane & 1) << 3);
     // S^T of this wave: keys 32*kw + (0..31) of the tile in LDS x its 32 query rows
-    auto qk_tile = [&]() {
+    auto qk_tile = [&](const char *kbuf) {
         f32x16_t s;
 #pragma unroll
         for (int r = 0; r < 16; ++r) s[r] = 0.f;
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) {
             Frag a;
-            a.u = *reinterpret_cast<const u32x4_t *>(lds_k_rd + ks * 32);
+            a.u = *reinterpret_cast<const u32x4_t *>(kbuf + k_rd_off[ks]);
             s = Mma<T>::mfma(frag_as<T>(a), frag_as<T>(qf[ks]), s);
         }
         return s;
@@ -414,7 +402,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
         l_i = l_i * alpha + pair_sum<T>(pf[0]) + pair_sum<T>(pf[1]);
     };
 
-    auto pv_tile = [&](const Frag (&pf)[2]) {
+    auto pv_tile = [&](const Frag (&pf)[2], const char *vbuf) {
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2) {
 #pragma unroll
@@ -423,7 +411,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
 #pragma unroll
                 for (int jj = 0; jj < 2; ++jj) {
                     vf.s4[jj] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                        (__attribute__((address_space(3))) short4_t *)(lds_v_rd + (16 * s2 + 8 * jj) * V_PITCH + db * 64));
+                        (__attribute__((address_space(3))) short4_t *)(vbuf + v_rd_off[db] + (16 * s2 + 8 * jj) * ROW_BYTES));
                 }
                 oacc[db] = Mma<T>::mfma(frag_as<T>(vf), frag_as<T>(pf[s2]), oacc[db]);
             }
@@ -447,93 +435,78 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
     };
 
     // ---- software pipeline over tiles ----------------------------------------------
-    // Iteration `it` (t0 = tile it, t1 = it+1, ...; indices clamped to the last tile):
-    //   A : S_next = QK(t1) [Kbuf = K(t1)]  ||  softmax(S_cur = scores of t0)
-    //   barrier; store K(t2) -> Kbuf; load kreg <- K(t3)
-    //   B : O += P.V(t0)   [Vbuf = V(t0)]
-    //   barrier; store V(t1) -> Vbuf; load vreg <- V(t2)
-    // The QK MFMAs of the next tile share a basic block with the softmax VALU work of the
-    // current one; every LDS region is overwritten only after the barrier that follows its
-    // last read and read only after the barrier that follows its write.
+    // Step `it` (t0 = tile it, t1 = it+1, t2 = it+2; indices clamped to the last tile), with
+    // K/V double buffered in LDS (buffer parity = tile parity):
+    //   issue DMA  K(t2) -> Kbuf[it%2]   (held K(t0): last read before the previous barrier)
+    //              V(t1) -> Vbuf[(it+1)%2]
+    //   A : S_next = QK(t1) [Kbuf[(it+1)%2]]  ||  softmax(S_cur = scores of t0)
+    //   B : O += P.V(t0)    [Vbuf[it%2]]
+    //   wait for the DMA; barrier
+    // One barrier per tile; the QK MFMAs of the next tile share a basic block with the softmax
+    // VALU work of the current one.
     if (ntiles > 0) {
         const int last = ntiles - 1;
         Tile t0 = tile_at<MODE>(p, ix, ridx, m, nblk, 0);
         Tile t1 = tile_at<MODE>(p, ix, ridx, m, nblk, min(1, last));
         Tile t2 = tile_at<MODE>(p, ix, ridx, m, nblk, min(2, last));
         Tile t3 = tile_at<MODE>(p, ix, ridx, m, nblk, min(3, last));
-        // (global loads are issued in the same order as inside the loop -- gather ids, K, V -- so
-        // that the outstanding-load counters the waits are derived from agree on every path)
-        Tile t4 = tile_at<MODE>(p, ix, ridx, m, nblk, min(4, last));
-        int tokK[4] = {0, 0, 0, 0}, tokV[4] = {0, 0, 0, 0}, tokN[4] = {0, 0, 0, 0};
-        gather_ids(t0, tokK);
-        load_tile(t0, k_base, k_row, koff, tokK, kreg);
-        load_tile(t0, v_base, v_row, voff, tokK, vreg);
-        store_k(kreg);
-        store_v(vreg);
+        int tok0[4] = {0, 0, 0, 0}, tokV[4] = {0, 0, 0, 0}, tokK[4] = {0, 0, 0, 0}, tokN[4] = {0, 0, 0, 0};
+        gather_ids(t0, tok0);
         gather_ids(t1, tokV);
-        load_tile(t1, k_base, k_row, koff, tokV, kreg);
-        __syncthreads();
-        f32x16_t s_a = qk_tile();
-        __syncthreads();
-        store_k(kreg);
         gather_ids(t2, tokK);
         gather_ids(t3, tokN);
-        load_tile(t2, k_base, k_row, koff, tokK, kreg);
-        load_tile(t1, v_base, v_row, voff, tokV, vreg);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) tokV[i] = tokK[i];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) tokK[i] = tokN[i];
+        copy_tile(t0, k_base, k_row, false, tok0, lds_k0);
+        copy_tile(t0, v_base, v_row, true, tok0, lds_v0);
+        copy_tile(t1, k_base, k_row, false, tokV, lds_k1);
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+        f32x16_t s_a = qk_tile(lds_k0);
         __syncthreads();
 
-        // One pipeline step; the score registers ping-pong between two steps (no copies).
-        // On entry: Kbuf = K(t1), Vbuf = V(t0), kreg = K(t2) and vreg = V(t1) in flight;
-        // tokK / tokV = gathered token ids of t3 / t2 (if those are column tiles).
-        auto step = [&](f32x16_t &s_cur, f32x16_t &s_nxt, int it) {
+        // on entry: Kbuf[(it+1)%2] = K(t1), Vbuf[it%2] = V(t0) landed; tokK/tokV/tokN = gathered
+        // token ids of t2 / t1 / t3
+        auto step = [&](f32x16_t &s_cur, f32x16_t &s_nxt, int it, auto parity) {
+            constexpr int par = decltype(parity)::value;
             Frag pf[2];
             float alpha;
             bool rescale;
-            gather_ids(t4, tokN);          // needed one step from now: stays older than the K/V loads below
+            copy_tile(t2, k_base, k_row, false, tokK, par ? lds_k1 : lds_k0);
+            copy_tile(t1, v_base, v_row, true, tokV, par ? lds_v0 : lds_v1);
+            const char *kb = par ? lds_k0 : lds_k1;
             if (needs_mask(t0)) {
-                s_nxt = qk_tile();
+                s_nxt = qk_tile(kb);
                 softmax_tile(s_cur, t0, std::true_type{}, pf, alpha, rescale);
                 interleave_hint();
             } else {
-                s_nxt = qk_tile();
+                s_nxt = qk_tile(kb);
                 softmax_tile(s_cur, t0, std::false_type{}, pf, alpha, rescale);
                 interleave_hint();
             }
-            __syncthreads();
-            store_k(kreg);
-            load_tile(t3, k_base, k_row, koff, tokK, kreg);
             if (rescale) rescale_o(alpha);
-            pv_tile(pf);
-            __syncthreads();
-            store_v(vreg);
-            load_tile(t2, v_base, v_row, voff, tokV, vreg);
+            pv_tile(pf, par ? lds_v1 : lds_v0);
             t0 = t1;
             t1 = t2;
             t2 = t3;
-            t3 = t4;
-            t4 = tile_at<MODE>(p, ix, ridx, m, nblk, min(it + 5, last));
+            t3 = tile_at<MODE>(p, ix, ridx, m, nblk, min(it + 4, last));
 #pragma unroll
-            for (int i = 0; i < 4; ++i) tokV[i] = tokK[i];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) tokK[i] = tokN[i];
+            for (int i = 0; i < 4; ++i) { tokV[i] = tokK[i]; tokK[i] = tokN[i]; }
+            gather_ids(t3, tokN);
+            __builtin_amdgcn_s_waitcnt(0x0f70 | 0);   // vmcnt(0): the copies issued above have landed
+            __syncthreads();
         };
         f32x16_t s_b;
         for (int it = 0;;) {
-            step(s_a, s_b, it);
+            step(s_a, s_b, it, std::integral_constant<int, 0>{});
             if (++it >= ntiles) break;
-            step(s_b, s_a, it);
+            step(s_b, s_a, it, std::integral_constant<int, 1>{});
             if (++it >= ntiles) break;
         }
     }
 
     // ---- merge the two key halves: waves kw=1 hand (m, l, O) to waves kw=0 through LDS ----
     __syncthreads();
-    float *xo = reinterpret_cast<float *>(lds) + rw * (64 * 64);        // [reg 0..63][lane]
-    float *xml = reinterpret_cast<float *>(lds + 2 * 64 * 64 * 4) + rw * 128;   // [m|l][lane]
+    float *xo = reinterpret_cast<float *>(rw ? lds_k1 : lds_k0);       // [reg 0..63][lane]
+    float *xml = lds_ml + rw * 128;                                      // [m|l][lane]
     if (kw == 1) {
 #pragma unroll
         for (int db = 0; db < 4; ++db)
