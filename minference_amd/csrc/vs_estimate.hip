@@ -14,8 +14,9 @@
 //            registers, one (max, sum) pair per row per 1024-key chunk;
 //   reduce : combine the chunk pairs into M_i = max_i + log2(sum_i);
 //   scores : S = Q.K^T    -> lane <-> key: p = exp2(s - M_row); column sums are
-//            in-lane adds (+ one cross-half shuffle), diagonal sums go through
-//            LDS float atomics into a per-chunk window that is written out whole;
+//            in-lane adds (+ one cross-half shuffle); for the diagonal sums each wave parks
+//            its 64x32 probability block in LDS and every lane walks one diagonal with
+//            conflict-free strided reads (no atomics); the per-chunk window is written out whole;
 //   finalize: stitch the chunk windows together (each diagonal gets at most two
 //            pieces, added in a fixed order) and apply the forced +inf entries.
 // All arithmetic is fp32 on 16-bit inputs (the reference rounds q.k to bf16
@@ -122,11 +123,14 @@ __global__ __launch_bounds__(EST_THREADS) void est_stats_kernel(const EstParams 
     float m_run[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.f, 0.f};
     const int key_begin = w.chunk * KC + wave * (KC / 4);
     const int qpos0 = p.n - p.last_q;          // absolute position of query row 0
-    Frag kf[8];
+    Frag kf[8], kn[8];
+    load_k(p, kb, key_begin, lane, kn);
     for (int blk = 0; blk < KC / 4 / 32; ++blk) {
         const int c0 = key_begin + blk * 32;
         if (c0 >= p.n) break;
-        load_k(p, kb, c0, lane, kf);
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) kf[ks] = kn[ks];
+        load_k(p, kb, min(c0 + 32, p.n - 1), lane, kn);      // next block, in flight during this one
         f32x16_t st[2];
 #pragma unroll
         for (int nb = 0; nb < 2; ++nb) {
@@ -207,17 +211,28 @@ __global__ __launch_bounds__(LQ) void est_reduce_kernel(const EstParams p) {
 }
 
 // --------------------------------------------------------------- scores sweep
+// Diagonal sums without LDS float atomics (those run at a fraction of a lane per clock):
+// every wave parks its 64 x 32 probability block in a private LDS tile with a row pitch of
+// 33 floats, then lane d walks "its" diagonal (row i, key i + d) with conflict-free strided
+// reads -- 64 lanes cover d = -63..0, a second pass d = 1..31 -- and adds the 95 sums into a
+// private per-wave window with plain read-modify-write (one wave, in-order LDS: no race).
+constexpr int TP = 33;                       // tile row pitch (floats)
+constexpr int WWIN = KC / 4 + LQ;            // per-wave diagonal window (256 keys + 64)
+
 template <typename T>
 __global__ __launch_bounds__(EST_THREADS) void est_scores_kernel(const EstParams p) {
-    __shared__ float lds_win[WIN];
+    __shared__ float lds_tile[4][LQ * TP];
+    __shared__ float lds_wwin[4][WWIN];
     const WgId w = decode_wg(p);
     if (!w.valid) return;
     const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, g = lane >> 5;
     const char *kb = p.k + ((long long)w.b * p.ks[0] + (long long)w.hkv * p.ks[1]) * 2;
     const long long bh = (long long)w.b * p.hq + w.h;
+    float *tile = lds_tile[wave];
+    float *wwin = lds_wwin[wave];
 
-    for (int i = tid; i < WIN; i += EST_THREADS) lds_win[i] = 0.f;
+    for (int i = lane; i < WWIN; i += 64) wwin[i] = 0.f;
 
     Frag qf[2][8];
     load_q(p, w, lane, qf);
@@ -228,17 +243,20 @@ __global__ __launch_bounds__(EST_THREADS) void est_scores_kernel(const EstParams
 #pragma unroll
         for (int r = 0; r < 16; ++r)
             mrow[mb][r] = p.rowstat[bh * LQ + 32 * mb + 8 * (r >> 2) + 4 * g + (r & 3)];
-    __syncthreads();
 
     const int chunk0 = w.chunk * KC;
     const int key_begin = chunk0 + wave * (KC / 4);
     const int qpos0 = p.n - p.last_q;
+    const int rshift = LQ - p.last_q;          // rows are indexed as if last_q were 64
     float *vout = p.vertical + bh * p.n;
-    Frag kf[8];
+    Frag kf[8], kn[8];
+    load_k(p, kb, key_begin, lane, kn);
     for (int blk = 0; blk < KC / 4 / 32; ++blk) {
         const int c0 = key_begin + blk * 32;
         if (c0 >= p.n) break;
-        load_k(p, kb, c0, lane, kf);
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) kf[ks] = kn[ks];
+        load_k(p, kb, min(c0 + 32, p.n - 1), lane, kn);      // next block, in flight during this one
         const int c = c0 + l32;                 // this lane's key
         const bool edge = c0 + 31 > qpos0 || c0 + 32 > p.n;
         float colsum = 0.f;
@@ -255,17 +273,41 @@ __global__ __launch_bounds__(EST_THREADS) void est_scores_kernel(const EstParams
                 float pr = __builtin_amdgcn_exp2f(fmaf(s[r], p.scale_log2, -mrow[mb][r]));
                 if (edge) pr = (c <= qpos0 + i && c < p.n) ? pr : 0.f;
                 colsum += pr;
-                // diagonal index j = c + (last_q - 1 - i); window position j - chunk0
-                // (rows i >= last_q carry pr == 0; their position is clamped into the window)
-                atomicAdd(&lds_win[max(c - chunk0 + (p.last_q - 1 - i), 0)], pr);
+                tile[i * TP + l32] = pr;
             }
         }
         colsum += __shfl_xor(colsum, 32);
         if (g == 0 && c < p.n) vout[c] = colsum;
+        __builtin_amdgcn_wave_barrier();
+        // diagonal d = key - row (block-local key n, row i): window slot = 32*blk + d + 63 - rshift
+        // pass 1: lane <-> d = lane - 63 (d in [-63, 0]); pass 2: lane <-> d = lane + 1 (d in [1, 31])
+        float d1 = 0.f, d2 = 0.f;
+#pragma unroll
+        for (int n = 0; n < 32; ++n) {
+            const int i1 = n - (lane - 63);           // row on diagonal d1 at key n
+            if (i1 < LQ) d1 += tile[i1 * TP + n];
+            const int i2 = n - (lane + 1);
+            if (i2 >= 0) d2 += tile[i2 * TP + n];
+        }
+        // (rows i >= last_q hold exact zeros, so shifting by rshift only renames empty slots)
+        const int slot1 = 32 * blk + lane - rshift;
+        if (slot1 >= 0) wwin[slot1] += d1;
+        const int slot2 = 32 * blk + 64 + lane - rshift;
+        if (lane < 31 && slot2 >= 0) wwin[slot2] += d2;
+        __builtin_amdgcn_wave_barrier();
     }
     __syncthreads();
+    // chunk window position q = (key - chunk0) + (last_q - 1 - i): wave wv contributes its slot q - 64*4*wv/4...
     float *wout = p.win + (bh * p.nchunks + w.chunk) * WIN;
-    for (int i = tid; i < WIN; i += EST_THREADS) wout[i] = lds_win[i];
+    for (int q = tid; q < WIN; q += EST_THREADS) {
+        float acc = 0.f;
+#pragma unroll
+        for (int wv = 0; wv < 4; ++wv) {
+            const int sl = q - wv * (KC / 4);
+            if (sl >= 0 && sl < WWIN) acc += lds_wwin[wv][sl];
+        }
+        wout[q] = acc;
+    }
 }
 
 // ------------------------------------------------------------------- finalize
