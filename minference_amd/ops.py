@@ -36,14 +36,14 @@ def _prep(t: torch.Tensor) -> torch.Tensor:
 def _check_qkv(q, k, v):
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
         raise ValueError("q, k, v must be [batch, heads, n, head_dim]")
-    if not q.is_cuda:
-        raise RuntimeError("sparse attention operators need GPU tensors (there is no CPU path)")
     if k.shape != v.shape or q.shape[0] != k.shape[0] or q.shape[2:] != k.shape[2:]:
         raise ValueError(f"shape mismatch: q {tuple(q.shape)} k {tuple(k.shape)} v {tuple(v.shape)}")
     if q.shape[1] % k.shape[1] != 0:
         raise ValueError("query heads must be a multiple of key/value heads")
     if not (q.dtype == k.dtype == v.dtype):
         raise ValueError("q, k, v must share a dtype")
+    if not q.is_cuda:
+        raise RuntimeError("sparse attention operators need GPU tensors (there is no CPU path)")
 
 
 class _Call:

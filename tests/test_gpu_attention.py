@@ -142,3 +142,21 @@ def test_head_dim_64_is_padded(gpu):
     out = dense_causal_attention(q.to(gpu), k.to(gpu), v.to(gpu))
     assert out.shape == q.shape
     check(out, sdpa_causal(q, k, v), "d64")
+
+
+def test_golden_fixtures(gpu):
+    """The committed fixtures (tests/golden/small_cases.npz, written by make_golden.py from the
+    CPU oracle): index tensors bit-exact, the three operators within tolerance (fp16 inputs)."""
+    import os
+    import minference_amd as M
+    z = np.load(os.path.join(os.path.dirname(__file__), "golden", "small_cases.npz"))
+    n = int(z["n"])
+    out = M.convert_vertical_slash_indexes(torch.from_numpy(z["seqlens"]).to(gpu), torch.from_numpy(z["vertical"]).to(gpu),
+                                           torch.from_numpy(z["slash"]).to(gpu), n)
+    for got, name in zip(out, ["block_count", "block_offset", "column_count", "column_index"]):
+        assert np.array_equal(got.cpu().numpy(), z[name]), name
+    q, k, v = (torch.from_numpy(z[x]).to(gpu) for x in ("q", "k", "v"))
+    check(M.vertical_slash_sparse_attention(q, k, v, torch.from_numpy(z["vertical"]).to(gpu),
+                                            torch.from_numpy(z["slash"]).to(gpu)), torch.from_numpy(z["vs_out"]), "golden-vs")
+    check(M.streaming_forward(q, k, v, 8, 48), torch.from_numpy(z["ashape_out"]), "golden-ashape")
+    check(M.block_sparse_attention(q, k, v, 2), torch.from_numpy(z["bs_out"]), "golden-bs")

@@ -1,0 +1,96 @@
+"""Host-side logic that needs no GPU: per-head pattern planning of the dispatcher
+(reference minference/modules/minference_forward.py:594-674), argument checks of the
+operators, generators."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from minference_amd import prefill
+from tests import gen
+
+
+def cfg(best_pattern, **kw):
+    return {"best_pattern": best_pattern, **kw}
+
+
+def test_default_pattern_and_grouping():
+    layer = {"0": ["vertical_and_slash", 30, 800, 0.9], "1": ["stream_llm", 128, 4096, 0.8],
+             "3": ["block_sparse", 100, 6096, 0.7], "2": ["vertical_and_slash", 30, 800, 0.5]}
+    plan = prefill._head_plan(cfg([layer]), 0, 6)
+    assert plan[("vertical_and_slash", 30, 800)] == [0, 2]
+    assert plan[("stream_llm", 128, 4096)] == [1]
+    assert plan[("block_sparse", 100, 6096)] == [3]
+    assert plan[("vertical_and_slash", 1000, 6096)] == [4, 5]      # default entry (:621)
+
+
+def test_minference_ratio_truncates_like_the_reference():
+    layer = {"0": ["vertical_and_slash", 1000, 6096, 1]}
+    plan = prefill._head_plan(cfg([layer], minference_ratio=0.33), 0, 1)
+    assert list(plan) == [("vertical_and_slash", int(1000 * 0.33), int(6096 * 0.33))]
+
+
+def test_kv_head_selection_for_gqa_groups():
+    k = torch.arange(8).float().reshape(1, 8, 1, 1)
+    # whole groups -> the kv heads themselves (shared, not expanded)
+    sel = prefill._kv_for_heads(k, [4, 5, 6, 7, 12, 13, 14, 15], 4)
+    assert sel.flatten().tolist() == [1, 3]
+    # partial groups -> one kv head per query head
+    sel = prefill._kv_for_heads(k, [0, 5, 6], 4)
+    assert sel.flatten().tolist() == [0, 1, 1]
+    assert prefill._kv_for_heads(k, [2, 7], 1).flatten().tolist() == [2, 7]
+
+
+def test_is_search_is_rejected():
+    with pytest.raises(NotImplementedError):
+        prefill.minference_prefill_forward(torch.zeros(1, 1, 64, 128), torch.zeros(1, 1, 64, 128),
+                                           torch.zeros(1, 1, 64, 128),
+                                           {"layer_idx": 0, "attn_forward_config": {"is_search": True}})
+
+
+def test_shipped_pattern_files_have_the_expected_format():
+    path = "/root/reference/minference/configs/Llama_3_8B_Instruct_262k_kv_out_v32_fit_o_best_pattern.json"
+    if not os.path.exists(path):
+        pytest.skip("reference configs not present on this box")
+    pat = prefill.load_best_pattern(path)
+    assert len(pat) == 32 and len(pat[0]) == 32
+    plan = prefill._head_plan(cfg(pat), 5, 32)
+    assert sum(len(v) for v in plan.values()) == 32
+    for (ty, vs, ss) in plan:
+        assert ty in ("vertical_and_slash", "stream_llm", "block_sparse") and vs > 0 and ss > 0
+
+
+def test_operators_reject_cpu_tensors_and_bad_shapes():
+    import minference_amd as M
+    q = torch.zeros(1, 2, 64, 128, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError):
+        M.streaming_forward(q, q, q, 4, 16)
+    with pytest.raises(ValueError):
+        M.vertical_slash_sparse_attention(q, q, q, torch.zeros(1, 2, 4), torch.zeros(1, 2, 4), block_size_M=128)
+    with pytest.raises(ValueError):
+        M.block_sparse_attention(q, q, q, 10, block_size_N=32)
+    with pytest.raises(ValueError):
+        M.ops._check_qkv(q, q[:, :1], q)            # k/v shape mismatch
+    with pytest.raises(ValueError):
+        M.ops._check_qkv(torch.zeros(1, 3, 64, 128), torch.zeros(1, 2, 64, 128), torch.zeros(1, 2, 64, 128))
+
+
+def test_index_generator_matches_config3_description():
+    v, s = gen.vs_index_inputs(2, 4096, 100, 600, seed=300)
+    assert v.dtype == np.int32 and s.dtype == np.int32
+    for h in range(2):
+        assert (np.diff(v[0, h]) > 0).all() and (np.diff(s[0, h]) < 0).all()
+        assert set(range(4)) <= set(v[0, h].tolist()) and set(range(64)) <= set(s[0, h].tolist())
+
+
+def test_planted_layer_is_deterministic_and_structured():
+    q, k, v, meta = gen.planted_layer(2048, hq=4, hk=2, seed=7)
+    q2, k2, _, _ = gen.planted_layer(2048, hq=4, hk=2, seed=7)
+    assert torch.equal(q, q2) and torch.equal(k, k2)
+    assert q.shape == (1, 4, 2048, 128) and k.shape == (1, 2, 2048, 128) and q.dtype == torch.bfloat16
+    # positional code: last three dims of K are the base-128 digits of the position
+    pos = (k[0, 0, :, -3].float() * 16384 + k[0, 0, :, -2].float() * 128 + k[0, 0, :, -1].float())
+    assert torch.equal(pos, torch.arange(2048).float())
+    assert len(meta["heavy"]) == 2 and len(meta["heavy"][0]) == 32

@@ -1,0 +1,95 @@
+"""Pins the attention side of the oracle (masks + fp32 masked-dense softmax) through special
+cases that reduce to torch's scaled_dot_product_attention and per-element brute force."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+from tests import gen
+
+
+def sdpa(q, k, v, mask=None, causal=False):
+    return torch.nn.functional.scaled_dot_product_attention(
+        q[None, None].float(), k[None, None].float(), v[None, None].float(),
+        attn_mask=None if mask is None else torch.as_tensor(mask)[None, None], is_causal=causal)[0, 0]
+
+
+def test_masked_attention_equals_sdpa_with_mask():
+    q, k, v = gen.qkv(1, 1, 1, 200, 32, seed=1, scale=1.0)
+    rng = np.random.default_rng(0)
+    mask = np.tril(rng.random((200, 200)) < 0.3) | np.eye(200, dtype=bool)
+    out = O.masked_attention(q[0, 0], k[0, 0], v[0, 0], mask)
+    assert torch.allclose(out, sdpa(q[0, 0], k[0, 0], v[0, 0], mask), atol=1e-5)
+
+
+def test_vs_mask_all_offsets_is_causal():
+    n = 300
+    vi = np.zeros((1, 1, 1), np.int32)
+    si = np.arange(n, dtype=np.int32)[::-1][None, None]
+    bc, bo, cc, ci = O.vs_index_build([n], vi, si, n)
+    m = O.vs_mask(bc[0, 0], bo[0, 0], cc[0, 0], ci[0, 0], n)
+    assert np.array_equal(m, np.tril(np.ones((n, n), bool)))
+
+
+def test_vs_mask_matches_definition_bruteforce():
+    # the mask must be exactly {(r, c): c <= r, (r - c in S) up to 64-block granularity} U verticals:
+    # check the two guarantees that matter: every selected diagonal/vertical element is kept, and
+    # nothing above the diagonal is kept except listed columns (which are < row-block start)
+    n = 1000
+    vi, si = gen.vs_index_inputs(1, n, 20, 40, seed=2, force_v=2, force_s=3)
+    bc, bo, cc, ci = O.vs_index_build([n], vi, si, n)
+    m = O.vs_mask(bc[0, 0], bo[0, 0], cc[0, 0], ci[0, 0], n)
+    r, c = np.nonzero(m)
+    assert (c <= r).all()
+    S, V = set(si[0, 0].tolist()), set(vi[0, 0].tolist())
+    for rr in range(0, n, 37):
+        for cc_ in range(rr + 1):
+            if (rr - cc_) in S or cc_ in V:
+                assert m[rr, cc_], (rr, cc_)
+
+
+def test_block_sparse_index_properties_and_dense_limit():
+    n = 640
+    q, k, v = gen.qkv(1, 2, 2, n, 16, seed=3, scale=1.0)
+    bi = O.bs_block_index(q, k, 4)
+    assert bi.shape == (1, 2, 10, 4) and bi.dtype == torch.int32
+    for h in range(2):
+        for m in range(10):
+            row = bi[0, h, m].numpy()
+            assert (np.diff(row) > 0).all()
+            assert (row[: min(m + 1, 4)] <= m).all()      # causal picks sort first (reference :81-85)
+    # top_k >= number of blocks -> every causal block -> plain causal attention
+    out = O.block_sparse_attention(q, k, v, 100)
+    ref = torch.stack([sdpa(q[0, h], k[0, h], v[0, h], causal=True) for h in range(2)])[None]
+    assert torch.allclose(out, ref, atol=1e-5)
+    # forced diagonal + first block option
+    bf = O.bs_block_index(q, k, 3, force_diag_first=True)
+    for m in range(10):
+        assert 0 in bf[0, 0, m].tolist() and m in bf[0, 0, m].tolist()
+
+
+def test_ashape_mask_closed_form():
+    n, n_init, n_local = 257, 10, 40
+    m = O.ashape_mask(n, n_init, n_local)
+    for r in range(n):
+        for c in range(n):
+            exp = (c <= r) and ((r - c) < n_local or c < n_init)
+            assert m[r, c] == exp
+    assert np.array_equal(O.ashape_mask(100, 0, 100), np.tril(np.ones((100, 100), bool)))
+    q, k, v = gen.qkv(1, 1, 1, 100, 16, seed=4, scale=1.0)
+    out = O.streaming_forward(q, k, v, 4, 1000)
+    assert torch.allclose(out[0, 0], sdpa(q[0, 0], k[0, 0], v[0, 0], causal=True), atol=1e-5)
+
+
+def test_golden_fixtures_reproduce():
+    import os
+    path = os.path.join(os.path.dirname(__file__), "golden", "small_cases.npz")
+    z = np.load(path)
+    bc, bo, cc, ci = O.vs_index_build(z["seqlens"], z["vertical"], z["slash"], int(z["n"]))
+    assert np.array_equal(bc, z["block_count"]) and np.array_equal(bo, z["block_offset"])
+    assert np.array_equal(cc, z["column_count"]) and np.array_equal(ci, z["column_index"])
+    q, k, v = (torch.from_numpy(z[x]).float() for x in ("q", "k", "v"))
+    out = O.vertical_slash_sparse_attention(q, k, v, torch.from_numpy(z["vertical"]), torch.from_numpy(z["slash"]))
+    assert np.allclose(out.numpy(), z["vs_out"], atol=1e-6)
+    assert np.allclose(O.streaming_forward(q, k, v, 8, 48).numpy(), z["ashape_out"], atol=1e-6)
+    assert np.allclose(O.block_sparse_attention(q, k, v, 2).numpy(), z["bs_out"], atol=1e-6)
