@@ -95,8 +95,7 @@ def main():
         if record: e[0].record()
         vert, slash = M.vertical_slash_scores(q, k)
         if record: e[1].record()
-        v_idx = M.topk_indices(vert, vertical_size)
-        s_idx = M.topk_indices(slash, slash_size, reverse_base=n - 1)
+        v_idx, s_idx = M.estimate.topk_vertical_slash(vert, slash, vertical_size, slash_size)
         if record: e[2].record()
         bc, bo, cc, ci = M.convert_vertical_slash_indexes(seqlens, v_idx, s_idx, n, 64, 64, zero_fill=False)
         if record: e[3].record()

@@ -175,6 +175,16 @@ int minf_vs_estimate(const void *q, const void *k, const int64_t *q_stride,
 int minf_topk_indices(const float *scores, int rows, int n, int64_t row_stride, int k,
                       int32_t *out, int64_t out_stride, int reverse_base, void *stream);
 
+/*
+ * Two selections of minf_topk_indices in one launch (same rows / n / row_stride; separate k,
+ * output and reverse_base): the vertical and the slash top-k of a layer
+ * (reference minference/modules/minference_forward.py:607 and :612).
+ */
+int minf_topk_indices_pair(const float *scores_a, int k_a, int32_t *out_a, int64_t out_stride_a,
+                           int reverse_base_a, const float *scores_b, int k_b, int32_t *out_b,
+                           int64_t out_stride_b, int reverse_base_b, int rows, int n,
+                           int64_t row_stride, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -25,10 +25,25 @@ __device__ __forceinline__ unsigned order_key(float x) {
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);   // monotone for all finite/inf floats
 }
 
-__global__ __launch_bounds__(TK_THREADS) void topk_kernel(const float *__restrict__ scores,
-                                                           long long row_stride, int n, int k,
-                                                           int32_t *__restrict__ out,
-                                                           long long out_stride, int reverse_base) {
+struct TopkProblem {
+    const float *scores;
+    long long row_stride;
+    int k;
+    int32_t *out;
+    long long out_stride;
+    int reverse_base;
+};
+
+// blockIdx.y selects one of two problems over rows of the same length n (vertical and slash
+// scores of a layer are selected in one launch so that twice as many CUs are busy)
+__global__ __launch_bounds__(TK_THREADS) void topk_kernel(const TopkProblem p0, const TopkProblem p1, int n) {
+    const TopkProblem &pr = blockIdx.y == 0 ? p0 : p1;
+    const float *__restrict__ scores = pr.scores;
+    const long long row_stride = pr.row_stride;
+    const int k = pr.k;
+    int32_t *__restrict__ out = pr.out;
+    const long long out_stride = pr.out_stride;
+    const int reverse_base = pr.reverse_base;
     __shared__ unsigned hist[256];
     __shared__ unsigned sh_prefix, sh_need;
     __shared__ int wave_gt[TK_WAVES], wave_eq[TK_WAVES];
@@ -118,7 +133,22 @@ extern "C" int minf_topk_indices(const float *scores, int rows, int n, int64_t r
     if (!scores || !out || rows < 0 || n <= 0 || k <= 0) return MINF_ERR_INVALID_ARG;
     if (row_stride < n || out_stride < (k < n ? k : n)) return MINF_ERR_INVALID_ARG;
     if (rows == 0) return MINF_OK;
-    hipLaunchKernelGGL(topk_kernel, dim3((unsigned)rows), dim3(TK_THREADS), 0, (hipStream_t)stream,
-                       scores, (long long)row_stride, n, k, out, (long long)out_stride, reverse_base);
+    TopkProblem p{scores, (long long)row_stride, k, out, (long long)out_stride, reverse_base};
+    hipLaunchKernelGGL(topk_kernel, dim3((unsigned)rows, 1), dim3(TK_THREADS), 0, (hipStream_t)stream, p, p, n);
+    return minf_launch_status();
+}
+
+extern "C" int minf_topk_indices_pair(const float *scores_a, int k_a, int32_t *out_a, int64_t out_stride_a,
+                                      int reverse_base_a, const float *scores_b, int k_b, int32_t *out_b,
+                                      int64_t out_stride_b, int reverse_base_b, int rows, int n,
+                                      int64_t row_stride, void *stream) {
+    if (!scores_a || !out_a || !scores_b || !out_b || rows < 0 || n <= 0 || k_a <= 0 || k_b <= 0)
+        return MINF_ERR_INVALID_ARG;
+    if (row_stride < n || out_stride_a < (k_a < n ? k_a : n) || out_stride_b < (k_b < n ? k_b : n))
+        return MINF_ERR_INVALID_ARG;
+    if (rows == 0) return MINF_OK;
+    TopkProblem pa{scores_a, (long long)row_stride, k_a, out_a, (long long)out_stride_a, reverse_base_a};
+    TopkProblem pb{scores_b, (long long)row_stride, k_b, out_b, (long long)out_stride_b, reverse_base_b};
+    hipLaunchKernelGGL(topk_kernel, dim3((unsigned)rows, 2), dim3(TK_THREADS), 0, (hipStream_t)stream, pa, pb, n);
     return minf_launch_status();
 }

@@ -86,6 +86,19 @@ def estimate_vertical_slash(q, k, vertical_size, slash_size, last_q=LAST_Q,
     v = min(N, max(int(vertical_size), 30))
     s = min(N, max(int(slash_size), 50))
     vertical, slash = vertical_slash_scores(q, k, last_q, force_vertical, force_slash)
-    v_idx = topk_indices(vertical, v)
-    s_idx = topk_indices(slash, s, reverse_base=N - 1)
+    return topk_vertical_slash(vertical, slash, v, s)
+
+
+def topk_vertical_slash(vertical, slash, v, s):
+    """Both selections in one launch: -> (v_idx ascending positions, s_idx descending offsets)."""
+    B, H, N = vertical.shape
+    v, s = min(int(v), N), min(int(s), N)
+    v_idx = torch.empty((B, H, v), dtype=torch.int32, device=vertical.device)
+    s_idx = torch.empty((B, H, s), dtype=torch.int32, device=vertical.device)
+    lib = _lib.load()
+    with torch.cuda.device(vertical.device):
+        st = lib.minf_topk_indices_pair(vertical.data_ptr(), v, v_idx.data_ptr(), v, -1,
+                                        slash.data_ptr(), s, s_idx.data_ptr(), s, N - 1,
+                                        B * H, N, N, _lib.stream_ptr(vertical.device))
+    _lib.check(st, "minf_topk_indices_pair")
     return v_idx, s_idx
