@@ -16,15 +16,23 @@
 // the probabilities of a lane are exactly the B operand of the second MFMA once
 // the contraction (token) index is permuted the same way on the V side.
 //
-// LDS: K and V tiles are [64 tokens][128] 16-bit, 256 B per row, no padding;
-// 16-byte chunks are XOR-swizzled (K: chunk ^ row%16, V: chunk ^ 4*(row%4)) so
-// that ds_read_b128 of 16 rows and the 4-row transpose reads hit distinct banks.
-// Global->LDS goes through registers in half tiles (32 keys), prefetched a tile ahead, and the
-// main loop is software-pipelined over half tiles: the QK^T MFMAs of half tile h+1 are issued
-// next to the softmax VALU work of half tile h (see the schedule above the loop).
+// LDS: K and V tiles are [64 tokens][128] 16-bit with padded row pitches (K 272 B, V 320 B), so
+// the ds_read_b128 of 32 K rows and the 4-row transpose reads of V hit distinct banks and every
+// read address is a per-lane base plus an immediate offset.  Global->LDS goes through registers,
+// fetched one tile ahead; contiguous tiles use one scalar base per tile, gathered (vertical
+// column) tiles one 256-byte row per token.
+//
+// Other choices that measure faster on MI355X:
+//  * index entries (block offsets, column ids) are wave-uniform and read through the constant
+//    address space, i.e. scalar loads that do not queue behind the K/V vector loads;
+//  * the running max is only raised when a tile exceeds it by more than 2^8 (probabilities stay
+//    below 2^8, far inside fp32/bf16 range), so most tiles skip the O^T rescale;
+//  * the cross-half max uses v_permlane32_swap, the row sums v_dot2 on the rounded probabilities
+//    (the same values the second MFMA consumes);
+//  * s_setprio raises the wave while it issues MFMAs so the partner wave's softmax fills the gaps;
+//  * the epilogue transposes O^T through LDS so each global store is 16 B of one 256-byte row.
 #include "minf_common.h"
 #include <math.h>
-#include <type_traits>
 
 namespace {
 
@@ -41,10 +49,8 @@ enum { MODE_VS = 0, MODE_BS = 1, MODE_ASHAPE = 2, MODE_DENSE = 3 };
 constexpr int BM = 64;        // query rows per workgroup
 constexpr int BN = 64;        // keys per tile
 constexpr int HD = 128;       // head_dim
-constexpr int NTHREADS = 256; // 4 wavefronts: 2 row halves x 2 key halves
+constexpr int NTHREADS = 128; // 2 wavefronts
 constexpr int ROW_BYTES = HD * 2;
-constexpr int TILE_BYTES = BN * ROW_BYTES;          // 16 KB, rows unpadded, 16-byte chunks XOR-swizzled
-constexpr int LDS_BYTES = 4 * TILE_BYTES + 1024;    // K x2, V x2 (double buffered) [+ merge scratch]
 
 struct AttnParams {
     const char *q, *k, *v;
@@ -65,17 +71,8 @@ struct AttnParams {
     long long total_wg;
 };
 
-// The index tensors are read-only for the whole launch.  Their wave-uniform entries (counts,
-// block offsets, block ids) are read through constant-address-space pointers so that they become
-// scalar loads: a vector load whose result is needed at once would make the wave wait for every
-// K/V prefetch issued before it.  The gathered column ids stay vector loads (one per lane).
 typedef const __attribute__((address_space(4))) int *cint_ptr;
-struct IdxPtrs {
-    cint_ptr bc, bo, cc, bidx;
-    const int *ci;
-};
 __device__ __forceinline__ cint_ptr as_const(const int *p) { return (cint_ptr)(unsigned long long)p; }
-
 template <typename T> struct Mma;
 template <> struct Mma<__bf16> {
     typedef bf16x8_t vec;
@@ -111,7 +108,6 @@ template <> __device__ __forceinline__ void cvt8<_Float16>(const float *x, Frag 
     for (int j = 0; j < 8; ++j) f.h[j] = (_Float16)x[j];
 }
 
-// sum of the 8 (rounded) values of a fragment, via the 2-way dot-product instructions
 typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
 typedef __attribute__((__vector_size__(2 * sizeof(_Float16)))) _Float16 f16x2_t;
 template <typename T> __device__ __forceinline__ float pair_sum(const Frag &f);
@@ -119,23 +115,16 @@ template <> __device__ __forceinline__ float pair_sum<__bf16>(const Frag &f) {
     const bf16x2_t one = {(__bf16)1.0f, (__bf16)1.0f};
     float acc = 0.f;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        bf16x2_t pr = {f.b[2 * j], f.b[2 * j + 1]};
-        acc = __builtin_amdgcn_fdot2_f32_bf16(pr, one, acc, false);
-    }
+    for (int j = 0; j < 4; ++j) { bf16x2_t pr = {f.b[2 * j], f.b[2 * j + 1]}; acc = __builtin_amdgcn_fdot2_f32_bf16(pr, one, acc, false); }
     return acc;
 }
 template <> __device__ __forceinline__ float pair_sum<_Float16>(const Frag &f) {
     const f16x2_t one = {(_Float16)1.0f, (_Float16)1.0f};
     float acc = 0.f;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        f16x2_t pr = {f.h[2 * j], f.h[2 * j + 1]};
-        acc = __builtin_amdgcn_fdot2(pr, one, acc, false);
-    }
+    for (int j = 0; j < 4; ++j) { f16x2_t pr = {f.h[2 * j], f.h[2 * j + 1]}; acc = __builtin_amdgcn_fdot2(pr, one, acc, false); }
     return acc;
 }
-
 // One tile of keys: either 64 consecutive tokens from `start`, or 64 gathered
 // token ids read from `gather` (entries >= nvalid are padding).
 struct Tile {
@@ -145,10 +134,10 @@ struct Tile {
 };
 
 template <int MODE>
-__device__ __forceinline__ int tile_count(const AttnParams &p, const IdxPtrs &ix, long long ridx, int m, int &nblk) {
+__device__ __forceinline__ int tile_count(const AttnParams &p, long long ridx, int m, int &nblk) {
     if constexpr (MODE == MODE_VS) {
-        nblk = ix.bc[ridx];
-        return nblk + ((ix.cc[ridx] + BN - 1) >> 6);
+        nblk = as_const(p.bc)[ridx];
+        return nblk + ((as_const(p.cc)[ridx] + BN - 1) >> 6);
     } else if constexpr (MODE == MODE_BS) {
         nblk = min(m + 1, p.max_blocks);
         return nblk;
@@ -166,20 +155,20 @@ __device__ __forceinline__ int tile_count(const AttnParams &p, const IdxPtrs &ix
 }
 
 template <int MODE>
-__device__ __forceinline__ Tile tile_at(const AttnParams &p, const IdxPtrs &ix, long long ridx, int m, int nblk, int it) {
+__device__ __forceinline__ Tile tile_at(const AttnParams &p, long long ridx, int m, int nblk, int it) {
     Tile t;
     t.gathered = 0;
     t.nvalid = BN;
     if constexpr (MODE == MODE_VS) {
         if (it < nblk) {
-            t.start = ix.bo[ridx * p.nnz_s + it];
+            t.start = as_const(p.bo)[ridx * p.nnz_s + it];
         } else {
             t.gathered = 1;
             t.start = (it - nblk) * BN;
-            t.nvalid = min(BN, ix.cc[ridx] - t.start);
+            t.nvalid = min(BN, as_const(p.cc)[ridx] - t.start);
         }
     } else if constexpr (MODE == MODE_BS) {
-        t.start = ix.bidx[((ridx / p.rows) * p.bidx_rows + m) * p.max_blocks + it] * BN;
+        t.start = as_const(p.bidx)[((ridx / p.rows) * p.bidx_rows + m) * p.max_blocks + it] * BN;
     } else if constexpr (MODE == MODE_ASHAPE) {
         int lo_key = m * BM - p.n_local + 1;
         int t_lo = lo_key > 0 ? (lo_key >> 6) : 0;
@@ -192,18 +181,9 @@ __device__ __forceinline__ Tile tile_at(const AttnParams &p, const IdxPtrs &ix, 
 
 template <typename T, int MODE>
 __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams p) {
-    IdxPtrs ix;
-    ix.bc = as_const(p.bc); ix.bo = as_const(p.bo); ix.cc = as_const(p.cc); ix.bidx = as_const(p.bidx);
-    ix.ci = p.ci;
-    // K tile, V tile, and 1 KB for the (max, sum) pairs of the final merge; the O partials of
-    // the merge reuse the K/V space.
-    // K and V double buffers as four separate LDS objects: the compiler only lets an LDS read
-    // run ahead of an in-flight global->LDS copy when it can prove they touch different objects.
-    __shared__ __attribute__((aligned(16))) char lds_k0[TILE_BYTES];
-    __shared__ __attribute__((aligned(16))) char lds_k1[TILE_BYTES];
-    __shared__ __attribute__((aligned(16))) char lds_v0[TILE_BYTES];
-    __shared__ __attribute__((aligned(16))) char lds_v1[TILE_BYTES];
-    __shared__ float lds_ml[256];
+    constexpr int KP = ROW_BYTES + 16, VP = ROW_BYTES + 64;
+    __shared__ __attribute__((aligned(16))) char lds_k[BN * KP];
+    __shared__ __attribute__((aligned(16))) char lds_v[BN * VP];
 
     // ---- which (batch, head, row block): XCD-aware remap --------------------
     // Consecutive workgroup ids are dealt round-robin to the 8 XCDs; give each
@@ -216,7 +196,10 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
     const int group = p.hq / p.hk;
     long long rest = logical;
     const int hin = (int)(rest % group); rest /= group;
-    const int m = p.rows - 1 - (int)(rest % p.rows); rest /= p.rows;   // heavy (late) rows first
+    // Dense causal work grows with the row block, so the heavy (late) blocks go first; the sparse
+    // modes have near-constant work per row block and measure faster in ascending order.
+    const int mi = (int)(rest % p.rows); rest /= p.rows;
+    const int m = MODE == MODE_DENSE ? p.rows - 1 - mi : mi;
     const int hkv = (int)(rest % p.hk);
     const int b = (int)(rest / p.hk);
     const int h = hkv * group + hin;
@@ -224,14 +207,12 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
     const int tid = (int)threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    const int rw = wave & 1;          // which 32 query rows of the block
-    const int kw = wave >> 1;         // which 32 keys of every tile
     const int l32 = lane & 31;
     const int g = lane >> 5;
 
     const int seqlen = p.seqlens ? min(p.seqlens[b], p.n) : p.n;
     const int row0 = m * BM;
-    const int qrow = row0 + rw * 32 + l32;          // this lane's query row
+    const int qrow = row0 + wave * 32 + l32;          // this lane's query row
     char *o_base = p.o + ((long long)b * p.os[0] + (long long)h * p.os[1]) * 2;
 
     if (row0 >= seqlen) {
@@ -262,289 +243,220 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
     }
 
     int nblk = 0;
-    const int ntiles = tile_count<MODE>(p, ix, ridx, m, nblk);
+    const int ntiles = tile_count<MODE>(p, ridx, m, nblk);
 
-    // ---- global -> LDS copies without a register round trip --------------------------------
-    // global_load_lds_dwordx4: every lane fetches 16 bytes from its own global address and the
-    // wave's 64 x 16 B land CONTIGUOUSLY in LDS at a wave-uniform base (lane i -> base + 16*i).
-    // One instruction therefore fills 4 tile rows (16 lanes x 16 B each); wave w owns rows
-    // 16*w .. 16*w+15 of every tile (4 instructions per matrix).  Bank-conflict-free reads need
-    // the 16-byte chunks of a row permuted (K: chunk ^ row%16, V: chunk ^ 4*(row%4)); with DMA
-    // the permutation is applied on the global side: lane (row, c') loads global chunk c'^swz(row).
+    // ---- global -> register staging: thread covers rows i*8 + tid/16, chunk tid%16
+    const int ld_r = tid >> 4;       // 0..7
+    const int ld_c = tid & 15;       // 16-byte chunk in the row
+    u32x4_t kreg[8], vreg[8];
+
     // Rows that do not exist (past seqlen, or padding of a gathered tile) are read from a
-    // clamped, valid address: their scores are always masked to -inf, so their probabilities are
-    // exactly 0 and the K/V contents never matter.
-    const int cp_r = lane >> 4;                  // row inside the 4-row group
-    const int cp_c = lane & 15;                  // LDS chunk
-    // token ids of this lane's 4 rows of a gathered (column) tile
-    auto gather_ids = [&](const Tile &t, int (&tok)[4]) {
+    // clamped, valid address instead of being zeroed: their scores are always masked to
+    // -inf below, so their probabilities are exactly 0 and K/V contents never matter.
+    auto issue_loads = [&](const Tile &t) {
+        if (!(MODE == MODE_VS && t.gathered) && t.start >= 0 && t.start + BN <= seqlen) {
+            const char *kb = k_base + (long long)t.start * k_row;
+            const char *vb = v_base + (long long)t.start * v_row;
+            const unsigned ko = (unsigned)(ld_r * k_row + ld_c * 16), vo = (unsigned)(ld_r * v_row + ld_c * 16);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                kreg[i] = *reinterpret_cast<const u32x4_t *>(kb + (long long)i * 8 * k_row + ko);
+                vreg[i] = *reinterpret_cast<const u32x4_t *>(vb + (long long)i * 8 * v_row + vo);
+            }
+            return;
+        }
+        int tok[8];
         if (MODE == MODE_VS && t.gathered) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                tok[j] = ix.ci[ridx * p.nnz_v + t.start + min(16 * wave + 4 * j + cp_r, t.nvalid - 1)];
+            for (int i = 0; i < 8; ++i) {
+                const int r = i * 8 + ld_r;
+                tok[i] = p.ci[ridx * p.nnz_v + t.start + min(r, t.nvalid - 1)];
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) tok[i] = t.start + i * 8 + ld_r;
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int tk = max(0, min(tok[i], seqlen - 1));
+            kreg[i] = *reinterpret_cast<const u32x4_t *>(k_base + tk * k_row + ld_c * 16);
+            vreg[i] = *reinterpret_cast<const u32x4_t *>(v_base + tk * v_row + ld_c * 16);
         }
     };
-    auto copy_tile = [&](const Tile &t, const char *base, long long rowstride, bool is_v, const int (&gtok)[4],
-                         char *ldsbuf) {
-        const bool gathered = MODE == MODE_VS && t.gathered;
+    auto store_lds = [&]() {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int r = 16 * wave + 4 * j + cp_r;          // tile row
-            const int tok = gathered ? gtok[j] : t.start + r;
-            const int tk = max(0, min(tok, seqlen - 1));
-            const int c = is_v ? (cp_c ^ ((r & 3) << 2)) : (cp_c ^ (r & 15));
-            const char *gp = base + tk * rowstride + c * 16;
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
-                                             (__attribute__((address_space(3))) void *)(ldsbuf + (16 * wave + 4 * j) * ROW_BYTES),
-                                             16, 0, 0);
+        for (int i = 0; i < 8; ++i) {
+            const int r = i * 8 + ld_r;
+            *reinterpret_cast<u32x4_t *>(lds_k + r * KP + (ld_c << 4)) = kreg[i];
+            *reinterpret_cast<u32x4_t *>(lds_v + r * VP + (ld_c << 4)) = vreg[i];
         }
     };
 
-    // ---- accumulators (this wave's share: its 32 rows x its 32 keys of every tile) -----
+    // ---- accumulators -------------------------------------------------------
     f32x16_t oacc[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int r = 0; r < 16; ++r) oacc[i][r] = 0.f;
-    float m_i = -INFINITY;   // reference max of the row (log2 domain, scaled); lags the true max by <= 8
+    float m_i = -INFINITY;   // running max (log2 domain, scaled)
     float l_i = 0.f;         // this lane's share of the running sum
 
+    // LDS read addresses that do not depend on the tile
+    // K: row = 32*blk + l32, logical chunk 2*ks + g
+    const int k_rd_row = l32;
     // V transpose read: row = T0 + (lane%16)/4, col = 32*db + 16*((lane/16)%2) + 4*(lane%4)
     const int v_rd_rsub = (lane & 15) >> 2;
-    const int wrow_lo = row0 + rw * 32, wrow_hi = wrow_lo + 31;
+    const int v_rd_chunk = (((lane >> 4) & 1) << 1) + ((lane & 3) >> 1);   // + 4*db
+    const int v_rd_byte = (lane & 1) << 3;
 
-    // K read: row 32*kw + l32, logical chunk 2*ks + g -> physical chunk ^ (row % 16)
-    int k_rd_off[8];
+    Tile cur, nxt;
+    if (ntiles > 0) {
+        cur = tile_at<MODE>(p, ridx, m, nblk, 0);
+        issue_loads(cur);
+    }
+
+    for (int it = 0; it < ntiles; ++it) {
+        __syncthreads();            // previous tile fully consumed
+        store_lds();
+        __syncthreads();
+        if (it + 1 < ntiles) {
+            nxt = tile_at<MODE>(p, ridx, m, nblk, it + 1);
+            issue_loads(nxt);
+        }
+
+        __builtin_amdgcn_s_setprio(2);
+        // ---- S^T = K . Q^T --------------------------------------------------
+        f32x16_t s0, s1;
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) k_rd_off[ks] = (32 * kw + l32) * ROW_BYTES + (((2 * ks + g) ^ (l32 & 15)) << 4);
-    // V transpose read: row 32*kw + 16*s2 + 8*jj + 4*g + rsub (row % 4 == rsub), logical chunk
-    // 4*db + vc -> physical 4*(db ^ rsub) + vc
-    const int v_rd_vc = (((lane >> 4) & 1) << 1) + ((lane & 3) >> 1);
-    int v_rd_off[4];
-#pragma unroll
-    for (int db = 0; db < 4; ++db)
-        v_rd_off[db] = (32 * kw + 4 * g + v_rd_rsub) * ROW_BYTES + ((((db ^ v_rd_rsub) << 2) + v_rd_vc) << 4) + ((lane & 1) << 3);
-    // S^T of this wave: keys 32*kw + (0..31) of the tile in LDS x its 32 query rows
-    auto qk_tile = [&](const char *kbuf) {
-        f32x16_t s;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) s[r] = 0.f;
+        for (int r = 0; r < 16; ++r) { s0[r] = 0.f; s1[r] = 0.f; }
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) {
-            Frag a;
-            a.u = *reinterpret_cast<const u32x4_t *>(kbuf + k_rd_off[ks]);
-            s = Mma<T>::mfma(frag_as<T>(a), frag_as<T>(qf[ks]), s);
+            const int x = 2 * ks + g;
+            Frag a0, a1;
+            a0.u = *reinterpret_cast<const u32x4_t *>(lds_k + k_rd_row * KP + (x << 4));
+            a1.u = *reinterpret_cast<const u32x4_t *>(lds_k + (32 + k_rd_row) * KP + (x << 4));
+            s0 = Mma<T>::mfma(frag_as<T>(a0), frag_as<T>(qf[ks]), s0);
+            s1 = Mma<T>::mfma(frag_as<T>(a1), frag_as<T>(qf[ks]), s1);
         }
-        return s;
-    };
 
-    // does this wave have to mask anything in its keys [32*kw, 32*kw+32) of tile t ?
-    auto needs_mask = [&](const Tile &t) {
-        if (MODE == MODE_VS && t.gathered) return t.nvalid < 32 * kw + 32;
-        const int c_lo = t.start + 32 * kw, c_hi = c_lo + 31;
-        if constexpr (MODE == MODE_ASHAPE) {
-            const bool causal_ok = c_hi <= wrow_lo && c_hi < seqlen;
-            const bool in_window = (wrow_hi - c_lo) < p.n_local;
-            const bool in_sink = c_hi < p.n_init;
-            return !(causal_ok && (in_window || in_sink));
-        }
-        return (c_hi > wrow_lo) || (c_hi >= seqlen);
-    };
-
-    // online softmax of this wave's 32x32 score block (exp2 domain); s -> probabilities, packed
-    // into the B-operand fragments of the two PV k-steps; alpha = factor for the O accumulators.
-    // Element r of this lane is tile-local key 32*kw + 4*g + tkc, tkc = 8*(r/4) + r%4.
-    // keep <=> tkc <= hi && (tkc > wlo || tkc < slim).
-    auto softmax_tile = [&](f32x16_t &s, const Tile &t, auto masked, Frag (&pf)[2], float &alpha, bool &rescale) {
-        if constexpr (decltype(masked)::value) {
-            int hi, wlo = -1, slim = 0;
-            const int sh = 4 * g + 32 * kw;
-            if (MODE == MODE_VS && t.gathered) {
-                hi = t.nvalid - 1 - sh;
+        __builtin_amdgcn_s_setprio(0);
+        // ---- mask -----------------------------------------------------------
+        // element (blk, r) of this lane is tile-local key tk = tkc + 4*g with the compile-time
+        // part tkc = 32*blk + 8*(r/4) + r%4.  keep <=> tk <= hi && (tk > wlo || tk < slim).
+        bool need_mask;
+        const int wrow_lo = row0 + wave * 32, wrow_hi = wrow_lo + 31;
+        int hi, wlo = -1, slim = 0;      // per-lane bounds on tkc (4*g already subtracted)
+        if (MODE == MODE_VS && cur.gathered) {
+            need_mask = cur.nvalid < BN;
+            hi = cur.nvalid - 1 - 4 * g;
+        } else {
+            hi = min(qrow, seqlen - 1) - cur.start - 4 * g;
+            if constexpr (MODE == MODE_ASHAPE) {
+                const int c_lo = cur.start, c_hi = cur.start + BN - 1;
+                const bool causal_ok = c_hi <= wrow_lo && c_hi < seqlen;
+                const bool in_window = (wrow_hi - c_lo) < p.n_local;
+                const bool in_sink = c_hi < p.n_init;
+                need_mask = !(causal_ok && (in_window || in_sink));
+                wlo = qrow - cur.start - p.n_local - 4 * g;
+                slim = p.n_init - cur.start - 4 * g;
             } else {
-                hi = min(qrow, seqlen - 1) - t.start - sh;
-                if constexpr (MODE == MODE_ASHAPE) {
-                    wlo = qrow - t.start - p.n_local - sh;
-                    slim = p.n_init - t.start - sh;
-                }
+                need_mask = (cur.start + BN - 1 > wrow_lo) || (cur.start + BN > seqlen);
             }
+        }
+        if (need_mask) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int tkc = 8 * (r >> 2) + (r & 3);
-                bool kp = tkc <= hi;
-                if constexpr (MODE == MODE_ASHAPE) kp = kp & ((tkc > wlo) | (tkc < slim));
-                s[r] = kp ? s[r] : -INFINITY;
+                bool k0 = tkc <= hi, k1 = (tkc + 32) <= hi;
+                if constexpr (MODE == MODE_ASHAPE) {
+                    k0 = k0 & ((tkc > wlo) | (tkc < slim));
+                    k1 = k1 & (((tkc + 32) > wlo) | ((tkc + 32) < slim));
+                }
+                s0[r] = k0 ? s0[r] : -INFINITY;
+                s1[r] = k1 ? s1[r] : -INFINITY;
             }
         }
-        float mx = fmaxf(s[0], s[1]);
+
+        // ---- online softmax (exp2 domain) -------------------------------------
+        float mx = s0[0];
 #pragma unroll
-        for (int r = 2; r < 16; ++r) mx = fmaxf(mx, s[r]);
-        {
-            // max over the two lane halves (lanes l and l^32 hold the same query row)
-            const unsigned u = __float_as_uint(mx);
-            auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-            mx = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
-        }
-        // lazy reference max: only move it when the row max grew by more than 2^8
+        for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s0[r]);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s1[r]);
+        { const unsigned u = __float_as_uint(mx); auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false); mx = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1])); }
         const float cand = mx * p.scale_log2;
         const bool grow = cand > m_i + 8.0f;
-        const float m_next = grow ? cand : m_i;
-        alpha = grow ? __builtin_amdgcn_exp2f(m_i - m_next) : 1.0f;
-        rescale = __any(grow);
-        m_i = m_next;
-        const float m_sub = (m_next == -INFINITY) ? 0.f : m_next;
-        float pr[16];
+        const float m_new = grow ? cand : m_i;
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = grow ? __builtin_amdgcn_exp2f(m_i - m_use) : 1.0f;
+        m_i = m_new;
+        float psum = 0.f;
+        float pv[32];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) pr[r] = __builtin_amdgcn_exp2f(fmaf(s[r], p.scale_log2, -m_sub));
-        cvt8<T>(&pr[0], pf[0]);
-        cvt8<T>(&pr[8], pf[1]);
-        // row sum of the ROUNDED probabilities (what the PV product really uses)
-        l_i = l_i * alpha + pair_sum<T>(pf[0]) + pair_sum<T>(pf[1]);
-    };
+        for (int r = 0; r < 16; ++r) {
+            pv[r] = __builtin_amdgcn_exp2f(fmaf(s0[r], p.scale_log2, -m_use));
+            pv[16 + r] = __builtin_amdgcn_exp2f(fmaf(s1[r], p.scale_log2, -m_use));
+        }
+        Frag pfr[4];
+#pragma unroll
+        for (int s = 0; s < 4; ++s) { cvt8<T>(&pv[8 * s], pfr[s]); psum += pair_sum<T>(pfr[s]); }
+        l_i = l_i * alpha + psum;
+        if (__any(alpha != 1.0f)) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
+        }
 
-    auto pv_tile = [&](const Frag (&pf)[2], const char *vbuf) {
+        __builtin_amdgcn_s_setprio(2);
+        // ---- O^T += V^T . P^T -------------------------------------------------
 #pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2) {
+        for (int s = 0; s < 4; ++s) {
+            const Frag &pf = pfr[s];
 #pragma unroll
             for (int db = 0; db < 4; ++db) {
                 Frag vf;
 #pragma unroll
                 for (int jj = 0; jj < 2; ++jj) {
+                    const int row = 16 * s + 8 * jj + 4 * g + v_rd_rsub;
+                    const int chunk = (4 * db + v_rd_chunk);
                     vf.s4[jj] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                        (__attribute__((address_space(3))) short4_t *)(vbuf + v_rd_off[db] + (16 * s2 + 8 * jj) * ROW_BYTES));
+                        (__attribute__((address_space(3))) short4_t *)(lds_v + row * VP + (chunk << 4) + v_rd_byte));
                 }
-                oacc[db] = Mma<T>::mfma(frag_as<T>(vf), frag_as<T>(pf[s2]), oacc[db]);
+                oacc[db] = Mma<T>::mfma(frag_as<T>(vf), frag_as<T>(pf), oacc[db]);
             }
         }
-    };
-    auto rescale_o = [&](float alpha) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
-    };
-    // Ask the scheduler to spread the 8 QK MFMAs of a phase between the softmax VALU work of the
-    // same basic block: (1 LDS read, 1 MFMA, 10 VALU) x 8.
-    auto interleave_hint = [&]() {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x002, 10, 0);
-        }
-    };
-
-    // ---- software pipeline over tiles ----------------------------------------------
-    // Step `it` (t0 = tile it, t1 = it+1, t2 = it+2; indices clamped to the last tile), with
-    // K/V double buffered in LDS (buffer parity = tile parity):
-    //   issue DMA  K(t2) -> Kbuf[it%2]   (held K(t0): last read before the previous barrier)
-    //              V(t1) -> Vbuf[(it+1)%2]
-    //   A : S_next = QK(t1) [Kbuf[(it+1)%2]]  ||  softmax(S_cur = scores of t0)
-    //   B : O += P.V(t0)    [Vbuf[it%2]]
-    //   wait for the DMA; barrier
-    // One barrier per tile; the QK MFMAs of the next tile share a basic block with the softmax
-    // VALU work of the current one.
-    if (ntiles > 0) {
-        const int last = ntiles - 1;
-        Tile t0 = tile_at<MODE>(p, ix, ridx, m, nblk, 0);
-        Tile t1 = tile_at<MODE>(p, ix, ridx, m, nblk, min(1, last));
-        Tile t2 = tile_at<MODE>(p, ix, ridx, m, nblk, min(2, last));
-        Tile t3 = tile_at<MODE>(p, ix, ridx, m, nblk, min(3, last));
-        int tok0[4] = {0, 0, 0, 0}, tokV[4] = {0, 0, 0, 0}, tokK[4] = {0, 0, 0, 0}, tokN[4] = {0, 0, 0, 0};
-        gather_ids(t0, tok0);
-        gather_ids(t1, tokV);
-        gather_ids(t2, tokK);
-        gather_ids(t3, tokN);
-        copy_tile(t0, k_base, k_row, false, tok0, lds_k0);
-        copy_tile(t0, v_base, v_row, true, tok0, lds_v0);
-        copy_tile(t1, k_base, k_row, false, tokV, lds_k1);
-        __builtin_amdgcn_s_waitcnt(0);
-        __syncthreads();
-        f32x16_t s_a = qk_tile(lds_k0);
-        __syncthreads();
-
-        // on entry: Kbuf[(it+1)%2] = K(t1), Vbuf[it%2] = V(t0) landed; tokK/tokV/tokN = gathered
-        // token ids of t2 / t1 / t3
-        auto step = [&](f32x16_t &s_cur, f32x16_t &s_nxt, int it, auto parity) {
-            constexpr int par = decltype(parity)::value;
-            Frag pf[2];
-            float alpha;
-            bool rescale;
-            copy_tile(t2, k_base, k_row, false, tokK, par ? lds_k1 : lds_k0);
-            copy_tile(t1, v_base, v_row, true, tokV, par ? lds_v0 : lds_v1);
-            const char *kb = par ? lds_k0 : lds_k1;
-            if (needs_mask(t0)) {
-                s_nxt = qk_tile(kb);
-                softmax_tile(s_cur, t0, std::true_type{}, pf, alpha, rescale);
-                interleave_hint();
-            } else {
-                s_nxt = qk_tile(kb);
-                softmax_tile(s_cur, t0, std::false_type{}, pf, alpha, rescale);
-                interleave_hint();
-            }
-            if (rescale) rescale_o(alpha);
-            pv_tile(pf, par ? lds_v1 : lds_v0);
-            t0 = t1;
-            t1 = t2;
-            t2 = t3;
-            t3 = tile_at<MODE>(p, ix, ridx, m, nblk, min(it + 4, last));
-#pragma unroll
-            for (int i = 0; i < 4; ++i) { tokV[i] = tokK[i]; tokK[i] = tokN[i]; }
-            gather_ids(t3, tokN);
-            __builtin_amdgcn_s_waitcnt(0x0f70 | 0);   // vmcnt(0): the copies issued above have landed
-            __syncthreads();
-        };
-        f32x16_t s_b;
-        for (int it = 0;;) {
-            step(s_a, s_b, it, std::integral_constant<int, 0>{});
-            if (++it >= ntiles) break;
-            step(s_b, s_a, it, std::integral_constant<int, 1>{});
-            if (++it >= ntiles) break;
-        }
+        __builtin_amdgcn_s_setprio(0);
+        cur = nxt;
     }
 
-    // ---- merge the two key halves: waves kw=1 hand (m, l, O) to waves kw=0 through LDS ----
-    __syncthreads();
-    float *xo = reinterpret_cast<float *>(rw ? lds_k1 : lds_k0);       // [reg 0..63][lane]
-    float *xml = lds_ml + rw * 128;                                      // [m|l][lane]
-    if (kw == 1) {
-#pragma unroll
-        for (int db = 0; db < 4; ++db)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) xo[(db * 16 + r) * 64 + lane] = oacc[db][r];
-        xml[lane] = m_i;
-        xml[64 + lane] = l_i;
-    }
-    __syncthreads();
-    if (kw == 1) return;
+    // ---- epilogue: O = O^T / l, transposed through LDS so that every global store is 16 bytes
+    // of one row and 16 lanes cover a whole 256-byte row ---------------------------------------
     {
-        const float m1 = xml[lane], l1 = xml[64 + lane];
-        const float mm = fmaxf(m_i, m1);
-        const float mu = (mm == -INFINITY) ? 0.f : mm;
-        const float a0 = __builtin_amdgcn_exp2f(m_i - mu), a1 = __builtin_amdgcn_exp2f(m1 - mu);
-        l_i = l_i * a0 + l1 * a1;
-#pragma unroll
-        for (int db = 0; db < 4; ++db)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) oacc[db][r] = oacc[db][r] * a0 + xo[(db * 16 + r) * 64 + lane] * a1;
-    }
-
-    // ---- epilogue: O = O^T / l, store ------------------------------------------
-    float l_tot = l_i + __shfl_xor(l_i, 32);
-    const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
-    if (qrow < p.n) {
+        float l_tot = l_i + __shfl_xor(l_i, 32);
+        const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+        constexpr int OP = ROW_BYTES + 8;                 // pitch: 8-byte lane writes spread over all banks
+        __syncthreads();                                  // K/V tiles no longer needed
+        char *ot = lds_k + wave * 32 * OP;                // 32 rows per wave (8448 B <= half of lds_k)
         const bool live = qrow < seqlen;
-        char *orow = o_base + (long long)qrow * p.os[2] * 2;
 #pragma unroll
         for (int db = 0; db < 4; ++db)
 #pragma unroll
             for (int rq = 0; rq < 4; ++rq) {
-                // d = 32*db + 8*rq + 4*g + 0..3
                 union { T e[4]; u32x2_t u; } out4;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) out4.e[e] = live ? (T)(oacc[db][rq * 4 + e] * inv) : (T)0.f;
-                *reinterpret_cast<u32x2_t *>(orow + (32 * db + 8 * rq + 4 * g) * 2) = out4.u;
+                *reinterpret_cast<u32x2_t *>(ot + l32 * OP + (32 * db + 8 * rq + 4 * g) * 2) = out4.u;
             }
+        __builtin_amdgcn_wave_barrier();
+        // lane -> (row = 4*i + lane/16, chunk = lane%16)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int r = 4 * i + (lane >> 4);
+            const int grow = row0 + wave * 32 + r;
+            const u32x4_t val = *reinterpret_cast<const u32x4_t *>(ot + r * OP + (lane & 15) * 16);
+            if (grow < p.n) *reinterpret_cast<u32x4_t *>(o_base + (long long)grow * p.os[2] * 2 + (lane & 15) * 16) = val;
+        }
     }
 }
 
