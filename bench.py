@@ -25,6 +25,10 @@ sys.path.insert(0, ROOT)
 TILE_FLOP = 4 * 64 * 64 * 128           # QK^T + PV of one 64x64x128 tile
 PEAK_BF16_TFLOPS = 2500.0               # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
+# HBM bytes per launch of the vertical-slash attention kernel on the default workload (seq 131072,
+# seed 100), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a 1 GiB copy kernel
+# (profiles/sparse_path_c2_128k_hbm_traffic.txt): 2.191 GB read + 1.074 GB written.
+ATTN_TRAFFIC_BYTES_C2 = 2_190_874_000 + 1_073_742_000
 
 
 def cpu_baseline(budget_s=25.0):
@@ -64,6 +68,9 @@ def main():
     ap.add_argument("--seq", type=int, default=131072)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-dense", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch one plain 1 GiB -> 1 GiB device copy kernel, the known-size "
+                         "reference that scales FETCH_SIZE / WRITE_SIZE in a rocprofv3 --pmc run")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU only: this build has no multi-GPU path "
@@ -131,6 +138,13 @@ def main():
     est_bytes = hk * n * 128 * 2 * 2 + hq * 64 * 128 * 2 + hq * 2 * n * 4       # K read twice + Q + outputs
 
     extra = {}
+    if args.calibrate_copy:
+        src = torch.ones(1 << 28, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        torch.mul(src, 2.0, out=dst)                   # one elementwise kernel: reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        extra["calibrate_copy_bytes_each_way"] = src.numel() * 4
+        del src, dst
     if not args.no_dense:
         def timed(f, reps=2):
             f(); torch.cuda.synchronize()
@@ -166,7 +180,8 @@ def main():
                     "estimate": round(est_bytes / (stage_avg["estimate"] * 1e-3) / 1e9, 1)},
         "roofline": {"kernel": "attn_fwd_kernel<bf16, vertical-slash>", "bound": "mfma",
                      "achieved": round(eff_tflops, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(eff_tflops / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "frac": round(eff_tflops / PEAK_BF16_TFLOPS, 4),
+                     "traffic": ATTN_TRAFFIC_BYTES_C2 if n == 131072 else None,
                      "launch_ms": round(attn_ms, 3), "flop_per_launch": tiles * TILE_FLOP},
         **extra,
     }

@@ -29,7 +29,9 @@
 //    below 2^8, far inside fp32/bf16 range), so most tiles skip the O^T rescale;
 //  * the cross-half max uses v_permlane32_swap, the row sums v_dot2 on the rounded probabilities
 //    (the same values the second MFMA consumes);
-//  * s_setprio raises the wave while it issues MFMAs so the partner wave's softmax fills the gaps;
+//  * s_setprio raises the wave while it issues MFMAs so the partner wave's softmax fills the gaps
+//    (not in dense mode: at 128K dense is bound by L2 reuse between workgroups that stream the
+//    same K/V, and both the priority switch and the scalar-base loads measure 20 % slower there);
 //  * the epilogue transposes O^T through LDS so each global store is 16 B of one 256-byte row.
 #include "minf_common.h"
 #include <math.h>
@@ -254,7 +256,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
     // clamped, valid address instead of being zeroed: their scores are always masked to
     // -inf below, so their probabilities are exactly 0 and K/V contents never matter.
     auto issue_loads = [&](const Tile &t) {
-        if (!(MODE == MODE_VS && t.gathered) && t.start >= 0 && t.start + BN <= seqlen) {
+        if (MODE != MODE_DENSE && !(MODE == MODE_VS && t.gathered) && t.start >= 0 && t.start + BN <= seqlen) {
             const char *kb = k_base + (long long)t.start * k_row;
             const char *vb = v_base + (long long)t.start * v_row;
             const unsigned ko = (unsigned)(ld_r * k_row + ld_c * 16), vo = (unsigned)(ld_r * v_row + ld_c * 16);
@@ -324,7 +326,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
             issue_loads(nxt);
         }
 
-        __builtin_amdgcn_s_setprio(2);
+        if (MODE != MODE_DENSE) __builtin_amdgcn_s_setprio(2);
         // ---- S^T = K . Q^T --------------------------------------------------
         f32x16_t s0, s1;
 #pragma unroll
@@ -339,7 +341,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
             s1 = Mma<T>::mfma(frag_as<T>(a1), frag_as<T>(qf[ks]), s1);
         }
 
-        __builtin_amdgcn_s_setprio(0);
+        if (MODE != MODE_DENSE) __builtin_amdgcn_s_setprio(0);
         // ---- mask -----------------------------------------------------------
         // element (blk, r) of this lane is tile-local key tk = tkc + 4*g with the compile-time
         // part tkc = 32*blk + 8*(r/4) + r%4.  keep <=> tk <= hi && (tk > wlo || tk < slim).
@@ -408,7 +410,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
                 for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
         }
 
-        __builtin_amdgcn_s_setprio(2);
+        if (MODE != MODE_DENSE) __builtin_amdgcn_s_setprio(2);
         // ---- O^T += V^T . P^T -------------------------------------------------
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
@@ -426,7 +428,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
                 oacc[db] = Mma<T>::mfma(frag_as<T>(vf), frag_as<T>(pf), oacc[db]);
             }
         }
-        __builtin_amdgcn_s_setprio(0);
+        if (MODE != MODE_DENSE) __builtin_amdgcn_s_setprio(0);
         cur = nxt;
     }
 
