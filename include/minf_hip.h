@@ -185,6 +185,28 @@ int minf_topk_indices_pair(const float *scores_a, int k_a, int32_t *out_a, int64
                            int64_t out_stride_b, int reverse_base_b, int rows, int n,
                            int64_t row_stride, void *stream);
 
+/*
+ * Block index of top-k block-sparse attention: replaces _build_block_index (reference
+ * minference/ops/block_sparse_flash_attention.py:151-166) together with the zero padding its
+ * caller applies first (:178-180).  Q and K are mean-pooled over 64-token blocks (the token axis
+ * padded with 64 - n%64 zero rows, i.e. a whole extra block when n%64 == 0), every (query block,
+ * key block) pair is scored with the pooled vectors, key blocks above the diagonal get -inf, and
+ * the min(top_k, rows) best key blocks of every query block are written in ascending order (ties:
+ * lowest block id first; torch.topk leaves the tie order unspecified).  fp32 arithmetic.
+ * force_diag_first != 0 additionally keeps the diagonal block and block 0 of every query block.
+ *   rows = minf_bs_block_index_rows(n) = (n + 64 - n%64) / 64
+ *   block_index [batch, heads_q, rows, min(top_k, rows)] int32, contiguous
+ *   q [batch, heads_q, n, 128], k [batch, heads_kv, n, 128]: base pointer + element strides
+ *   workspace: minf_bs_block_index_workspace_bytes() bytes, 16-byte aligned
+ */
+int minf_bs_block_index_rows(int n);
+size_t minf_bs_block_index_workspace_bytes(int batch, int heads_q, int heads_kv, int n);
+int minf_bs_block_index(const void *q, const void *k, const int64_t *q_stride,
+                        const int64_t *k_stride, int batch, int heads_q, int heads_kv, int n,
+                        int head_dim, int dtype, int top_k, int force_diag_first,
+                        int32_t *block_index, void *workspace, size_t workspace_bytes,
+                        void *stream);
+
 #ifdef __cplusplus
 }
 #endif

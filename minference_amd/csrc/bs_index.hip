@@ -1,0 +1,204 @@
+// Block index of block-sparse attention for gfx950: mean-pool Q and K over 64-token blocks,
+// score every (query block, key block) pair with the pooled vectors, keep the top-k key blocks
+// per query block in ascending order (reference
+// minference/ops/block_sparse_flash_attention.py:151-166, with the zero padding of :178-180
+// folded in: the token axis is padded by 64 - n%64 zeros, a whole block when n%64 == 0).
+//
+//   bs_pool_kernel    one workgroup per (head, block): 64 rows x 128 dims of 16-bit input summed in
+//                     fp32 (each thread 4 rows x 8 dims, then a fixed-order LDS reduction) -> mean.
+//                     HBM-bound: reads Q and K once.
+//   bs_scores_kernel  pooled Q . pooled K^T on the fp32 matrix cores (v_mfma_f32_32x32x2_f32), one
+//                     wave per 32 query blocks x 32 key blocks, operands loaded straight from global
+//                     memory in MFMA layout; applies the block-causal mask (-inf above the diagonal)
+//                     and, optionally, forces the diagonal block and block 0 (+inf).
+//   top-k             the shared radix-select kernel (ascending index order, ties -> lowest index).
+//
+// Arithmetic is fp32 throughout; the reference pools and multiplies in the input dtype (bf16/fp16
+// rounding after the mean and after the product), which this build does not imitate.
+#include "minf_common.h"
+#include <math.h>
+
+extern "C" int minf_topk_indices(const float *scores, int rows, int n, int64_t row_stride, int k,
+                                 int32_t *out, int64_t out_stride, int reverse_base, void *stream);
+
+namespace {
+
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
+typedef __attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned u32x4_t;
+
+constexpr int HD = 128;
+constexpr int BLK = 64;
+
+struct PoolParams {
+    const char *x;            // [batch, heads, n, 128] 16-bit, element strides below
+    long long xs[3];
+    float *out;               // [batch*heads, rows, 128] fp32
+    int heads, n, rows;
+};
+
+template <typename T> __device__ __forceinline__ float to_f32(unsigned short bits);
+template <> __device__ __forceinline__ float to_f32<__bf16>(unsigned short bits) {
+    return __uint_as_float((unsigned)bits << 16);
+}
+template <> __device__ __forceinline__ float to_f32<_Float16>(unsigned short bits) {
+    union { unsigned short u; _Float16 h; } c;
+    c.u = bits;
+    return (float)c.h;
+}
+
+template <typename T> __global__ __launch_bounds__(256) void bs_pool_kernel(const PoolParams p) {
+    __shared__ float red[16][HD + 4];
+    const int blk = blockIdx.x;
+    const int bh = blockIdx.y;
+    const int b = bh / p.heads, h = bh % p.heads;
+    const int tid = (int)threadIdx.x;
+    const int c = tid & 15, r4 = tid >> 4;
+    const char *base = p.x + ((long long)b * p.xs[0] + (long long)h * p.xs[1]) * 2;
+    float acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int tok = blk * BLK + r4 + 16 * j;
+        if (tok < p.n) {
+            const u32x4_t raw = *reinterpret_cast<const u32x4_t *>(base + (long long)tok * p.xs[2] * 2 + c * 16);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                acc[2 * e] += to_f32<T>((unsigned short)(raw[e] & 0xffffu));
+                acc[2 * e + 1] += to_f32<T>((unsigned short)(raw[e] >> 16));
+            }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) red[r4][c * 8 + e] = acc[e];
+    __syncthreads();
+    if (tid < HD) {
+        float s = 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s += red[r][tid];
+        p.out[((long long)bh * p.rows + blk) * HD + tid] = s * (1.0f / BLK);
+    }
+}
+
+struct ScoreParams {
+    const float *qp, *kp;     // pooled [batch*heads_q, rows, 128], [batch*heads_kv, rows, 128]
+    float *scores;            // [batch*heads_q, rows, pitch]
+    int heads_q, heads_kv, rows, pitch, force;
+    int mtiles, ntiles;
+};
+
+// lane l supplies row l%32 and, for MFMA step (s, j), contraction index 8*s + 4*(l/32) + j:
+// sixteen 16-byte loads cover the lane's half of the 128-dim row.
+__device__ __forceinline__ void load_operand(const float *base, int row, int rows, int g, f32x4_t (&x)[16]) {
+    const float *src = base + (long long)min(row, rows - 1) * HD + 4 * g;
+#pragma unroll
+    for (int s = 0; s < 16; ++s) x[s] = *reinterpret_cast<const f32x4_t *>(src + 8 * s);
+}
+
+__global__ __launch_bounds__(256) void bs_scores_kernel(const ScoreParams p) {
+    const int lane = (int)threadIdx.x & 63, wave = (int)threadIdx.x >> 6;
+    const int l32 = lane & 31, g = lane >> 5;
+    const int mt = p.mtiles - 1 - (int)blockIdx.x;            // heavy (late) query tiles first
+    const int bh = blockIdx.y;
+    const int b = bh / p.heads_q, h = bh % p.heads_q;
+    const int hkv = h / (p.heads_q / p.heads_kv);
+    const float *qbase = p.qp + (long long)bh * p.rows * HD;
+    const float *kbase = p.kp + ((long long)b * p.heads_kv + hkv) * p.rows * HD;
+    float *out = p.scores + (long long)bh * p.rows * p.pitch;
+    const int m0 = mt * 32;
+
+    f32x4_t aq[16], bk[16];
+    load_operand(qbase, m0 + l32, p.rows, g, aq);             // A operand: query blocks -> accumulator rows
+    for (int nt = wave; nt < p.ntiles; nt += 4) {
+        const int n0 = nt * 32;
+        f32x16_t acc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+        if (n0 <= m0 + 31) {
+            load_operand(kbase, n0 + l32, p.rows, g, bk);     // B operand: key blocks -> accumulator columns
+#pragma unroll
+            for (int s = 0; s < 16; ++s)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(aq[s][j], bk[s][j], acc, 0, 0, 0);
+        }
+        // accumulator element r of lane l: query block m0 + 8*(r/4) + 4*g + r%4, key block n0 + l%32,
+        // so every store instruction writes two full 128-byte row segments
+        const int ncol = n0 + l32;
+        if (ncol < p.pitch) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int mrow = m0 + 8 * (r >> 2) + 4 * g + (r & 3);
+                float x = ncol <= mrow ? acc[r] : -INFINITY;
+                if (p.force && (ncol == mrow || ncol == 0)) x = INFINITY;
+                if (mrow < p.rows) out[(long long)mrow * p.pitch + ncol] = x;
+            }
+        }
+    }
+}
+
+inline int padded_rows(int n) { return (n + (BLK - (n & (BLK - 1)))) / BLK; }
+inline int score_pitch(int rows) { return (rows + 3) & ~3; }
+inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+}  // namespace
+
+extern "C" int minf_bs_block_index_rows(int n) { return n < 0 ? 0 : padded_rows(n); }
+
+extern "C" size_t minf_bs_block_index_workspace_bytes(int batch, int heads_q, int heads_kv, int n) {
+    if (batch <= 0 || heads_q <= 0 || heads_kv <= 0 || n <= 0) return 0;
+    const size_t rows = (size_t)padded_rows(n);
+    return align256((size_t)batch * heads_q * rows * HD * 4) + align256((size_t)batch * heads_kv * rows * HD * 4) +
+           align256((size_t)batch * heads_q * rows * score_pitch((int)rows) * 4);
+}
+
+extern "C" int minf_bs_block_index(const void *q, const void *k, const int64_t *q_stride,
+                                   const int64_t *k_stride, int batch, int heads_q, int heads_kv,
+                                   int n, int head_dim, int dtype, int top_k, int force_diag_first,
+                                   int32_t *block_index, void *workspace, size_t workspace_bytes,
+                                   void *stream) {
+    if (!q || !k || !q_stride || !k_stride || !block_index) return MINF_ERR_INVALID_ARG;
+    if (batch < 0 || heads_q <= 0 || heads_kv <= 0 || n <= 0 || top_k <= 0) return MINF_ERR_INVALID_ARG;
+    if (heads_q % heads_kv != 0) return MINF_ERR_INVALID_ARG;
+    if (head_dim != HD) return MINF_ERR_UNSUPPORTED;
+    if (dtype != MINF_BF16 && dtype != MINF_F16) return MINF_ERR_UNSUPPORTED;
+    if (((uintptr_t)q | (uintptr_t)k) & 15) return MINF_ERR_ALIGNMENT;
+    for (int i = 0; i < 3; ++i)
+        if ((q_stride[i] | k_stride[i]) & 7) return MINF_ERR_ALIGNMENT;
+    if (batch == 0) return MINF_OK;
+    const size_t need = minf_bs_block_index_workspace_bytes(batch, heads_q, heads_kv, n);
+    if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 15)) return MINF_ERR_WORKSPACE;
+    const int rows = padded_rows(n);
+    const int pitch = score_pitch(rows);
+    if ((long long)batch * heads_q * rows > 0x7fffffffLL || (long long)batch * heads_q > 65535) return MINF_ERR_UNSUPPORTED;
+
+    char *ws = (char *)workspace;
+    float *qp = (float *)ws;
+    ws += align256((size_t)batch * heads_q * rows * HD * 4);
+    float *kp = (float *)ws;
+    ws += align256((size_t)batch * heads_kv * rows * HD * 4);
+    float *scores = (float *)ws;
+    hipStream_t st = (hipStream_t)stream;
+
+    PoolParams pq{(const char *)q, {q_stride[0], q_stride[1], q_stride[2]}, qp, heads_q, n, rows};
+    PoolParams pk{(const char *)k, {k_stride[0], k_stride[1], k_stride[2]}, kp, heads_kv, n, rows};
+    if (dtype == MINF_BF16) {
+        hipLaunchKernelGGL(bs_pool_kernel<__bf16>, dim3(rows, batch * heads_q), dim3(256), 0, st, pq);
+        hipLaunchKernelGGL(bs_pool_kernel<__bf16>, dim3(rows, batch * heads_kv), dim3(256), 0, st, pk);
+    } else {
+        hipLaunchKernelGGL(bs_pool_kernel<_Float16>, dim3(rows, batch * heads_q), dim3(256), 0, st, pq);
+        hipLaunchKernelGGL(bs_pool_kernel<_Float16>, dim3(rows, batch * heads_kv), dim3(256), 0, st, pk);
+    }
+    int status = minf_launch_status();
+    if (status != MINF_OK) return status;
+
+    ScoreParams sp{qp, kp, scores, heads_q, heads_kv, rows, pitch, force_diag_first ? 1 : 0,
+                   (rows + 31) / 32, (pitch + 31) / 32};
+    hipLaunchKernelGGL(bs_scores_kernel, dim3(sp.mtiles, batch * heads_q), dim3(256), 0, st, sp);
+    status = minf_launch_status();
+    if (status != MINF_OK) return status;
+
+    const int kk = top_k < rows ? top_k : rows;
+    return minf_topk_indices(scores, batch * heads_q * rows, rows, pitch, kk, block_index, kk, -1, stream);
+}

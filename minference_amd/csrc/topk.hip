@@ -1,7 +1,8 @@
 // Top-k index selection over fp32 score rows for gfx950 (vertical / slash
 // candidates: k = 1000 / 6096 of up to ~10^6 entries per head).
 //
-// One 1024-thread workgroup per row:
+// Rows longer than 4096 entries, one 1024-thread workgroup per row (shorter rows: one wavefront
+// per row, see topk_wave_kernel):
 //   1. MSB-first radix select (4 x 8 bits, LDS histogram) finds the exact value
 //      T of the k-th largest entry and how many entries equal to T are needed;
 //   2. every wavefront counts, over its contiguous slice, entries > T and == T;
@@ -126,6 +127,73 @@ __global__ __launch_bounds__(TK_THREADS) void topk_kernel(const TopkProblem p0, 
     }
 }
 
+// Short rows (n <= 64 * ITEMS <= 4096, e.g. the block scores of block-sparse attention): one
+// wavefront per row, the row held in registers (lane l owns indices l, l+64, ...).  The k-th
+// largest key is found bit by bit: T = the largest value with count(key >= T) >= k, 32 counting
+// passes of one compare + ballot popcount per element (no LDS, no barriers); the emit is the same
+// ordered ballot-prefix write as in the wide kernel, so both kernels select identical sets.
+constexpr int TKW_WAVES = 4;
+template <int ITEMS>
+__global__ __launch_bounds__(TKW_WAVES * 64) void topk_wave_kernel(const TopkProblem p0, const TopkProblem p1,
+                                                                   int n, int rows) {
+    const TopkProblem &pr = blockIdx.y == 0 ? p0 : p1;
+    const int lane = (int)threadIdx.x & 63, wave = (int)threadIdx.x >> 6;
+    const int row = (int)blockIdx.x * TKW_WAVES + wave;
+    if (row >= rows) return;
+    const float *__restrict__ x = pr.scores + (long long)row * pr.row_stride;
+    int32_t *__restrict__ o = pr.out + (long long)row * pr.out_stride;
+    const int k = pr.k, reverse_base = pr.reverse_base;
+    if (k >= n) {
+        for (int i = lane; i < n; i += 64) o[i] = reverse_base >= 0 ? reverse_base - i : i;
+        return;
+    }
+    unsigned key[ITEMS];
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) {
+        const int i = j * 64 + lane;
+        key[j] = i < n ? order_key(x[i]) : 0u;      // padding sorts below every real score
+    }
+    unsigned T = 0;
+    for (int bit = 31; bit >= 0; --bit) {
+        const unsigned cand = T | (1u << bit);
+        int cnt = 0;
+#pragma unroll
+        for (int j = 0; j < ITEMS; ++j) cnt += __builtin_popcountll(__ballot(key[j] >= cand));
+        if (cnt >= k) T = cand;
+    }
+    int cgt = 0;
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) cgt += __builtin_popcountll(__ballot(key[j] > T));
+    const int r = k - cgt;                           // entries equal to T that are taken, lowest index first
+    int gt_before = 0, eq_before = 0;
+    const uint64_t lt = minf_lanemask_lt();
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) {
+        const int i = j * 64 + lane;
+        const bool gt = key[j] > T, eq = key[j] == T;
+        const uint64_t mg = __ballot(gt), me = __ballot(eq);
+        const int e_here = eq_before + __builtin_popcountll(me & lt);
+        if (gt || (eq && e_here < r)) {
+            const int pos = gt_before + __builtin_popcountll(mg & lt) + min(e_here, r);
+            o[pos] = reverse_base >= 0 ? reverse_base - i : i;
+        }
+        gt_before += __builtin_popcountll(mg);
+        eq_before += __builtin_popcountll(me);
+    }
+}
+
+void launch_topk(const TopkProblem &pa, const TopkProblem &pb, int problems, int rows, int n, hipStream_t st) {
+    const dim3 grid_w((unsigned)((rows + TKW_WAVES - 1) / TKW_WAVES), (unsigned)problems);
+    if (n <= 64 * 4)
+        hipLaunchKernelGGL(topk_wave_kernel<4>, grid_w, dim3(TKW_WAVES * 64), 0, st, pa, pb, n, rows);
+    else if (n <= 64 * 16)
+        hipLaunchKernelGGL(topk_wave_kernel<16>, grid_w, dim3(TKW_WAVES * 64), 0, st, pa, pb, n, rows);
+    else if (n <= 64 * 64)
+        hipLaunchKernelGGL(topk_wave_kernel<64>, grid_w, dim3(TKW_WAVES * 64), 0, st, pa, pb, n, rows);
+    else
+        hipLaunchKernelGGL(topk_kernel, dim3((unsigned)rows, (unsigned)problems), dim3(TK_THREADS), 0, st, pa, pb, n);
+}
+
 }  // namespace
 
 extern "C" int minf_topk_indices(const float *scores, int rows, int n, int64_t row_stride, int k,
@@ -134,7 +202,7 @@ extern "C" int minf_topk_indices(const float *scores, int rows, int n, int64_t r
     if (row_stride < n || out_stride < (k < n ? k : n)) return MINF_ERR_INVALID_ARG;
     if (rows == 0) return MINF_OK;
     TopkProblem p{scores, (long long)row_stride, k, out, (long long)out_stride, reverse_base};
-    hipLaunchKernelGGL(topk_kernel, dim3((unsigned)rows, 1), dim3(TK_THREADS), 0, (hipStream_t)stream, p, p, n);
+    launch_topk(p, p, 1, rows, n, (hipStream_t)stream);
     return minf_launch_status();
 }
 
@@ -149,6 +217,6 @@ extern "C" int minf_topk_indices_pair(const float *scores_a, int k_a, int32_t *o
     if (rows == 0) return MINF_OK;
     TopkProblem pa{scores_a, (long long)row_stride, k_a, out_a, (long long)out_stride_a, reverse_base_a};
     TopkProblem pb{scores_b, (long long)row_stride, k_b, out_b, (long long)out_stride_b, reverse_base_b};
-    hipLaunchKernelGGL(topk_kernel, dim3((unsigned)rows, 2), dim3(TK_THREADS), 0, (hipStream_t)stream, pa, pb, n);
+    launch_topk(pa, pb, 2, rows, n, (hipStream_t)stream);
     return minf_launch_status();
 }

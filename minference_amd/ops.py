@@ -12,7 +12,7 @@ result is a new tensor of the query's shape and dtype.  In addition to the
 reference, K/V may have fewer heads than Q (grouped-query attention) and are
 then read in place instead of being expanded.  All arithmetic runs in
 libminf_hip.so on the caller's current stream; torch is only used for memory,
-the index sort and (for the block-sparse index) nothing else.
+and the index sort of the vertical-slash wrapper.
 """
 from __future__ import annotations
 
@@ -50,7 +50,7 @@ class _Call:
     """Holds the (possibly cast/padded) tensors of one operator call and the
     filled ``minf_qkvo`` struct."""
 
-    def __init__(self, q, k, v, seqlens=None):
+    def __init__(self, q, k, v, seqlens=None, need_out=True):
         _check_qkv(q, k, v)
         self.out_dtype = q.dtype
         self.head_dim = q.shape[-1]
@@ -71,7 +71,8 @@ class _Call:
         self.q, self.k, self.v = _prep(q), _prep(k), _prep(v)
         B, H, N, _ = self.q.shape
         self.B, self.H, self.N, self.Hk = B, H, N, self.k.shape[1]
-        self.o = torch.empty((B, H, N, _SUPPORTED_D), dtype=self.q.dtype, device=q.device)
+        self.o = torch.empty((B, H, N, _SUPPORTED_D) if need_out else (1, 1, 1, _SUPPORTED_D),
+                             dtype=self.q.dtype, device=q.device)
         s = _lib.QKVO()
         s.q, s.k, s.v, s.o = self.q.data_ptr(), self.k.data_ptr(), self.v.data_ptr(), self.o.data_ptr()
         for name, t in (("q_stride", self.q), ("k_stride", self.k), ("v_stride", self.v), ("o_stride", self.o)):
@@ -156,27 +157,29 @@ def block_sparse_attention_from_index(query, key, value, block_index):
 
 def _build_block_index(query, key, top_k, block_size_M=64, block_size_N=64, force_diag_first=False):
     """Top-k key blocks per query block from mean-pooled Q/K
-    (block_sparse_flash_attention.py:151-166).  Pooling, scores and the top-k run in torch for
-    now (fp32); K/V heads are expanded only at pooled (1/64) size."""
-    B, H, N, D = query.shape
-    Hk = key.shape[1]
-    pad = block_size_M - (N & (block_size_M - 1))          # reference :178 (a full block if N%64==0)
-    def pool(x):
-        x = torch.nn.functional.pad(x.float(), [0, 0, 0, pad])
-        return x.reshape(x.shape[0], x.shape[1], -1, block_size_M, D).mean(dim=-2)
-    qp, kp = pool(query), pool(key)
-    if Hk != H:
-        kp = kp.repeat_interleave(H // Hk, dim=1)
-    R = qp.shape[2]
-    p = torch.einsum("bhmk,bhnk->bhmn", qp, kp)
-    ar = torch.arange(R, device=query.device)
-    p = p.masked_fill(ar[:, None] < ar[None, :], float("-inf"))
-    if force_diag_first:
-        p[..., ar, ar] = float("inf")
-        p[..., :, 0] = float("inf")
-    top_k = min(top_k, R)
-    order = torch.argsort(p, dim=-1, descending=True, stable=True)[..., :top_k]
-    return order.to(torch.int32).sort(dim=-1).values.contiguous()
+    (block_sparse_flash_attention.py:151-166, including the zero padding its caller applies at
+    :178-180).  Pooling, block scores (fp32 matrix cores) and the top-k all run in libminf_hip.so;
+    K may have fewer heads than Q.  Returns int32 [batch, heads_q, rows, min(top_k, rows)] with
+    rows = (n + 64 - n % 64) / 64, every row ascending."""
+    if block_size_M != 64 or block_size_N != 64:
+        raise ValueError("only 64x64 blocks are supported")
+    c = _Call(query, key, key, need_out=False)           # casts / pads head_dim exactly like the attention call
+    lib = _lib.load()
+    rows = lib.minf_bs_block_index_rows(c.N)
+    kk = min(int(top_k), rows)
+    if kk <= 0:
+        raise ValueError("top_k must be positive")
+    ws_bytes = lib.minf_bs_block_index_workspace_bytes(c.B, c.H, c.Hk, c.N)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=c.q.device)
+    out = torch.empty((c.B, c.H, rows, kk), dtype=torch.int32, device=c.q.device)
+    qs = (ctypes.c_int64 * 3)(*c.q.stride()[:3])
+    ks = (ctypes.c_int64 * 3)(*c.k.stride()[:3])
+    with torch.cuda.device(c.q.device):
+        st = lib.minf_bs_block_index(c.q.data_ptr(), c.k.data_ptr(), qs, ks, c.B, c.H, c.Hk, c.N,
+                                     _SUPPORTED_D, c.struct.dtype, int(top_k), int(bool(force_diag_first)),
+                                     out.data_ptr(), ws.data_ptr(), ws_bytes, _lib.stream_ptr(c.q.device))
+    _lib.check(st, "minf_bs_block_index")
+    return out
 
 
 def block_sparse_attention(query, key, value, top_k: int, block_size_M: int = 64, block_size_N: int = 64):

@@ -160,3 +160,81 @@ def test_golden_fixtures(gpu):
                                             torch.from_numpy(z["slash"]).to(gpu)), torch.from_numpy(z["vs_out"]), "golden-vs")
     check(M.streaming_forward(q, k, v, 8, 48), torch.from_numpy(z["ashape_out"]), "golden-ashape")
     check(M.block_sparse_attention(q, k, v, 2), torch.from_numpy(z["bs_out"]), "golden-bs")
+
+
+def _check_block_index(bi_gpu, p, top_k):
+    """bi_gpu [H, R, K] against oracle block scores p [H, R, R] (fp32): ascending unique rows, and
+    the same selection as the oracle's rule up to near-ties of the fp32 scores (the GPU sums in a
+    different order): everything clearly above the k-th score is selected, nothing clearly below."""
+    H, R, K = bi_gpu.shape
+    assert K == min(top_k, R)
+    exact = 0
+    order = np.argsort(-p, axis=-1, kind="stable")[..., :K]
+    want = np.sort(order, axis=-1)
+    for h in range(H):
+        for m in range(R):
+            row = bi_gpu[h, m]
+            assert (np.diff(row) > 0).all(), (h, m)
+            assert row.min() >= 0 and row.max() < R
+            if (row == want[h, m]).all():
+                exact += 1
+                continue
+            kth = p[h, m, order[h, m, K - 1]]
+            tol = 1e-5 * max(1.0, abs(kth)) if np.isfinite(kth) else 0.0
+            sel = np.zeros(R, bool); sel[row] = True
+            if np.isfinite(kth):
+                assert sel[p[h, m] > kth + tol].all(), (h, m)
+                assert (p[h, m][sel] >= kth - tol).all(), (h, m)
+            else:                                   # fewer finite scores than k: all finite ones are in
+                assert sel[np.isfinite(p[h, m]) | (p[h, m] == np.inf)].all(), (h, m)
+    assert exact >= 0.98 * H * R, f"only {exact}/{H * R} rows identical to the oracle"
+
+
+def _oracle_block_scores(q, k, hq, force):
+    n = q.shape[2]
+    pad = 64 - (n & 63)
+    qp = torch.nn.functional.pad(q, [0, 0, 0, pad]).float().reshape(1, hq, -1, 64, q.shape[-1]).mean(-2)
+    kp = torch.nn.functional.pad(expand(k, hq), [0, 0, 0, pad]).float().reshape(1, hq, -1, 64, q.shape[-1]).mean(-2)
+    p = torch.einsum("bhmk,bhnk->bhmn", qp, kp)[0].numpy().copy()
+    R = p.shape[-1]
+    ar = np.arange(R)
+    p[:, ar[:, None] < ar[None, :]] = -np.inf
+    if force:
+        p[:, ar, ar] = np.inf
+        p[:, :, 0] = np.inf
+    return p
+
+
+@pytest.mark.parametrize("n,top_k,hq,hk,force,dtype", [
+    (1024, 4, 2, 2, False, torch.bfloat16), (2000, 8, 4, 2, False, torch.bfloat16),
+    (640, 100, 1, 1, False, torch.float16), (4160, 16, 8, 2, True, torch.bfloat16),
+    (63, 3, 2, 1, False, torch.bfloat16), (8192, 100, 2, 1, True, torch.bfloat16)])
+def test_block_index_kernel_vs_oracle(gpu, n, top_k, hq, hk, force, dtype):
+    from minference_amd.ops import _build_block_index
+    print(f"case block-index n={n} top_k={top_k} hq={hq} hk={hk} force={force}", flush=True)
+    q, k, _ = make(1, hq, hk, n, 40, dtype)
+    bi = _build_block_index(q.to(gpu), k.to(gpu), top_k, force_diag_first=force)
+    R = (n + 64 - (n & 63)) // 64
+    assert tuple(bi.shape) == (1, hq, R, min(top_k, R)) and bi.dtype == torch.int32
+    p = _oracle_block_scores(q, k, hq, force)
+    _check_block_index(bi[0].cpu().numpy(), p, top_k)
+    # and the oracle's own index builder agrees with the score matrix used above
+    pad = 64 - (n & 63)
+    ob = O.bs_block_index(torch.nn.functional.pad(q, [0, 0, 0, pad]),
+                          torch.nn.functional.pad(expand(k, hq), [0, 0, 0, pad]), top_k, force_diag_first=force)
+    _check_block_index(ob[0].numpy(), p, top_k)
+
+
+def test_block_sparse_config4_shape_scaled(gpu):
+    # BASELINE config 4 scaled to 8192 tokens: top-100 key blocks incl. diagonal and block 0, GQA
+    from minference_amd.ops import _build_block_index, block_sparse_attention_from_index
+    n, hq, hk = 8192, 4, 1
+    q, k, v = make(1, hq, hk, n, 41, torch.bfloat16)
+    bi = _build_block_index(q.to(gpu), k.to(gpu), 100, force_diag_first=True)
+    out = block_sparse_attention_from_index(q.to(gpu), k.to(gpu), v.to(gpu), bi)
+    bic = bi.cpu().numpy()
+    assert (bic[0, :, :, 0] == 0).all()
+    for m in range(n // 64):
+        assert (bic[0, :, m, : min(m + 1, 100)] == m).any(axis=-1).all()
+    ref = torch.stack([O.masked_attention(q[0, h], k[0, 0], v[0, 0], O.bs_mask(bic[0, h], n)) for h in range(hq)])[None]
+    check(out, ref, "bs-c4")

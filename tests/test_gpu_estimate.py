@@ -41,7 +41,8 @@ def test_forcing(gpu):
     assert torch.isinf(slash[..., -100:]).all() and torch.isfinite(slash[..., :-100]).all()
 
 
-@pytest.mark.parametrize("n,k", [(1000, 10), (5000, 1000), (131072, 6096), (70001, 1000), (300, 300), (64, 100)])
+@pytest.mark.parametrize("n,k", [(1000, 10), (5000, 1000), (131072, 6096), (70001, 1000), (300, 300), (64, 100),
+                                 (200, 7), (256, 255), (2049, 100), (4096, 4000), (4097, 100), (65, 1)])
 def test_topk_exact_vs_oracle(gpu, n, k):
     from minference_amd.estimate import topk_indices
     g = torch.Generator().manual_seed(n + k)
@@ -49,6 +50,7 @@ def test_topk_exact_vs_oracle(gpu, n, k):
     x[0, : min(30, n)] = torch.inf
     x[1, -min(100, n):] = torch.inf
     x[2] = (x[2] * 50).floor() / 50             # many ties
+    x[2, n // 2:] = -torch.inf                   # masked tail, as in block-causal score rows
     got = topk_indices(x.to(gpu), k).cpu()
     ref = O.topk_lowest_index(x, min(k, n)).to(torch.int32)
     assert torch.equal(got, ref)
