@@ -213,6 +213,25 @@ def vs_mask(block_count, block_offset, column_count, column_index, n, seqlen=Non
     return mask
 
 
+def vs_mask_rows(block_count_m, block_offset_m, column_count_m, column_index_m, m, n, seqlen=None):
+    """Rows [64m, min(64m+64, n)) of vs_mask() from the index entries of row block m alone
+    (pit_sparse_flash_attention_v2.py:104-148): [rows, n] bool.  For full-size inputs where the
+    [n, n] mask does not fit."""
+    seqlen = n if seqlen is None else seqlen
+    r0, r1 = m * 64, min(m * 64 + 64, n)
+    mask = np.zeros((r1 - r0, n), dtype=bool)
+    if r0 >= seqlen:
+        return mask
+    rr = np.arange(r0, r1)
+    for off in np.asarray(block_offset_m, dtype=np.int64)[: int(block_count_m)]:
+        cols = np.arange(off, off + 64)
+        cols = cols[(cols < seqlen) & (cols < n)]
+        mask[:, cols] |= cols[None, :] <= rr[:, None]
+    mask[:, np.asarray(column_index_m, dtype=np.int64)[: int(column_count_m)]] = True
+    mask[rr >= seqlen, :] = False
+    return mask
+
+
 def bs_block_index(q: torch.Tensor, k: torch.Tensor, top_k: int, force_diag_first: bool = False):
     """block_sparse_flash_attention.py:151-166 on tensors already padded to a
     multiple of 64 (the caller pads, :178-180).  fp32 arithmetic; ties -> lowest

@@ -1,4 +1,5 @@
 """GPU tests of the per-head dispatcher and the fused vertical-slash layer path."""
+import numpy as np
 import pytest
 import torch
 
@@ -57,3 +58,104 @@ def test_config1_shape_fp32_full(gpu):
     ref = O.vertical_slash_sparse_attention(q[:, :1], k[:, :1], v[:, :1], v_idx[:, :1].cpu(), s_idx[:, :1].cpu())
     err = (out[:, :1] - ref).abs()
     assert err.max() <= 2e-2 and err.mean() <= 1e-3
+
+
+def test_config2_full_size_sampled_row_blocks(gpu):
+    """BASELINE config 2 at full length (131072 tokens, GQA 4:1, bf16, vertical 1000, slash 6096,
+    planted structure; 4 query heads to keep the host work small) with a ragged tail (n % 64 != 0):
+    the whole GPU path (estimate -> top-k -> index -> attention), then for sampled (head, row block)
+    pairs, incl. the first, the last partial one and the forced-diagonal region, the fp32
+    masked-dense oracle on the index entries the GPU produced."""
+    import minference_amd as M
+    n, hq, hk = 131072 - 37, 4, 1
+    q, k, v, _ = gen.planted_layer(n, hq, hk, seed=100, dtype=torch.bfloat16)
+    qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
+    v_idx, s_idx = M.estimate_vertical_slash(qg, kg, 1000, 6096)
+    seqlens = torch.full((1,), n, dtype=torch.int32, device=gpu)
+    bc, bo, cc, ci = M.convert_vertical_slash_indexes(seqlens, v_idx, s_idx, n, 64, 64)
+    out = M.vertical_slash_attention_from_index(qg, kg, vg, bc, bo, cc, ci, seqlens)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all()
+    # the index rows the GPU built are the reference algorithm's rows (C restatement, bit-exact)
+    rows = (n + 63) // 64
+    vi_c, si_c = v_idx.cpu().numpy(), s_idx.cpu().numpy()
+    for h, m in [(0, 0), (1, 1), (2, 777), (3, rows - 1), (0, rows - 2), (1, 1024)]:
+        print(f"case c2-full head={h} row-block={m}", flush=True)
+        rbo, rci = O.vs_index_row_py(vi_c[0, h].tolist(), si_c[0, h].tolist(), m, n)
+        rbc, rcc = len(rbo), len(rci)
+        assert int(bc[0, h, m]) == rbc and int(cc[0, h, m]) == rcc
+        assert bo[0, h, m, :rbc].cpu().tolist() == rbo and ci[0, h, m, :rcc].cpu().tolist() == rci
+        mask = O.vs_mask_rows(rbc, rbo, rcc, rci, m, n)
+        r0, r1 = m * 64, min(m * 64 + 64, n)
+        s = (q[0, h, r0:r1].float() @ k[0, 0].float().T) * (128 ** -0.5)
+        s = torch.where(torch.as_tensor(mask), s, torch.tensor(-torch.inf))
+        ref = torch.softmax(s, dim=-1) @ v[0, 0].float()
+        err = (out[0, h, r0:r1].float().cpu() - ref).abs()
+        print(f"  max-abs {err.max().item():.3e} mean-abs {err.mean().item():.3e}", flush=True)
+        assert err.max() <= 2e-2 and err.mean() <= 1e-3
+
+
+def _rows_reference(q_rows, k, v, mask):
+    s = (q_rows.float() @ k.float().T) * (q_rows.shape[-1] ** -0.5)
+    s = torch.where(torch.as_tensor(mask), s, torch.tensor(-torch.inf))
+    return torch.softmax(s, dim=-1) @ v.float()
+
+
+def test_config4_full_size_sampled_row_blocks(gpu):
+    """BASELINE config 4 at full length (131072 tokens, top-100 key blocks incl. diagonal and block
+    0, GQA, bf16; 2 query heads): block index from the HIP kernels checked against fp32 pooled
+    scores for sampled query blocks, attention checked on the same row blocks."""
+    from minference_amd.ops import _build_block_index, block_sparse_attention_from_index
+    n, hq, hk, top_k = 131072, 2, 1, 100
+    q, k, v, _ = gen.planted_layer(n, hq, hk, seed=101, dtype=torch.bfloat16)
+    qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
+    bi = _build_block_index(qg, kg, top_k, force_diag_first=True)
+    out = block_sparse_attention_from_index(qg, kg, vg, bi)
+    torch.cuda.synchronize()
+    R = n // 64 + 1
+    assert tuple(bi.shape) == (1, hq, R, top_k)
+    kp = torch.nn.functional.pad(k[0, 0].float(), [0, 0, 0, 64]).reshape(R, 64, 128).mean(1)
+    bic = bi[0].cpu().numpy()
+    for h, m in [(0, 0), (1, 5), (0, 99), (1, 100), (0, 1500), (1, 2047)]:
+        print(f"case c4-full head={h} query-block={m}", flush=True)
+        row = bic[h, m]
+        assert (np.diff(row) > 0).all()
+        p = (q[0, h, m * 64: m * 64 + 64].float().mean(0) @ kp.T).numpy()
+        p[m + 1:] = -np.inf
+        p[m] = p[0] = np.inf
+        kth = np.sort(p)[::-1][top_k - 1]
+        sel = np.zeros(R, bool); sel[row] = True
+        if np.isfinite(kth):
+            tol = 1e-5 * max(1.0, abs(kth))
+            assert sel[p > kth + tol].all() and (p[sel] >= kth - tol).all()
+        else:
+            assert sel[: m + 1].all()
+        mask = np.zeros((64, n), bool)
+        rr = np.arange(m * 64, m * 64 + 64)
+        for j in row[: min(m + 1, top_k)]:
+            cols = np.arange(j * 64, min(j * 64 + 64, n))
+            mask[:, cols] |= cols[None, :] <= rr[:, None]
+        err = (out[0, h, m * 64: m * 64 + 64].float().cpu() - _rows_reference(q[0, h, m * 64: m * 64 + 64], k[0, 0], v[0, 0], mask)).abs()
+        print(f"  max-abs {err.max().item():.3e} mean-abs {err.mean().item():.3e}", flush=True)
+        assert err.max() <= 2e-2 and err.mean() <= 1e-3
+
+
+def test_config5_ashape_heads_full_size_sampled_row_blocks(gpu):
+    """BASELINE config 5's A-shape heads at full length (262144 tokens, sink 128 + local 4096, GQA,
+    bf16; 2 query heads), sampled row blocks against the closed-form mask
+    {k : r - n_local < k <= r} U {k < n_init : k <= r - n_local}."""
+    import minference_amd as M
+    n, hq, hk, n_init, n_local = 262144 - 5, 2, 1, 128, 4096
+    q, k, v = gen.qkv(1, hq, hk, n, 128, seed=55, dtype=torch.bfloat16, scale=1.0)
+    out = M.streaming_forward(q.to(gpu), k.to(gpu), v.to(gpu), n_init, n_local)
+    torch.cuda.synchronize()
+    rows = (n + 63) // 64
+    for h, m in [(0, 0), (1, 1), (0, 63), (1, 64), (0, 65), (1, 2000), (0, rows - 1)]:
+        print(f"case c5-ashape head={h} row-block={m}", flush=True)
+        r0, r1 = m * 64, min(m * 64 + 64, n)
+        r = np.arange(r0, r1)[:, None]
+        c = np.arange(n)[None, :]
+        mask = ((c <= r) & (c > r - n_local)) | ((c < n_init) & (c <= r - n_local))
+        err = (out[0, h, r0:r1].float().cpu() - _rows_reference(q[0, h, r0:r1], k[0, 0], v[0, 0], mask)).abs()
+        print(f"  max-abs {err.max().item():.3e} mean-abs {err.mean().item():.3e}", flush=True)
+        assert err.max() <= 2e-2 and err.mean() <= 1e-3

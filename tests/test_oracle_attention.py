@@ -48,6 +48,16 @@ def test_vs_mask_matches_definition_bruteforce():
                 assert m[rr, cc_], (rr, cc_)
 
 
+def test_vs_mask_rows_is_a_slice_of_vs_mask():
+    for n, seqlen in ((1000, None), (777, 700)):
+        vi, si = gen.vs_index_inputs(1, n, 20, 40, seed=3, force_v=2, force_s=3)
+        bc, bo, cc, ci = O.vs_index_build([seqlen or n], vi, si, n)
+        full = O.vs_mask(bc[0, 0], bo[0, 0], cc[0, 0], ci[0, 0], n, seqlen)
+        for m in range((n + 63) // 64):
+            part = O.vs_mask_rows(bc[0, 0, m], bo[0, 0, m], cc[0, 0, m], ci[0, 0, m], m, n, seqlen)
+            assert np.array_equal(part, full[m * 64: m * 64 + 64])
+
+
 def test_block_sparse_index_properties_and_dense_limit():
     n = 640
     q, k, v = gen.qkv(1, 2, 2, n, 16, seed=3, scale=1.0)
