@@ -108,7 +108,7 @@ __device__ __forceinline__ void load_k(const EstParams &p, const char *kb, int c
 
 // ---------------------------------------------------------------- stats sweep
 template <typename T>
-__global__ __launch_bounds__(EST_THREADS) void est_stats_kernel(const EstParams p) {
+__global__ __launch_bounds__(EST_THREADS, 3) void est_stats_kernel(const EstParams p) {
     __shared__ float lds_m[4][LQ], lds_l[4][LQ];
     const WgId w = decode_wg(p);
     if (!w.valid) return;
@@ -219,8 +219,10 @@ __global__ __launch_bounds__(LQ) void est_reduce_kernel(const EstParams p) {
 constexpr int TP = 33;                       // tile row pitch (floats)
 constexpr int WWIN = KC / 4 + LQ;            // per-wave diagonal window (256 keys + 64)
 
+// (min 2 waves per SIMD: caps the kernel at 256 registers; it is latency bound and one resident
+// wave per SIMD ran 1.4x slower)
 template <typename T>
-__global__ __launch_bounds__(EST_THREADS) void est_scores_kernel(const EstParams p) {
+__global__ __launch_bounds__(EST_THREADS, 2) void est_scores_kernel(const EstParams p) {
     __shared__ float lds_tile[4][LQ * TP];
     __shared__ float lds_wwin[4][WWIN];
     const WgId w = decode_wg(p);

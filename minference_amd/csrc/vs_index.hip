@@ -176,6 +176,295 @@ __global__ __launch_bounds__(IDX_WAVES *MINF_WAVE) void vs_index_kernel(
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Translation-invariant fast path.
+//
+// For an entry that is neither skipped (o >= end_m) nor clipped (end_m - o < 64), t = end_m - o,
+// so the whole range logic depends on the row block only through a shift: once a range STARTS at
+// list entry g, everything the reference does from g on (ranges, blocks) is the same for every row
+// block, moved by end_m.  vs_index_prep_kernel therefore walks each head's slash list ONCE, as a
+// virtual row whose end is V = slash[0] + 64 (nothing skipped, nothing clipped), and tabulates
+//   cpos[k]   start of the k-th block,                     k < nblocks
+//   cpre[i]   index of the first block of the range that starts at entry i, else -1
+//   crun[i]   ordinal of that range, else -1
+//   run_a[r], run_e[r]   [start, end) of range r
+// all in the virtual row's coordinates (real position = virtual + end_m - V).
+// vs_index_fast_kernel then handles a row block as follows: entries from the first valid one are
+// processed exactly like vs_index_kernel until a range starts at an entry that also starts a range
+// of the table (at once when no entry is skipped or clipped; after a few entries otherwise: chains
+// that start at different entries meet at the first gap both see); from there the remaining blocks
+// are copied from cpos with a shift (coalesced), and each remaining vertical x is emitted iff it is
+// not inside one of the remaining tabulated ranges, is not below the end of the last range of the
+// explicit part, and is below the last entry's t - the reference's merge rule restated per element.
+#define IDX_TAB_HDR 4
+__device__ __forceinline__ long long idx_tab_ints(int nnz_s) { return IDX_TAB_HDR + 5ll * nnz_s; }
+
+__global__ __launch_bounds__(MINF_WAVE) void vs_index_prep_kernel(const int32_t *__restrict__ slash,
+                                                                  int32_t *__restrict__ tables, int nnz_s) {
+    const int lane = minf_lane();
+    const long long bh = blockIdx.x;
+    const int32_t *sl = slash + bh * (long long)nnz_s;
+    int32_t *hdr = tables + bh * idx_tab_ints(nnz_s);
+    int32_t *cpos = hdr + IDX_TAB_HDR, *cpre = cpos + nnz_s, *crun = cpre + nnz_s;
+    int32_t *run_a = crun + nnz_s, *run_e = run_a + nnz_s;
+    const int V = sl[0] + 64;
+
+    int nb = 0, nr = 0;
+    int carried_e = 0, carried_t = 0, cur_a = 0;
+    const int nchunks = (nnz_s + MINF_WAVE - 1) / MINF_WAVE;
+    for (int c = 0; c < nchunks; ++c) {
+        const int base = c * MINF_WAVE;
+        const int cnt = min(MINF_WAVE, nnz_s - base);
+        const bool valid = lane < cnt;
+        int t = valid ? max(V - sl[base + lane], 64) : 0;
+        const int tlast = minf_readlane(t, cnt - 1);
+        if (!valid) t = tlast;
+        if (c == 0) {
+            const int t0 = minf_readlane(t, 0);
+            cur_a = t0 - 64;
+            carried_e = t0 - 64;
+            carried_t = t0;
+        }
+        int a = cur_a;
+        int tprev = __shfl_up(t, 1);
+        if (lane == 0) tprev = carried_t;
+        int start = 0;
+        bool is_start = (c == 0 && lane == 0);
+        for (;;) {
+            int eprev = a + ((((tprev - a) + 63) >> 6) << 6);
+            if (lane == 0) eprev = carried_e;
+            const bool brk = (lane >= start) && (t > eprev + 64);
+            const uint64_t bm = __ballot(brk);
+            if (bm == 0) break;
+            const int j = __builtin_ctzll(bm);
+            const int tj = minf_readlane(t, j);
+            if (lane >= j) a = tj - 64;
+            if (lane == j) is_start = true;
+            start = j + 1;
+        }
+        is_start = is_start && valid;
+        const int e = a + ((((t - a) + 63) >> 6) << 6);
+        int eprev = __shfl_up(e, 1);
+        if (lane == 0) eprev = carried_e;
+        const bool changed = valid && (e != eprev);
+        const uint64_t cm = __ballot(changed), sm = __ballot(is_start);
+        const uint64_t lt = minf_lanemask_lt();
+        const int kpos = nb + __builtin_popcountll(cm & lt);
+        if (changed) cpos[kpos] = e - 64;
+        if (valid) {
+            const int r = nr + __builtin_popcountll(sm & lt);
+            cpre[base + lane] = is_start ? kpos : -1;
+            crun[base + lane] = is_start ? r : -1;
+            if (is_start) {
+                run_a[r] = a;
+                if (r > 0) run_e[r - 1] = eprev;
+            }
+        }
+        nb += __builtin_popcountll(cm);
+        nr += __builtin_popcountll(sm);
+        carried_e = minf_readlane(e, cnt - 1);
+        carried_t = tlast;
+        cur_a = minf_readlane(a, cnt - 1);
+    }
+    if (lane == 0) {
+        run_e[nr - 1] = carried_e;
+        hdr[0] = nb;
+        hdr[1] = nr;
+        hdr[2] = V;
+        hdr[3] = 0;
+    }
+}
+
+__global__ __launch_bounds__(IDX_WAVES *MINF_WAVE) void vs_index_fast_kernel(
+    const int32_t *__restrict__ seqlens, const int32_t *__restrict__ vertical,
+    const int32_t *__restrict__ slash, const int32_t *__restrict__ tables,
+    int32_t *__restrict__ block_count, int32_t *__restrict__ block_offset,
+    int32_t *__restrict__ column_count, int32_t *__restrict__ column_index, int heads, int rows,
+    int nnz_v, int nnz_s, int zero_fill, int32_t *error_flag, long long total_rows) {
+    __shared__ int lds_t[IDX_WAVES][MINF_WAVE];
+    __shared__ int lds_a[IDX_WAVES][MINF_WAVE];
+    __shared__ int lds_e[IDX_WAVES][MINF_WAVE];
+
+    const int lane = minf_lane();
+    const int wave = (int)(threadIdx.x >> 6);
+    const long long ro = (long long)blockIdx.x * IDX_WAVES + wave;   // (b*H + h)*rows + m
+    if (ro >= total_rows) return;
+    const int m = (int)(ro % rows);
+    const long long bh = ro / rows;
+    const int b = (int)(bh / heads);
+
+    int32_t *bo_row = block_offset + ro * (long long)nnz_s;
+    int32_t *ci_row = column_index + ro * (long long)nnz_v;
+    const int32_t *vert = vertical + bh * (long long)nnz_v;
+    const int32_t *sl = slash + bh * (long long)nnz_s;
+    const int32_t *hdr = tables + bh * idx_tab_ints(nnz_s);
+    const int32_t *cpos = hdr + IDX_TAB_HDR, *cpre = cpos + nnz_s, *crun = cpre + nnz_s;
+    const int32_t *run_a = crun + nnz_s, *run_e = run_a + nnz_s;
+
+    const int seqlen = seqlens[b];
+    const int start_m = m * 64;
+    const int end_m = start_m + 64;
+    const uint64_t lt = minf_lanemask_lt();
+
+    int nb = 0, ncol = 0;
+    bool live = start_m < seqlen;
+
+    int s0 = nnz_s;
+    if (live) {
+        int lo = 0, hi = nnz_s;
+        while (lo < hi) {
+            int mid = (lo + hi) >> 1;
+            if (sl[mid] >= end_m) lo = mid + 1; else hi = mid;
+        }
+        s0 = lo;
+        if (s0 >= nnz_s) {           // the reference would read past the list here
+            live = false;
+            if (error_flag && lane == 0) *error_flag = 1;
+        }
+    }
+
+    if (live) {
+        int vp = 0;
+        int g = -1;                  // list entry from which the tables apply
+        int e_lim = INT_MIN;         // end of the last explicitly built range
+        if (s0 == 0 && end_m - sl[0] >= 64) {
+            g = 0;
+        } else {
+            const int n = nnz_s - s0;
+            const int nchunks = (n + MINF_WAVE - 1) / MINF_WAVE;
+            int carried_e = 0, carried_t = 0, cur_a = 0;
+            int ep0 = INT_MIN;
+            for (int c = 0; c < nchunks; ++c) {
+                const int base = s0 + c * MINF_WAVE;
+                int cnt = min(MINF_WAVE, nnz_s - base);
+                bool valid = lane < cnt;
+                int t = valid ? max(end_m - sl[base + lane], 64) : 0;
+                int tlast = minf_readlane(t, cnt - 1);
+                if (!valid) t = tlast;
+                if (c == 0) {
+                    const int t0 = minf_readlane(t, 0);
+                    cur_a = t0 - 64;
+                    carried_e = t0 - 64;
+                    carried_t = t0;
+                }
+                int a = cur_a;
+                int tprev = __shfl_up(t, 1);
+                if (lane == 0) tprev = carried_t;
+                int start = 0, cut = -1;
+                for (;;) {
+                    int eprev = a + ((((tprev - a) + 63) >> 6) << 6);
+                    if (lane == 0) eprev = carried_e;
+                    const bool brk = (lane >= start) && (t > eprev + 64);
+                    const uint64_t bm = __ballot(brk);
+                    if (bm == 0) break;
+                    const int j = __builtin_ctzll(bm);
+                    if (cpre[base + j] >= 0) { cut = j; break; }      // a tabulated range starts here
+                    const int tj = minf_readlane(t, j);
+                    if (lane >= j) a = tj - 64;
+                    start = j + 1;
+                }
+                if (cut == 0) {          // nothing of this chunk belongs to the explicit part
+                    g = base;
+                    e_lim = carried_e;
+                    break;
+                }
+                if (cut > 0) {           // entries [0, cut) only; later lanes repeat entry cut-1
+                    cnt = cut;
+                    valid = lane < cnt;
+                    tlast = minf_readlane(t, cnt - 1);
+                    const int alast = minf_readlane(a, cnt - 1);
+                    if (!valid) { t = tlast; a = alast; }
+                }
+                const int e = a + ((((t - a) + 63) >> 6) << 6);
+                int eprev = __shfl_up(e, 1);
+                if (lane == 0) eprev = carried_e;
+                const bool changed = valid && (e != eprev);
+                const uint64_t cm = __ballot(changed);
+                if (changed) bo_row[nb + __builtin_popcountll(cm & lt)] = e - 64;
+                nb += __builtin_popcountll(cm);
+
+                if (vp < nnz_v && vert[vp] < tlast) {
+                    lds_t[wave][lane] = t;
+                    lds_a[wave][lane] = a;
+                    lds_e[wave][lane] = e;
+                    __builtin_amdgcn_wave_barrier();
+                    while (vp < nnz_v) {
+                        const int x = (vp + lane < nnz_v) ? vert[vp + lane] : INT_MAX;
+                        const bool ok = x < tlast;
+                        const uint64_t okm = __ballot(ok);
+                        const int k = __builtin_popcountll(okm);
+                        bool emit = false;
+                        if (ok) {
+                            int lo = 0, hi = MINF_WAVE - 1;      // first i with t[i] > x (exists)
+                            while (lo < hi) {
+                                int mid = (lo + hi) >> 1;
+                                if (lds_t[wave][mid] > x) hi = mid; else lo = mid + 1;
+                            }
+                            const int ai = lds_a[wave][lo];
+                            const int ep = lo == 0 ? ep0 : lds_e[wave][lo - 1];
+                            emit = (x < ai) && (x >= ep);
+                        }
+                        const uint64_t em = __ballot(emit);
+                        if (emit) ci_row[ncol + __builtin_popcountll(em & lt)] = x;
+                        ncol += __builtin_popcountll(em);
+                        vp += k;
+                        if (k < MINF_WAVE) break;
+                    }
+                    __builtin_amdgcn_wave_barrier();
+                }
+                carried_e = minf_readlane(e, cnt - 1);
+                carried_t = tlast;
+                cur_a = minf_readlane(a, cnt - 1);
+                ep0 = carried_e;
+                if (cut > 0) {
+                    g = base + cut;
+                    e_lim = carried_e;
+                    break;
+                }
+            }
+        }
+        if (g >= 0) {
+            const int shift = end_m - hdr[2];
+            const int k0 = cpre[g], r0 = crun[g];
+            const int nblk = hdr[0] - k0, nruns = hdr[1];
+            for (int k = lane; k < nblk; k += MINF_WAVE) bo_row[nb + k] = cpos[k0 + k] + shift;
+            nb += nblk;
+            const int t_end = end_m - sl[nnz_s - 1];      // t of the last entry (not clipped here)
+            while (vp < nnz_v) {
+                const int x = (vp + lane < nnz_v) ? vert[vp + lane] : INT_MAX;
+                const bool ok = x < t_end;
+                const int k = __builtin_popcountll(__ballot(ok));
+                bool emit = false;
+                if (ok && x >= e_lim) {
+                    const int xv = x - shift;
+                    int lo = r0, hi = nruns;                  // first range >= r0 that ends after xv
+                    while (lo < hi) {
+                        int mid = (lo + hi) >> 1;
+                        if (run_e[mid] > xv) hi = mid; else lo = mid + 1;
+                    }
+                    emit = !(lo < nruns && run_a[lo] <= xv);
+                }
+                const uint64_t em = __ballot(emit);
+                if (emit) ci_row[ncol + __builtin_popcountll(em & lt)] = x;
+                ncol += __builtin_popcountll(em);
+                vp += k;
+                if (k < MINF_WAVE) break;
+            }
+        }
+    }
+
+    if (zero_fill || live) {
+        if (lane == 0) {
+            block_count[ro] = nb;
+            column_count[ro] = ncol;
+        }
+    }
+    if (zero_fill) {
+        zero_range(bo_row, nb, nnz_s, lane);
+        zero_range(ci_row, ncol, nnz_v, lane);
+    }
+}
+
 extern "C" int minf_vs_index_build(const int32_t *seqlens, const int32_t *vertical_idx,
                                    const int32_t *slash_idx, int32_t *block_count,
                                    int32_t *block_offset, int32_t *column_count,
@@ -193,6 +482,40 @@ extern "C" int minf_vs_index_build(const int32_t *seqlens, const int32_t *vertic
     hipLaunchKernelGGL(vs_index_kernel, dim3((unsigned)nblk), dim3(IDX_WAVES * MINF_WAVE), 0,
                        (hipStream_t)stream, seqlens, vertical_idx, slash_idx, block_count,
                        block_offset, column_count, column_index, heads, rows, nnz_v, nnz_s,
+                       zero_fill, error_flag, total);
+    return minf_launch_status();
+}
+
+
+extern "C" size_t minf_vs_index_workspace_bytes(int batch, int heads, int nnz_s) {
+    if (batch <= 0 || heads <= 0 || nnz_s <= 0) return 0;
+    return (size_t)batch * heads * (IDX_TAB_HDR + 5 * (size_t)nnz_s) * sizeof(int32_t);
+}
+
+extern "C" int minf_vs_index_build_ws(const int32_t *seqlens, const int32_t *vertical_idx,
+                                      const int32_t *slash_idx, int32_t *block_count,
+                                      int32_t *block_offset, int32_t *column_count,
+                                      int32_t *column_index, int batch, int heads, int rows,
+                                      int nnz_v, int nnz_s, int zero_fill, int32_t *error_flag,
+                                      void *workspace, size_t workspace_bytes, void *stream) {
+    if (!seqlens || !vertical_idx || !slash_idx || !block_count || !block_offset ||
+        !column_count || !column_index)
+        return MINF_ERR_INVALID_ARG;
+    if (batch < 0 || heads < 0 || rows < 0 || nnz_v < 1 || nnz_s < 1) return MINF_ERR_INVALID_ARG;
+    const long long total = (long long)batch * heads * rows;
+    if (total == 0) return MINF_OK;
+    if (!workspace || workspace_bytes < minf_vs_index_workspace_bytes(batch, heads, nnz_s) ||
+        ((uintptr_t)workspace & 3))
+        return MINF_ERR_WORKSPACE;
+    const long long nblk = (total + IDX_WAVES - 1) / IDX_WAVES;
+    if (nblk > 0x7fffffffLL || (long long)batch * heads > 0x7fffffffLL) return MINF_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(vs_index_prep_kernel, dim3((unsigned)(batch * heads)), dim3(MINF_WAVE), 0,
+                       (hipStream_t)stream, slash_idx, (int32_t *)workspace, nnz_s);
+    int status = minf_launch_status();
+    if (status != MINF_OK) return status;
+    hipLaunchKernelGGL(vs_index_fast_kernel, dim3((unsigned)nblk), dim3(IDX_WAVES * MINF_WAVE), 0,
+                       (hipStream_t)stream, seqlens, vertical_idx, slash_idx, (const int32_t *)workspace,
+                       block_count, block_offset, column_count, column_index, heads, rows, nnz_v, nnz_s,
                        zero_fill, error_flag, total);
     return minf_launch_status();
 }

@@ -3,8 +3,10 @@
 Mirror of ``minference.cuda.convert_vertical_slash_indexes`` (reference
 csrc/kernels.cpp:7-18, csrc/vertical_slash_index.cu:127-167): same name,
 argument order and return order; outputs are int32 tensors on the inputs'
-device.  The work is done by ``minf_vs_index_build`` in libminf_hip.so on
-the caller's current stream (the reference used the legacy default stream).
+device.  The work is done by ``minf_vs_index_build_ws`` in libminf_hip.so (the
+table-driven builder; ``use_tables=False`` selects the plain wave-per-row
+``minf_vs_index_build``) on the caller's current stream (the reference used
+the legacy default stream).
 """
 from __future__ import annotations
 
@@ -21,7 +23,7 @@ def _i32_contig(t: torch.Tensor) -> torch.Tensor:
 
 def convert_vertical_slash_indexes(seqlens, vertical_indexes, slash_indexes, context_size,
                                    block_size_M=64, block_size_N=64, zero_fill=True,
-                                   error_flag=None):
+                                   error_flag=None, use_tables=True):
     """-> [block_count, block_offset, column_count, column_index].
 
     seqlens [B] int32, vertical_indexes [B,H,V] ascending, slash_indexes [B,H,S]
@@ -55,12 +57,16 @@ def convert_vertical_slash_indexes(seqlens, vertical_indexes, slash_indexes, con
         block_count.zero_()
         column_count.zero_()
     lib = _lib.load()
-    with torch.cuda.device(dev):
-        st = lib.minf_vs_index_build(
-            seqlens.data_ptr(), v.data_ptr(), s.data_ptr(), block_count.data_ptr(),
+    args = (seqlens.data_ptr(), v.data_ptr(), s.data_ptr(), block_count.data_ptr(),
             block_offset.data_ptr(), column_count.data_ptr(), column_index.data_ptr(),
             B, H, rows, V, S, 1 if zero_fill else 0,
-            error_flag.data_ptr() if error_flag is not None else None,
-            _lib.stream_ptr(dev))
+            error_flag.data_ptr() if error_flag is not None else None)
+    with torch.cuda.device(dev):
+        if use_tables:
+            ws_bytes = lib.minf_vs_index_workspace_bytes(B, H, S)
+            ws = torch.empty(max(ws_bytes, 4), dtype=torch.uint8, device=dev)
+            st = lib.minf_vs_index_build_ws(*args, ws.data_ptr(), ws_bytes, _lib.stream_ptr(dev))
+        else:
+            st = lib.minf_vs_index_build(*args, _lib.stream_ptr(dev))
     _lib.check(st, "minf_vs_index_build")
     return [block_count, block_offset, column_count, column_index]

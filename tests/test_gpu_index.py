@@ -11,12 +11,20 @@ pytestmark = pytest.mark.gpu
 
 
 def run_gpu(seqlens, v, s, n, dev, zero_fill=True):
+    """Table-driven builder (minf_vs_index_build_ws); with zero_fill the plain wave-per-row
+    builder (minf_vs_index_build) is run on the same inputs and must give the same tensors."""
     from minference_amd import convert_vertical_slash_indexes
-    out = convert_vertical_slash_indexes(
-        torch.tensor(seqlens, dtype=torch.int32, device=dev), torch.from_numpy(v).to(dev),
-        torch.from_numpy(np.ascontiguousarray(s)).to(dev), n, 64, 64, zero_fill=zero_fill)
+    args = (torch.tensor(seqlens, dtype=torch.int32, device=dev), torch.from_numpy(v).to(dev),
+            torch.from_numpy(np.ascontiguousarray(s)).to(dev), n, 64, 64)
+    out = convert_vertical_slash_indexes(*args, zero_fill=zero_fill)
     torch.cuda.synchronize()
-    return [o.cpu().numpy() for o in out]
+    out = [o.cpu().numpy() for o in out]
+    if zero_fill:
+        plain = convert_vertical_slash_indexes(*args, zero_fill=True, use_tables=False)
+        torch.cuda.synchronize()
+        for name, a, b in zip(["block_count", "block_offset", "column_count", "column_index"], out, plain):
+            assert np.array_equal(a, b.cpu().numpy()), f"table-driven and plain builders differ in {name}"
+    return out
 
 
 def assert_same(got, ref):
@@ -35,6 +43,37 @@ def test_random_lists(gpu, heads, n, nv, ns, seed):
     v, s = gen.vs_index_inputs(heads, n, nv, ns, seed=seed, force_v=min(4, nv), force_s=min(64, ns))
     ref = O.vs_index_build([n], v, s, n)
     assert_same(run_gpu([n], v, s, n, gpu), ref)
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2, 3])
+def test_structured_lists_all_rows(gpu, mode):
+    """Slash lists that stress the table-driven path: clusters with gaps just below / above the
+    64-token merge distance, duplicates, offsets up to n-1 (so most rows skip or clip entries and
+    join the tabulated ranges late), dense runs whose 64-phase depends on the first valid entry."""
+    rng = np.random.default_rng(100 + mode)
+    for trial in range(6):
+        n = int(rng.choice([1500, 4096, 9000, 20000]))
+        S = int(rng.integers(2, 400)); V = int(rng.integers(1, 200))
+        if mode == 0:
+            sl = np.sort(rng.choice(n, size=min(S, n), replace=False))[::-1]
+        elif mode == 1:
+            sl = np.unique(np.concatenate([np.arange(min(S, 300)), rng.integers(0, n, 7)]))[::-1]
+        elif mode == 2:
+            c = rng.integers(0, n, 6)
+            sl = np.sort(np.clip(np.concatenate([cc + rng.integers(-150, 150, S // 6 + 1) for cc in c]), 0, n - 1))[::-1]
+        else:
+            steps = rng.choice([1, 1, 2, 63, 64, 65, 127, 128, 129, 500], size=S)
+            sl = np.cumsum(steps); sl = sl[sl < n][::-1]
+            if sl.size == 0: sl = np.array([0])
+        vt = np.sort(rng.choice(n, size=min(V, n), replace=False))
+        if sl[-1] >= 64:
+            sl = np.concatenate([sl, [int(rng.integers(0, 64))]])   # every row block needs a valid entry
+        s = np.ascontiguousarray(sl[None, None].astype(np.int32))
+        v = np.ascontiguousarray(vt[None, None].astype(np.int32))
+        seqlen = n if trial % 3 else n - 77
+        print(f"case structured mode={mode} trial={trial} n={n} S={s.shape[-1]} V={v.shape[-1]} seqlen={seqlen}", flush=True)
+        ref = O.vs_index_build([seqlen], v, s, n)
+        assert_same(run_gpu([seqlen], v, s, n, gpu), ref)
 
 
 def test_hand_kat(gpu):
