@@ -45,7 +45,11 @@ __global__ __launch_bounds__(TK_THREADS) void topk_kernel(const TopkProblem p0, 
     int32_t *__restrict__ out = pr.out;
     const long long out_stride = pr.out_stride;
     const int reverse_base = pr.reverse_base;
-    __shared__ unsigned hist[256];
+    // 32 copies of the 256-bin histogram, copy = lane % 32 = LDS bank: score rows have few distinct
+    // exponents, so most lanes of a wave hit the same bin; with one copy per bank they neither
+    // serialise on one address nor conflict on a bank
+    __shared__ unsigned hist[256 * 32];
+    __shared__ unsigned bins[256];
     __shared__ unsigned sh_prefix, sh_need;
     __shared__ int wave_gt[TK_WAVES], wave_eq[TK_WAVES];
 
@@ -59,22 +63,35 @@ __global__ __launch_bounds__(TK_THREADS) void topk_kernel(const TopkProblem p0, 
     }
 
     // ---- 1. radix select --------------------------------------------------
+    const int nvec = (((uintptr_t)x & 15) == 0) ? (n >> 2) : 0;
     unsigned prefix = 0, mask = 0;
     unsigned need = (unsigned)k;     // rank (from the top) inside the current prefix bucket
     for (int shift = 24; shift >= 0; shift -= 8) {
-        if (tid < 256) hist[tid] = 0;
+        for (int i = tid; i < 256 * 32; i += TK_THREADS) hist[i] = 0;
         __syncthreads();
-        for (int i = tid; i < n; i += TK_THREADS) {
-            const unsigned u = order_key(x[i]);
-            if ((u & mask) == prefix) atomicAdd(&hist[(u >> shift) & 255u], 1u);
+        auto tally = [&](float xv) {
+            const unsigned u = order_key(xv);
+            if ((u & mask) == prefix) atomicAdd(&hist[(((u >> shift) & 255u) << 5) + (lane & 31)], 1u);
+        };
+        for (int i = tid; i < nvec; i += TK_THREADS) {       // 16-byte loads over the aligned part
+            const float4 q = reinterpret_cast<const float4 *>(x)[i];
+            tally(q.x); tally(q.y); tally(q.z); tally(q.w);
+        }
+        for (int i = nvec * 4 + tid; i < n; i += TK_THREADS) tally(x[i]);
+        __syncthreads();
+        if (tid < 256) {                 // fold the 32 copies of bin `tid` (rotated: one bank per thread)
+            unsigned sum = 0;
+#pragma unroll
+            for (int c = 0; c < 32; ++c) sum += hist[(tid << 5) + ((c + tid) & 31)];
+            bins[tid] = sum;
         }
         __syncthreads();
         if (tid == 0) {
             unsigned cum = 0;
             int b = 255;
             for (; b > 0; --b) {
-                if (cum + hist[b] >= need) break;
-                cum += hist[b];
+                if (cum + bins[b] >= need) break;
+                cum += bins[b];
             }
             sh_prefix = prefix | ((unsigned)b << shift);
             sh_need = need - cum;
@@ -91,7 +108,15 @@ __global__ __launch_bounds__(TK_THREADS) void topk_kernel(const TopkProblem p0, 
     const int begin = wave * per_wave;
     const int end = min(n, begin + per_wave);
     int cgt = 0, ceq = 0;
-    for (int i = begin + lane; i < end; i += 64) {
+    const bool vec = nvec > 0;                    // slices start at multiples of 64 elements
+    const int vend = vec ? begin + ((max(end - begin, 0)) & ~255) : begin;   // whole 256-element groups
+    for (int i = begin + 4 * lane; i < vend; i += 256) {
+        const float4 q = *reinterpret_cast<const float4 *>(x + i);
+        const unsigned u0 = order_key(q.x), u1 = order_key(q.y), u2 = order_key(q.z), u3 = order_key(q.w);
+        cgt += (u0 > T) + (u1 > T) + (u2 > T) + (u3 > T);
+        ceq += (u0 == T) + (u1 == T) + (u2 == T) + (u3 == T);
+    }
+    for (int i = vend + lane; i < end; i += 64) {
         const unsigned u = order_key(x[i]);
         cgt += u > T;
         ceq += u == T;
@@ -108,13 +133,44 @@ __global__ __launch_bounds__(TK_THREADS) void topk_kernel(const TopkProblem p0, 
 
     // ---- 3. ordered emit ---------------------------------------------------
     const int r = (int)need;
-    for (int base = begin; base < end; base += 64) {
+    const uint64_t lt = minf_lanemask_lt();
+    // 256 elements per step: lane l holds indices base + 4l .. 4l+3, so the rank of an element is
+    // (selected elements of lower lanes, all four components) + (selected lower components of its lane)
+    for (int base = begin; base < vend; base += 256) {
+        const int i0 = base + 4 * lane;
+        const float4 q = *reinterpret_cast<const float4 *>(x + i0);
+        const unsigned u[4] = {order_key(q.x), order_key(q.y), order_key(q.z), order_key(q.w)};
+        int g_lower = 0, e_lower = 0, g_all = 0, e_all = 0;
+        bool gt[4], eq[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            gt[c] = u[c] > T;
+            eq[c] = u[c] == T;
+            const uint64_t mg = __ballot(gt[c]), me = __ballot(eq[c]);
+            g_lower += __builtin_popcountll(mg & lt);
+            e_lower += __builtin_popcountll(me & lt);
+            g_all += __builtin_popcountll(mg);
+            e_all += __builtin_popcountll(me);
+        }
+        int g_here = gt_before + g_lower, e_here = eq_before + e_lower;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            if (gt[c] || (eq[c] && e_here < r)) {
+                const int i = i0 + c;
+                o[g_here + min(e_here, r)] = reverse_base >= 0 ? reverse_base - i : i;
+            }
+            g_here += gt[c];
+            e_here += eq[c];
+        }
+        gt_before += g_all;
+        eq_before += e_all;
+    }
+    for (int base = vend; base < end; base += 64) {
         const int i = base + lane;
         unsigned u = 0;
         bool gt = false, eq = false;
         if (i < end) { u = order_key(x[i]); gt = u > T; eq = u == T; }
         const uint64_t mg = __ballot(gt), me = __ballot(eq);
-        const uint64_t lt = minf_lanemask_lt();
         const int g_here = gt_before + __builtin_popcountll(mg & lt);
         const int e_here = eq_before + __builtin_popcountll(me & lt);
         const bool take = gt || (eq && e_here < r);
