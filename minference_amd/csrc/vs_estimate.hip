@@ -217,13 +217,15 @@ __global__ __launch_bounds__(LQ) void est_reduce_kernel(const EstParams p) {
 // reads -- 64 lanes cover d = -63..0, a second pass d = 1..31 -- and adds the 95 sums into a
 // private per-wave window with plain read-modify-write (one wave, in-order LDS: no race).
 constexpr int TP = 33;                       // tile row pitch (floats)
+constexpr int TROWS = 94;                    // 32 rows of a half block, 31 zero rows above, 31 below
 constexpr int WWIN = KC / 4 + LQ;            // per-wave diagonal window (256 keys + 64)
 
 // (min 2 waves per SIMD: caps the kernel at 256 registers; it is latency bound and one resident
 // wave per SIMD ran 1.4x slower)
 template <typename T>
 __global__ __launch_bounds__(EST_THREADS, 2) void est_scores_kernel(const EstParams p) {
-    __shared__ float lds_tile[4][LQ * TP];
+    // the four waves' tiles overlap in their zero rows: wave w starts 63 rows after wave w-1
+    __shared__ float lds_tile[(3 * 63 + TROWS) * TP];
     __shared__ float lds_wwin[4][WWIN];
     const WgId w = decode_wg(p);
     if (!w.valid) return;
@@ -231,10 +233,12 @@ __global__ __launch_bounds__(EST_THREADS, 2) void est_scores_kernel(const EstPar
     const int l32 = lane & 31, g = lane >> 5;
     const char *kb = p.k + ((long long)w.b * p.ks[0] + (long long)w.hkv * p.ks[1]) * 2;
     const long long bh = (long long)w.b * p.hq + w.h;
-    float *tile = lds_tile[wave];
+    float *tile = lds_tile + wave * 63 * TP;
     float *wwin = lds_wwin[wave];
 
     for (int i = lane; i < WWIN; i += 64) wwin[i] = 0.f;
+    for (int i = tid; i < (3 * 63 + TROWS) * TP; i += EST_THREADS) lds_tile[i] = 0.f;
+    __syncthreads();
 
     Frag qf[2][8];
     load_q(p, w, lane, qf);
@@ -271,32 +275,29 @@ __global__ __launch_bounds__(EST_THREADS, 2) void est_scores_kernel(const EstPar
             for (int ks = 0; ks < 8; ++ks) s = mma<T>(qf[mb][ks], kf[ks], s);
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int i = 32 * mb + 8 * (r >> 2) + 4 * g + (r & 3);
+                const int il = 8 * (r >> 2) + 4 * g + (r & 3);      // row inside this 32-row half
+                const int i = 32 * mb + il;
                 float pr = __builtin_amdgcn_exp2f(fmaf(s[r], p.scale_log2, -mrow[mb][r]));
                 if (edge) pr = (c <= qpos0 + i && c < p.n) ? pr : 0.f;
                 colsum += pr;
-                tile[i * TP + l32] = pr;
+                tile[(31 + il) * TP + l32] = pr;
             }
+            __builtin_amdgcn_wave_barrier();
+            // the 32x32 block has 63 diagonals d = n - il in [-31, 31]; lane <-> d + 31 walks its
+            // diagonal through rows n + 31 - lane, i.e. tile rows n + 62 - lane: rows outside
+            // [31, 62] are never written and stay zero, so no lane needs a bounds test and every
+            // read address is one per-lane base plus a constant
+            const float *dp = tile + (62 - min(lane, 62)) * TP;
+            float ds = 0.f;
+#pragma unroll
+            for (int n = 0; n < 32; ++n) ds += dp[n * (TP + 1)];
+            // global diagonal: key - row = (32*blk + n) - (32*mb + il) -> window slot + 63 - rshift
+            const int slot = 32 * blk + lane + 32 - 32 * mb - rshift;
+            if (lane < 63 && slot >= 0) wwin[slot] += ds;
+            __builtin_amdgcn_wave_barrier();
         }
         colsum += __shfl_xor(colsum, 32);
         if (g == 0 && c < p.n) vout[c] = colsum;
-        __builtin_amdgcn_wave_barrier();
-        // diagonal d = key - row (block-local key n, row i): window slot = 32*blk + d + 63 - rshift
-        // pass 1: lane <-> d = lane - 63 (d in [-63, 0]); pass 2: lane <-> d = lane + 1 (d in [1, 31])
-        float d1 = 0.f, d2 = 0.f;
-#pragma unroll
-        for (int n = 0; n < 32; ++n) {
-            const int i1 = n - (lane - 63);           // row on diagonal d1 at key n
-            if (i1 < LQ) d1 += tile[i1 * TP + n];
-            const int i2 = n - (lane + 1);
-            if (i2 >= 0) d2 += tile[i2 * TP + n];
-        }
-        // (rows i >= last_q hold exact zeros, so shifting by rshift only renames empty slots)
-        const int slot1 = 32 * blk + lane - rshift;
-        if (slot1 >= 0) wwin[slot1] += d1;
-        const int slot2 = 32 * blk + 64 + lane - rshift;
-        if (lane < 31 && slot2 >= 0) wwin[slot2] += d2;
-        __builtin_amdgcn_wave_barrier();
     }
     __syncthreads();
     // chunk window position q = (key - chunk0) + (last_q - 1 - i): wave wv contributes its slot q - 64*4*wv/4...
