@@ -27,8 +27,8 @@ PEAK_BF16_TFLOPS = 2500.0               # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the vertical-slash attention kernel on the default workload (seq 131072,
 # seed 100), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a 1 GiB copy kernel
-# (profiles/sparse_path_c2_128k_hbm_traffic.txt): 2.191 GB read + 1.074 GB written.
-ATTN_TRAFFIC_BYTES_C2 = 2_190_874_000 + 1_073_742_000
+# (profiles/sparse_path_c2_128k_hbm_traffic.txt): 2.097 GB read + 1.074 GB written.
+ATTN_TRAFFIC_BYTES_C2 = 2_097_082_000 + 1_073_742_000
 
 
 def cpu_baseline(budget_s=25.0):
@@ -60,12 +60,82 @@ def cpu_baseline(budget_s=25.0):
                       f"median of {len(times)} after 1 warm-up", **{k: round(x, 2) for k, x in stages.items()}}
 
 
+def _time_steps(torch, f, steps, warmup):
+    for _ in range(warmup):
+        f()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(steps):
+        f()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / steps
+
+
+def bench_index_c3(args, torch, gen, M, dev):
+    """BASELINE config 3: the vertical_slash_index builder alone, 32 heads, 1000 verticals, 6096
+    slashes drawn uniformly, full zero-filled tensors (the reference's output contract)."""
+    import numpy as np
+    out = {}
+    for n in (262144, 524288):
+        vi, si = gen.vs_index_inputs(32, n, 1000, 6096, seed=300)
+        seqlens = torch.tensor([n], dtype=torch.int32, device=dev)
+        vi_t, si_t = torch.from_numpy(vi).to(dev), torch.from_numpy(np.ascontiguousarray(si)).to(dev)
+        ms = _time_steps(torch, lambda: M.convert_vertical_slash_indexes(seqlens, vi_t, si_t, n), args.steps, args.warmup)
+        rows = n // 64
+        full = 4 * 32 * rows * (6096 + 1000 + 2)
+        out[n] = (ms, full)
+        torch.cuda.empty_cache()
+    ms, full = out[524288]
+    gbs = full / (ms * 1e-3) / 1e9
+    print(json.dumps({
+        "metric": "vertical_slash_index build, ms (BASELINE config 3, seq 524288)", "value": round(ms, 3),
+        "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 3),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "int32", "data": "synthetic",
+        "config": {"workload": "BASELINE config 3: index builder alone, 32 heads, 1000 verticals, 6096 slashes, "
+                               "full zero-filled outputs", "seq_len": 524288},
+        "ms_at_262144": round(out[262144][0], 3),
+        "roofline": {"kernel": "vs_index_prep_kernel + vs_index_fast_kernel", "bound": "hbm",
+                     "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None, "bytes_per_launch": full}}))
+
+
+def bench_block_sparse_c4(args, torch, gen, M, dev):
+    """BASELINE config 4: top-100 block-sparse attention (diagonal and block 0 always kept) on the
+    config 2 inputs, 131072 tokens, 32 q / 8 kv heads."""
+    from minference_amd.ops import _build_block_index, block_sparse_attention_from_index
+    n = args.seq
+    q, k, v, _ = gen.planted_layer(n, 32, 8, seed=100, dtype=torch.bfloat16)
+    q, k, v = q.to(dev), k.to(dev), v.to(dev)
+    ms_idx = _time_steps(torch, lambda: _build_block_index(q, k, 100, force_diag_first=True), args.steps, args.warmup)
+    bi = _build_block_index(q, k, 100, force_diag_first=True)
+    ms_att = _time_steps(torch, lambda: block_sparse_attention_from_index(q, k, v, bi), args.steps, args.warmup)
+    tiles = 32 * sum(min(m + 1, 100) for m in range((n + 63) // 64))
+    tf = tiles * TILE_FLOP / (ms_att * 1e-3) / 1e12
+    print(json.dumps({
+        "metric": "block-sparse prefill attn ms/layer @128K (BASELINE config 4)", "value": round(ms_idx + ms_att, 3),
+        "unit": "ms/layer", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_idx + ms_att, 3), "higher_is_better": False, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "BASELINE config 4: block-sparse top-100 (diagonal and first block kept), "
+                               "32 q / 8 kv heads, planted inputs of config 2", "seq_len": n},
+        "stage_ms": {"block_index": round(ms_idx, 3), "attention": round(ms_att, 3)}, "computed_tiles": tiles,
+        "roofline": {"kernel": "attn_fwd_kernel<bf16, block-sparse>", "bound": "mfma", "achieved": round(tf, 1),
+                     "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / PEAK_BF16_TFLOPS, 4),
+                     "traffic": None, "launch_ms": round(ms_att, 3), "flop_per_launch": tiles * TILE_FLOP}}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--seq", type=int, default=131072)
+    ap.add_argument("--workload", default="vs_c2", choices=["vs_c2", "index_c3", "block_sparse_c4"],
+                    help="vs_c2 (default): the headline layer, BASELINE config 2; index_c3: the index "
+                         "builder alone on config 3; block_sparse_c4: config 4 (secondary lines, used "
+                         "for the committed rocprofv3 summaries)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-dense", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -84,6 +154,10 @@ def main():
     _lib.load()                                        # fail loudly if the HIP library is missing
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.workload == "index_c3":
+        return bench_index_c3(args, torch, gen, M, dev)
+    if args.workload == "block_sparse_c4":
+        return bench_block_sparse_c4(args, torch, gen, M, dev)
     n, hq, hk = args.seq, 32, 8
     vertical_size, slash_size = 1000, 6096
 

@@ -40,6 +40,44 @@ __device__ __forceinline__ void zero_range(int32_t *p, int from, int to, int lan
     if (lane < tail) q[n4 * 4 + lane] = 0;
 }
 
+// Range starts of one chunk of 64 entries.  `t` ascends along the lanes (padding lanes repeat the
+// last entry); the state carried in from the previous chunk is the current range start `cur_a`,
+// the running range end `carried_e` and the previous entry `carried_t`.  Entry i starts a new
+// range iff t_i > e_{i-1} + 64, and t_{i-1} <= e_{i-1} < t_{i-1} + 64, so
+//   t_i >  t_{i-1} + 127  is always a start,      (decided for all lanes with one ballot)
+//   t_i <= t_{i-1} + 64   never is,
+// and only the lanes in between depend on the 64-phase of their range; those are resolved one by
+// one in lane order with scalar arithmetic.  Returns this lane's range start; `starts` gets the
+// mask of lanes that start a range.
+__device__ __forceinline__ int chunk_ranges(int t, int lane, int cur_a, int carried_e, int carried_t,
+                                            uint64_t &starts) {
+    int tprev = __shfl_up(t, 1);
+    if (lane == 0) tprev = carried_t;
+    const bool sure = lane == 0 ? (t > carried_e + 64) : (t > tprev + 127);
+    const bool maybe = lane != 0 && !sure && (t > tprev + 64);
+    uint64_t sm = __ballot(sure);
+    uint64_t mm = __ballot(maybe);
+    const uint64_t le = minf_lanemask_lt() | (1ull << lane);
+    const uint64_t below = sm & le;
+    const int j0 = below ? 63 - __builtin_clzll(below) : 0;
+    const int tj0 = __shfl(t, j0);
+    int a = below ? tj0 - 64 : cur_a;
+    while (mm) {
+        const int j = __builtin_ctzll(mm);
+        mm &= mm - 1;
+        const int ap = minf_readlane(a, j - 1), tp = minf_readlane(t, j - 1), tj = minf_readlane(t, j);
+        const int ep = ap + ((((tp - ap) + 63) >> 6) << 6);
+        if (tj > ep + 64) {
+            const uint64_t later = sm & ~((2ull << j) - 1ull);          // sure starts above lane j
+            const int next = later ? __builtin_ctzll(later) : 64;
+            if (lane >= j && lane < next) a = tj - 64;
+            sm |= 1ull << j;
+        }
+    }
+    starts = sm;
+    return a;
+}
+
 __global__ __launch_bounds__(IDX_WAVES *MINF_WAVE) void vs_index_kernel(
     const int32_t *__restrict__ seqlens, const int32_t *__restrict__ vertical,
     const int32_t *__restrict__ slash, int32_t *__restrict__ block_count,
@@ -104,21 +142,8 @@ __global__ __launch_bounds__(IDX_WAVES *MINF_WAVE) void vs_index_kernel(
                 carried_e = t0 - 64;
                 carried_t = t0;
             }
-            int a = cur_a;
-            int tprev = __shfl_up(t, 1);
-            if (lane == 0) tprev = carried_t;
-            int start = 0;
-            for (;;) {
-                int eprev = a + ((((tprev - a) + 63) >> 6) << 6);
-                if (lane == 0) eprev = carried_e;
-                const bool brk = (lane >= start) && (t > eprev + 64);
-                const uint64_t bm = __ballot(brk);
-                if (bm == 0) break;
-                const int j = __builtin_ctzll(bm);
-                const int tj = minf_readlane(t, j);
-                if (lane >= j) a = tj - 64;
-                start = j + 1;
-            }
+            uint64_t starts;
+            const int a = chunk_ranges(t, lane, cur_a, carried_e, carried_t, starts);
             const int e = a + ((((t - a) + 63) >> 6) << 6);
             int eprev = __shfl_up(e, 1);
             if (lane == 0) eprev = carried_e;
@@ -225,24 +250,9 @@ __global__ __launch_bounds__(MINF_WAVE) void vs_index_prep_kernel(const int32_t 
             carried_e = t0 - 64;
             carried_t = t0;
         }
-        int a = cur_a;
-        int tprev = __shfl_up(t, 1);
-        if (lane == 0) tprev = carried_t;
-        int start = 0;
-        bool is_start = (c == 0 && lane == 0);
-        for (;;) {
-            int eprev = a + ((((tprev - a) + 63) >> 6) << 6);
-            if (lane == 0) eprev = carried_e;
-            const bool brk = (lane >= start) && (t > eprev + 64);
-            const uint64_t bm = __ballot(brk);
-            if (bm == 0) break;
-            const int j = __builtin_ctzll(bm);
-            const int tj = minf_readlane(t, j);
-            if (lane >= j) a = tj - 64;
-            if (lane == j) is_start = true;
-            start = j + 1;
-        }
-        is_start = is_start && valid;
+        uint64_t starts;
+        const int a = chunk_ranges(t, lane, cur_a, carried_e, carried_t, starts);
+        const bool is_start = valid && (((starts >> lane) & 1ull) || (c == 0 && lane == 0));
         const int e = a + ((((t - a) + 63) >> 6) << 6);
         int eprev = __shfl_up(e, 1);
         if (lane == 0) eprev = carried_e;
@@ -347,22 +357,12 @@ __global__ __launch_bounds__(IDX_WAVES *MINF_WAVE) void vs_index_fast_kernel(
                     carried_e = t0 - 64;
                     carried_t = t0;
                 }
-                int a = cur_a;
-                int tprev = __shfl_up(t, 1);
-                if (lane == 0) tprev = carried_t;
-                int start = 0, cut = -1;
-                for (;;) {
-                    int eprev = a + ((((tprev - a) + 63) >> 6) << 6);
-                    if (lane == 0) eprev = carried_e;
-                    const bool brk = (lane >= start) && (t > eprev + 64);
-                    const uint64_t bm = __ballot(brk);
-                    if (bm == 0) break;
-                    const int j = __builtin_ctzll(bm);
-                    if (cpre[base + j] >= 0) { cut = j; break; }      // a tabulated range starts here
-                    const int tj = minf_readlane(t, j);
-                    if (lane >= j) a = tj - 64;
-                    start = j + 1;
-                }
+                uint64_t starts;
+                int a = chunk_ranges(t, lane, cur_a, carried_e, carried_t, starts);
+                // the first range start of this chunk that is also a tabulated range start
+                const bool tab = ((starts >> lane) & 1ull) && cpre[base + lane] >= 0;
+                const uint64_t tm = __ballot(tab);
+                const int cut = tm ? __builtin_ctzll(tm) : -1;
                 if (cut == 0) {          // nothing of this chunk belongs to the explicit part
                     g = base;
                     e_lim = carried_e;
