@@ -463,8 +463,11 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
 }
 
 int check_tensors(const minf_qkvo *t) {
-    if (!t || !t->q || !t->k || !t->v || !t->o) return MINF_ERR_INVALID_ARG;
+    if (!t) return MINF_ERR_INVALID_ARG;
     if (t->batch < 0 || t->heads_q <= 0 || t->heads_kv <= 0 || t->n < 0) return MINF_ERR_INVALID_ARG;
+    // empty problems (no batch or no tokens) have no storage: nothing to check, nothing is launched
+    const bool empty = t->batch == 0 || t->n == 0;
+    if (!empty && (!t->q || !t->k || !t->v || !t->o)) return MINF_ERR_INVALID_ARG;
     if (t->heads_q % t->heads_kv != 0) return MINF_ERR_INVALID_ARG;
     if (t->head_dim != HD) return MINF_ERR_UNSUPPORTED;
     if (t->dtype != MINF_BF16 && t->dtype != MINF_F16) return MINF_ERR_UNSUPPORTED;

@@ -238,3 +238,52 @@ def test_block_sparse_config4_shape_scaled(gpu):
         assert (bic[0, :, m, : min(m + 1, 100)] == m).any(axis=-1).all()
     ref = torch.stack([O.masked_attention(q[0, h], k[0, 0], v[0, 0], O.bs_mask(bic[0, h], n)) for h in range(hq)])[None]
     check(out, ref, "bs-c4")
+
+
+def test_ragged_seqlens_in_a_batch(gpu):
+    """Two sequences of different length padded to one tensor: rows at or past a sequence's length
+    come out as zeros, keys at or past it are never attended (pit_sparse_flash_attention_v2.py:67-69,
+    :110-113), the rest matches the fp32 oracle built with the same seqlens."""
+    from minference_amd import convert_vertical_slash_indexes, vertical_slash_attention_from_index
+    n, hq, hk, lens = 1000, 2, 1, [1000, 613]
+    q, k, v = make(2, hq, hk, n, 50, torch.bfloat16)
+    vi, si = gen.vs_index_inputs(hq, n, 30, 60, seed=8, batch=2, force_v=4, force_s=8)
+    seqlens = torch.tensor(lens, dtype=torch.int32, device=gpu)
+    idx = convert_vertical_slash_indexes(seqlens, torch.from_numpy(vi).to(gpu),
+                                         torch.from_numpy(np.ascontiguousarray(si)).to(gpu), n)
+    out = vertical_slash_attention_from_index(q.to(gpu), k.to(gpu), v.to(gpu), *idx, seqlens).float().cpu()
+    rbc, rbo, rcc, rci = O.vs_index_build(lens, vi, si, n)
+    for b in range(2):
+        assert torch.count_nonzero(out[b, :, lens[b]:]) == 0
+        for h in range(hq):
+            mask = O.vs_mask(rbc[b, h], rbo[b, h], rcc[b, h], rci[b, h], n, lens[b])
+            ref = O.masked_attention(q[b, h], k[b, 0], v[b, 0], mask)
+            err = (out[b, h, : lens[b]] - ref[: lens[b]]).abs()
+            assert err.max() <= MAX_ABS and err.mean() <= MEAN_ABS, (b, h, err.max())
+
+
+@pytest.mark.parametrize("n", [1, 37, 63, 65])
+def test_tiny_sequences_all_operators(gpu, n):
+    import minference_amd as M
+    print(f"case tiny n={n}", flush=True)
+    q, k, v = make(1, 2, 1, n, 60 + n, torch.bfloat16)
+    ref = sdpa_causal(q, expand(k, 2), expand(v, 2))
+    qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
+    check(M.dense_causal_attention(qg, kg, vg), ref, "tiny-dense")
+    check(M.streaming_forward(qg, kg, vg, 4, 1000), ref, "tiny-ashape")            # window covers everything
+    check(M.block_sparse_attention(qg, kg, vg, 100), ref, "tiny-bs")
+    # every diagonal kept -> causal
+    s_idx = torch.arange(n, dtype=torch.int64)[None, None].expand(1, 2, n).contiguous()
+    v_idx = torch.zeros((1, 2, 1), dtype=torch.int64)
+    check(M.vertical_slash_sparse_attention(qg, kg, vg, v_idx.to(gpu), s_idx.to(gpu)), ref, "tiny-vs")
+    v2, s2 = M.estimate_vertical_slash(qg, kg, 1000, 6096)                          # clamps to n
+    assert v2.shape[-1] == min(n, 1000) and s2.shape[-1] == min(n, 6096)
+    check(M.vertical_slash_sparse_attention(qg, kg, vg, v2, s2), ref, "tiny-vs-estimated")
+
+
+def test_empty_batch(gpu):
+    import minference_amd as M
+    q = torch.zeros((0, 2, 128, 128), dtype=torch.bfloat16, device=gpu)
+    k = torch.zeros((0, 1, 128, 128), dtype=torch.bfloat16, device=gpu)
+    assert tuple(M.dense_causal_attention(q, k, k).shape) == (0, 2, 128, 128)
+    assert tuple(M.streaming_forward(q, k, k, 4, 64).shape) == (0, 2, 128, 128)
