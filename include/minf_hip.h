@@ -148,6 +148,15 @@ int minf_bs_attn_fwd(const minf_qkvo *t, const int32_t *block_index, int rows,
 int minf_ashape_attn_fwd(const minf_qkvo *t, int n_init, int n_local, void *stream);
 
 /*
+ * Tri-shape: A-shape for the first n - n_last query rows, dense causal attention for the last
+ * n_last rows, in one launch of the same kernel.  Replaces tri_shape_kernel (reference
+ * minference/ops/streaming_kernel.py:820-833 and minference/modules/minference_forward.py:444-455),
+ * which runs the A-shape op on the truncated sequence, a dense einsum/softmax for the last rows
+ * and a torch.cat.  The caller clamps n_last to n - 1 like the reference.
+ */
+int minf_trishape_attn_fwd(const minf_qkvo *t, int n_init, int n_local, int n_last, void *stream);
+
+/*
  * Dense causal forward on the same tile engine (the in-house comparator for
  * the sparse-vs-dense speed-up; the reference uses flash_attn_func,
  * minference/modules/minference_forward.py:666).

@@ -9,7 +9,7 @@ operator without them raises.
 """
 from .index import convert_vertical_slash_indexes
 from .ops import (block_sparse_attention, block_sparse_attention_from_index, dense_causal_attention,
-                  streaming_forward, vertical_slash_attention_from_index,
+                  streaming_forward, tri_shape_forward, vertical_slash_attention_from_index,
                   vertical_slash_sparse_attention)
 
 from .estimate import estimate_vertical_slash, topk_indices, vertical_slash_scores
@@ -21,6 +21,6 @@ __all__ = [
     "minference_prefill_forward", "minference_prefill_kernel", "load_best_pattern",
     "vertical_slash_sparse_attention", "block_sparse_attention", "streaming_forward",
     "convert_vertical_slash_indexes", "vertical_slash_attention_from_index",
-    "block_sparse_attention_from_index", "dense_causal_attention",
+    "block_sparse_attention_from_index", "dense_causal_attention", "tri_shape_forward",
 ]
 __version__ = "0.1.0"

@@ -68,8 +68,8 @@ struct AttnParams {
     // block-sparse
     const int *bidx;
     int max_blocks, bidx_rows;
-    // a-shape
-    int n_init, n_local;
+    // a-shape; query rows >= dense_from attend to every earlier key (tri-shape), INT_MAX = none
+    int n_init, n_local, dense_from;
     long long total_wg;
 };
 
@@ -144,6 +144,10 @@ __device__ __forceinline__ int tile_count(const AttnParams &p, long long ridx, i
         nblk = min(m + 1, p.max_blocks);
         return nblk;
     } else if constexpr (MODE == MODE_ASHAPE) {
+        if (m * BM + BM - 1 >= p.dense_from) {     // block holds dense rows: every causal tile
+            nblk = m + 1;
+            return nblk;
+        }
         // window tiles t_lo..m, preceded by the sink tiles that lie before t_lo
         int lo_key = m * BM - p.n_local + 1;
         int t_lo = lo_key > 0 ? (lo_key >> 6) : 0;
@@ -358,8 +362,9 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
                 const bool causal_ok = c_hi <= wrow_lo && c_hi < seqlen;
                 const bool in_window = (wrow_hi - c_lo) < p.n_local;
                 const bool in_sink = c_hi < p.n_init;
-                need_mask = !(causal_ok && (in_window || in_sink));
-                wlo = qrow - cur.start - p.n_local - 4 * g;
+                const bool all_dense = wrow_lo >= p.dense_from, none_dense = wrow_hi < p.dense_from;
+                need_mask = all_dense ? !causal_ok : (none_dense ? !(causal_ok && (in_window || in_sink)) : true);
+                wlo = qrow >= p.dense_from ? -(1 << 30) : qrow - cur.start - p.n_local - 4 * g;
                 slim = p.n_init - cur.start - 4 * g;
             } else {
                 need_mask = (cur.start + BN - 1 > wrow_lo) || (cur.start + BN > seqlen);
@@ -493,7 +498,7 @@ void fill_params(AttnParams &p, const minf_qkvo *t) {
     p.rows = (t->n + BM - 1) / BM;
     p.bc = p.bo = p.cc = p.ci = nullptr; p.nnz_s = p.nnz_v = 0;
     p.bidx = nullptr; p.max_blocks = 0; p.bidx_rows = 0;
-    p.n_init = p.n_local = 0;
+    p.n_init = p.n_local = 0; p.dense_from = 0x7fffffff;
     p.total_wg = (long long)t->batch * t->heads_q * p.rows;
 }
 
@@ -549,6 +554,17 @@ extern "C" int minf_ashape_attn_fwd(const minf_qkvo *t, int n_init, int n_local,
     AttnParams p;
     fill_params(p, t);
     p.n_init = n_init; p.n_local = n_local;
+    return launch<MODE_ASHAPE>(p, t->dtype, stream);
+}
+
+extern "C" int minf_trishape_attn_fwd(const minf_qkvo *t, int n_init, int n_local, int n_last, void *stream) {
+    int st = check_tensors(t);
+    if (st) return st;
+    if (n_init < 0 || n_local < 1 || n_last < 0) return MINF_ERR_INVALID_ARG;
+    AttnParams p;
+    fill_params(p, t);
+    p.n_init = n_init; p.n_local = n_local;
+    p.dense_from = n_last < t->n ? t->n - n_last : 0;
     return launch<MODE_ASHAPE>(p, t->dtype, stream);
 }
 

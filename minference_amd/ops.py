@@ -202,6 +202,20 @@ def streaming_forward(q, k, v, n_init: int, n_local: int):
     return c.result()
 
 
+def tri_shape_forward(q, k, v, n_init: int, n_local: int, n_last: int = 100):
+    """Tri-shape attention: A-shape (n_init sink tokens + window of n_local) for all but the last
+    n_last query rows, dense causal attention for those (streaming_kernel.py:820-833,
+    minference_forward.py:444-455), in one launch."""
+    c = _Call(q, k, v)
+    n_last = min(int(n_last), c.N - 1)                   # reference: min(n_last, q.size(2) - 1)
+    lib = _lib.load()
+    with torch.cuda.device(c.q.device):
+        st = lib.minf_trishape_attn_fwd(c.ref, int(n_init), int(n_local), max(n_last, 0),
+                                        _lib.stream_ptr(c.q.device))
+    _lib.check(st, "minf_trishape_attn_fwd")
+    return c.result()
+
+
 def dense_causal_attention(q, k, v):
     """Dense causal attention on the same tile engine (comparator for speed-up figures)."""
     c = _Call(q, k, v)

@@ -277,6 +277,18 @@ def ashape_mask(n, n_init, n_local):
     return ((d >= 0) & (d < n_local)) | ((c < n_init) & (d >= n_local))
 
 
+def trishape_mask(n, n_init, n_local, n_last):
+    """tri_shape_kernel (streaming_kernel.py:820-833): the A-shape mask for rows < n - n_last
+    (a_shape_kernel on the truncated sequence: causality keeps those rows inside it), the full
+    causal row for the last n_last rows (:826-829); n_last is clamped to n - 1 (:822)."""
+    n_last = min(n_last, n - 1)
+    mask = ashape_mask(n, n_init, n_local)
+    if n_last > 0:
+        r = np.arange(n - n_last, n)[:, None]
+        mask[n - n_last:] = np.arange(n)[None, :] <= r
+    return mask
+
+
 def masked_attention(q, k, v, mask, scale=None):
     """Exact fp32 softmax attention of one head under a boolean mask.
     q [n,D], k,v [n,D] (any float dtype) -> [n,D] fp32.  Rows with an empty

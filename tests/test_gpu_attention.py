@@ -287,3 +287,15 @@ def test_empty_batch(gpu):
     k = torch.zeros((0, 1, 128, 128), dtype=torch.bfloat16, device=gpu)
     assert tuple(M.dense_causal_attention(q, k, k).shape) == (0, 2, 128, 128)
     assert tuple(M.streaming_forward(q, k, k, 4, 64).shape) == (0, 2, 128, 128)
+
+
+@pytest.mark.parametrize("n,n_init,n_local,n_last", [(1024, 128, 256, 100), (1500, 4, 100, 64), (777, 130, 70, 333),
+                                                     (640, 0, 50, 1), (900, 16, 64, 5000), (200, 8, 32, 0)])
+def test_tri_shape_vs_oracle(gpu, n, n_init, n_local, n_last):
+    from minference_amd import tri_shape_forward
+    print(f"case trishape n={n} init={n_init} local={n_local} last={n_last}", flush=True)
+    q, k, v = make(1, 2, 1, n, 70, torch.bfloat16)
+    out = tri_shape_forward(q.to(gpu), k.to(gpu), v.to(gpu), n_init, n_local, n_last)
+    mask = O.trishape_mask(n, n_init, n_local, n_last)
+    ref = torch.stack([O.masked_attention(q[0, h], k[0, 0], v[0, 0], mask) for h in range(2)])[None]
+    check(out, ref, "trishape")

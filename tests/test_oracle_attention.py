@@ -103,3 +103,18 @@ def test_golden_fixtures_reproduce():
     assert np.allclose(out.numpy(), z["vs_out"], atol=1e-6)
     assert np.allclose(O.streaming_forward(q, k, v, 8, 48).numpy(), z["ashape_out"], atol=1e-6)
     assert np.allclose(O.block_sparse_attention(q, k, v, 2).numpy(), z["bs_out"], atol=1e-6)
+
+
+def test_trishape_mask_definition_and_limits():
+    n, n_init, n_local, n_last = 300, 8, 40, 100
+    m = O.trishape_mask(n, n_init, n_local, n_last)
+    for r in range(n):
+        for c in range(n):
+            if r >= n - n_last:
+                want = c <= r
+            else:
+                want = (c <= r and c > r - n_local) or (c < n_init and c <= r - n_local)
+            assert m[r, c] == want, (r, c)
+    # n_last >= n clamps to n - 1: every row but the first is dense, and row 0 only sees key 0 anyway
+    assert np.array_equal(O.trishape_mask(50, 2, 5, 1000), np.tril(np.ones((50, 50), bool)))
+    assert np.array_equal(O.trishape_mask(50, 2, 5, 0), O.ashape_mask(50, 2, 5))
