@@ -126,16 +126,53 @@ def bench_block_sparse_c4(args, torch, gen, M, dev):
                      "traffic": None, "launch_ms": round(ms_att, 3), "flop_per_launch": tiles * TILE_FLOP}}))
 
 
+def bench_llama_c5(args, torch, dev):
+    """BASELINE config 5: random-init Llama-3-8B (32 layers, hidden 4096, 32 q / 8 kv heads, RoPE
+    theta 500000, SwiGLU 14336, vocab 128256), one 262144-token prefill, per-head patterns drawn
+    with seed 501 (70 % vertical_slash 1000/6096, 20 % block_sparse top-100, 10 % A-shape 128+4096)."""
+    from minference_amd.llama import LlamaConfig, LlamaPrefill, seeded_pattern_mix
+    n = args.seq if args.seq != 131072 else 262144
+    cfg = LlamaConfig(num_layers=args.layers)
+    model = LlamaPrefill(cfg, device=dev, seed=0)
+    ids = torch.randint(0, cfg.vocab_size, (n,), generator=torch.Generator().manual_seed(500))
+    afc = {"best_pattern": seeded_pattern_mix(cfg.num_layers, cfg.num_heads, seed=501)}
+
+    def run():
+        logits, _ = model.prefill(ids, afc)
+        return logits
+    for _ in range(args.warmup):
+        run()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        logits = run()
+    torch.cuda.synchronize()
+    sec = (time.perf_counter() - t0) / args.steps
+    assert torch.isfinite(logits).all()
+    print(json.dumps({
+        "metric": "Llama-3-8B prefill seconds @262144 tokens (BASELINE config 5)", "value": round(sec, 3),
+        "unit": "s/prefill", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(sec * 1e3, 1), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "BASELINE config 5: random-init Llama-3-8B architecture, random token ids, "
+                               "seeded 70/20/10 per-head mix of vertical_slash / block_sparse / A-shape",
+                   "seq_len": n, "layers": cfg.num_layers},
+        "tokens_per_s": round(n / sec, 1),
+        "linear_tflops_if_attention_were_free": round(model.flops_linear(n) / sec / 1e12, 1)}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--seq", type=int, default=131072)
-    ap.add_argument("--workload", default="vs_c2", choices=["vs_c2", "index_c3", "block_sparse_c4"],
+    ap.add_argument("--workload", default="vs_c2", choices=["vs_c2", "index_c3", "block_sparse_c4", "llama_c5"],
                     help="vs_c2 (default): the headline layer, BASELINE config 2; index_c3: the index "
                          "builder alone on config 3; block_sparse_c4: config 4 (secondary lines, used "
-                         "for the committed rocprofv3 summaries)")
+                         "for the committed rocprofv3 summaries); llama_c5: random-init Llama-3-8B "
+                         "prefill of 262144 tokens with config 5's seeded per-head pattern mix")
+    ap.add_argument("--layers", type=int, default=32, help="llama_c5: number of decoder layers")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-dense", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -158,6 +195,8 @@ def main():
         return bench_index_c3(args, torch, gen, M, dev)
     if args.workload == "block_sparse_c4":
         return bench_block_sparse_c4(args, torch, gen, M, dev)
+    if args.workload == "llama_c5":
+        return bench_llama_c5(args, torch, dev)
     n, hq, hk = args.seq, 32, 8
     vertical_size, slash_size = 1000, 6096
 
