@@ -16,25 +16,36 @@
 // the probabilities of a lane are exactly the B operand of the second MFMA once
 // the contraction (token) index is permuted the same way on the V side.
 //
-// LDS: K and V tiles are [64 tokens][128] 16-bit with padded row pitches (K 272 B, V 320 B), so
-// the ds_read_b128 of 32 K rows and the 4-row transpose reads of V hit distinct banks and every
-// read address is a per-lane base plus an immediate offset.  Global->LDS goes through registers,
-// fetched one tile ahead; contiguous tiles use one scalar base per tile, gathered (vertical
-// column) tiles one 256-byte row per token.
+// LDS: one K and one V tile per workgroup, [64 tokens][128] 16-bit, 256-byte rows whose 16-byte
+// chunks are XOR-permuted (K: chunk ^ row%16, V: chunk ^ 4*(row%4)) so that the ds_read_b128 of 32
+// K rows and the 4-row transpose reads of V hit distinct banks.  Tiles are copied global -> LDS
+// directly (global_load_lds_dwordx4, no staging registers, no LDS store instructions); the
+// permutation is applied on the global-address side.  32 KB of LDS and <= 256 registers keep four
+// workgroups (two waves per SIMD) resident per CU.
+//
+// One iteration of a wave (two workgroup barriers per tile, single buffers):
+//   wait own K(it) copies; barrier (all of K(it) visible, everyone done with V(it-1))
+//   issue V(it) copy; S^T = K.Q^T with the K fragments read two k-steps ahead of their MFMAs
+//   wait own V(it) copies; barrier (all of V(it) visible, everyone done with K(it))
+//   issue K(it+1) copy; row max; exponentials of keys 0..31
+//   O^T += V^T.P^T with the exponentials of keys 32..63 placed behind the first eight MFMAs and
+//   the V^T fragments of key group s+1 read under the MFMAs of group s
+// The compiler's own schedule read every fragment right before its MFMA (full LDS latency exposed
+// sixteen times per tile); the order above is pinned with sched_barrier / sched_group_barrier.
 //
 // Other choices that measure faster on MI355X:
-//  * index entries (block offsets, column ids) are wave-uniform and read through the constant
-//    address space, i.e. scalar loads that do not queue behind the K/V vector loads;
+//  * index entries (block offsets, column counts) are wave-uniform and read through the constant
+//    address space, i.e. scalar loads that do not queue behind the vector memory traffic; gathered
+//    column ids are fetched one per lane an iteration ahead and distributed with wave shuffles;
 //  * the running max is only raised when a tile exceeds it by more than 2^8 (probabilities stay
 //    below 2^8, far inside fp32/bf16 range), so most tiles skip the O^T rescale;
 //  * the cross-half max uses v_permlane32_swap, the row sums v_dot2 on the rounded probabilities
 //    (the same values the second MFMA consumes);
-//  * s_setprio raises the wave while it issues MFMAs so the partner wave's softmax fills the gaps
-//    (not in dense mode: at 128K dense is bound by L2 reuse between workgroups that stream the
-//    same K/V, and both the priority switch and the scalar-base loads measure 20 % slower there);
+//  * s_setprio raises the wave while it issues MFMAs (not in dense mode);
 //  * the epilogue transposes O^T through LDS so each global store is 16 B of one 256-byte row.
 #include "minf_common.h"
 #include <math.h>
+#include <type_traits>
 
 namespace {
 
@@ -53,6 +64,11 @@ constexpr int BN = 64;        // keys per tile
 constexpr int HD = 128;       // head_dim
 constexpr int NTHREADS = 128; // 2 wavefronts
 constexpr int ROW_BYTES = HD * 2;
+// Scheduling constants (measured on MI355X): K fragments are read QK_AHEAD k-steps ahead of their
+// MFMAs; VALU_PER_MFMA softmax instructions are placed behind each of the first eight PV MFMAs.
+constexpr int QK_AHEAD = 2;
+constexpr int VALU_PER_MFMA = 5;
+constexpr int VALU_MASK = 0x402;             // sched_group_barrier classes: VALU | transcendental
 
 struct AttnParams {
     const char *q, *k, *v;
@@ -187,9 +203,9 @@ __device__ __forceinline__ Tile tile_at(const AttnParams &p, long long ridx, int
 
 template <typename T, int MODE>
 __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams p) {
-    constexpr int KP = ROW_BYTES + 16, VP = ROW_BYTES + 64;
-    __shared__ __attribute__((aligned(16))) char lds_k[BN * KP];
-    __shared__ __attribute__((aligned(16))) char lds_v[BN * VP];
+    // two separate LDS objects: the compiler then lets reads of one overtake copies into the other
+    __shared__ __attribute__((aligned(16))) char lds_k[BN * ROW_BYTES];
+    __shared__ __attribute__((aligned(16))) char lds_v[BN * ROW_BYTES];
 
     // ---- which (batch, head, row block): XCD-aware remap --------------------
     // Consecutive workgroup ids are dealt round-robin to the 8 XCDs; give each
@@ -251,50 +267,49 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
     int nblk = 0;
     const int ntiles = tile_count<MODE>(p, ridx, m, nblk);
 
-    // ---- global -> register staging: thread covers rows i*8 + tid/16, chunk tid%16
-    const int ld_r = tid >> 4;       // 0..7
-    const int ld_c = tid & 15;       // 16-byte chunk in the row
-    u32x4_t kreg[8], vreg[8];
-
-    // Rows that do not exist (past seqlen, or padding of a gathered tile) are read from a
-    // clamped, valid address instead of being zeroed: their scores are always masked to
-    // -inf below, so their probabilities are exactly 0 and K/V contents never matter.
-    auto issue_loads = [&](const Tile &t) {
-        if (MODE != MODE_DENSE && !(MODE == MODE_VS && t.gathered) && t.start >= 0 && t.start + BN <= seqlen) {
-            const char *kb = k_base + (long long)t.start * k_row;
-            const char *vb = v_base + (long long)t.start * v_row;
-            const unsigned ko = (unsigned)(ld_r * k_row + ld_c * 16), vo = (unsigned)(ld_r * v_row + ld_c * 16);
+    // ---- global -> LDS copies without a register round trip (global_load_lds_dwordx4): every lane
+    // fetches 16 bytes from its own global address and the wave's 64 x 16 B land contiguously in
+    // LDS at a wave-uniform base (lane i -> base + 16*i), i.e. one instruction fills 4 tile rows;
+    // wave w owns rows 32*w .. 32*w+31 (8 instructions per matrix).  The 16-byte chunks of a row
+    // are permuted for conflict-free reads (K: chunk ^ row%16, V: chunk ^ 4*(row%4)); the
+    // permutation is applied on the global side: lane (row, c') loads global chunk c' ^ swz(row).
+    // Rows that do not exist (past seqlen, or padding of a gathered tile) are read from a clamped,
+    // valid address: their scores are masked to -inf, so their probabilities are exactly 0.
+    const int cp_r = lane >> 4;                  // row inside the 4-row group
+    const int cp_c = lane & 15;                  // LDS chunk
+    // gathered tiles: lane l holds the token id of tile row l (one load per lane, issued an
+    // iteration ahead); the copy fetches the ids of its own rows with wave shuffles
+    auto gather_ids = [&](const Tile &t) -> int {
+        if (MODE == MODE_VS && t.gathered) return p.ci[ridx * p.nnz_v + t.start + min(lane, t.nvalid - 1)];
+        return 0;
+    };
+    auto copy_tile = [&](const Tile &t, const char *base, long long rowstride, auto is_v_c, int idv,
+                         char *ldsbuf) {
+        constexpr bool is_v = decltype(is_v_c)::value;
+        const bool gathered = MODE == MODE_VS && t.gathered;
+        if (!gathered && t.start >= 0 && t.start + BN <= seqlen) {
+            const char *tb = base + (long long)t.start * rowstride;      // wave-uniform
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                kreg[i] = *reinterpret_cast<const u32x4_t *>(kb + (long long)i * 8 * k_row + ko);
-                vreg[i] = *reinterpret_cast<const u32x4_t *>(vb + (long long)i * 8 * v_row + vo);
+            for (int j = 0; j < 8; ++j) {
+                const int r = 32 * wave + 4 * j + cp_r;
+                const int c = is_v ? (cp_c ^ ((r & 3) << 2)) : (cp_c ^ (r & 15));
+                const char *gp = tb + (unsigned)(r * (int)rowstride + c * 16);
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
+                                                 (__attribute__((address_space(3))) void *)(ldsbuf + (32 * wave + 4 * j) * ROW_BYTES),
+                                                 16, 0, 0);
             }
             return;
         }
-        int tok[8];
-        if (MODE == MODE_VS && t.gathered) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const int r = i * 8 + ld_r;
-                tok[i] = p.ci[ridx * p.nnz_v + t.start + min(r, t.nvalid - 1)];
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) tok[i] = t.start + i * 8 + ld_r;
-        }
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int tk = max(0, min(tok[i], seqlen - 1));
-            kreg[i] = *reinterpret_cast<const u32x4_t *>(k_base + tk * k_row + ld_c * 16);
-            vreg[i] = *reinterpret_cast<const u32x4_t *>(v_base + tk * v_row + ld_c * 16);
-        }
-    };
-    auto store_lds = [&]() {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int r = i * 8 + ld_r;
-            *reinterpret_cast<u32x4_t *>(lds_k + r * KP + (ld_c << 4)) = kreg[i];
-            *reinterpret_cast<u32x4_t *>(lds_v + r * VP + (ld_c << 4)) = vreg[i];
+        for (int j = 0; j < 8; ++j) {
+            const int r = 32 * wave + 4 * j + cp_r;          // tile row
+            const int tok = gathered ? __shfl(idv, r) : t.start + r;
+            const int tk = max(0, min(tok, seqlen - 1));
+            const int c = is_v ? (cp_c ^ ((r & 3) << 2)) : (cp_c ^ (r & 15));
+            const char *gp = base + tk * rowstride + c * 16;
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
+                                             (__attribute__((address_space(3))) void *)(ldsbuf + (32 * wave + 4 * j) * ROW_BYTES),
+                                             16, 0, 0);
         }
     };
 
@@ -308,44 +323,70 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
     float l_i = 0.f;         // this lane's share of the running sum
 
     // LDS read addresses that do not depend on the tile
-    // K: row = 32*blk + l32, logical chunk 2*ks + g
-    const int k_rd_row = l32;
-    // V transpose read: row = T0 + (lane%16)/4, col = 32*db + 16*((lane/16)%2) + 4*(lane%4)
+    // K: row 32*blk + l32, logical chunk 2*ks + g -> physical chunk ^ (row % 16)
+    int k_rd_off[8];
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) k_rd_off[ks] = l32 * ROW_BYTES + (((2 * ks + g) ^ (l32 & 15)) << 4);
+    // V transpose read: row = 16*s + 8*jj + 4*g + rsub (row % 4 == rsub), logical chunk
+    // 4*db + vc -> physical 4*(db ^ rsub) + vc
     const int v_rd_rsub = (lane & 15) >> 2;
-    const int v_rd_chunk = (((lane >> 4) & 1) << 1) + ((lane & 3) >> 1);   // + 4*db
-    const int v_rd_byte = (lane & 1) << 3;
+    const int v_rd_vc = (((lane >> 4) & 1) << 1) + ((lane & 3) >> 1);
+    int v_rd_off[4];
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+        v_rd_off[db] = (4 * g + v_rd_rsub) * ROW_BYTES + ((((db ^ v_rd_rsub) << 2) + v_rd_vc) << 4) + ((lane & 1) << 3);
 
+    // Single K and V buffers, two barriers per tile:
+    //   [own K(it) copies landed] barrier B1 (also: every wave is done with V(it-1))
+    //   issue V(it) copy; fetch gathered ids of tile it+1; S^T = K.Q^T
+    //   [own V(it) copies landed] barrier B2 (also: every wave is done with K(it))
+    //   issue K(it+1) copy; softmax; O^T += V^T.P^T
     Tile cur, nxt;
+    int gt_cur = 0, gt_nxt = 0;
     if (ntiles > 0) {
         cur = tile_at<MODE>(p, ridx, m, nblk, 0);
-        issue_loads(cur);
+        gt_cur = gather_ids(cur);
+        copy_tile(cur, k_base, k_row, std::false_type{}, gt_cur, lds_k);
     }
 
     for (int it = 0; it < ntiles; ++it) {
-        __syncthreads();            // previous tile fully consumed
-        store_lds();
+        __builtin_amdgcn_s_waitcnt(0x0f70);      // vmcnt(0): this wave's part of K(it) is in LDS
         __syncthreads();
-        if (it + 1 < ntiles) {
-            nxt = tile_at<MODE>(p, ridx, m, nblk, it + 1);
-            issue_loads(nxt);
-        }
+        copy_tile(cur, v_base, v_row, std::true_type{}, gt_cur, lds_v);
+        nxt = tile_at<MODE>(p, ridx, m, nblk, min(it + 1, ntiles - 1));
+        gt_nxt = gather_ids(nxt);
 
         if (MODE != MODE_DENSE) __builtin_amdgcn_s_setprio(2);
         // ---- S^T = K . Q^T --------------------------------------------------
         f32x16_t s0, s1;
 #pragma unroll
         for (int r = 0; r < 16; ++r) { s0[r] = 0.f; s1[r] = 0.f; }
+        {
+            // K fragments are fetched QK_AHEAD k-steps before the MFMAs that consume them; the
+            // scheduling fences keep the compiler from sinking the reads back to their use
+            Frag a0[8], a1[8];
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) {
-            const int x = 2 * ks + g;
-            Frag a0, a1;
-            a0.u = *reinterpret_cast<const u32x4_t *>(lds_k + k_rd_row * KP + (x << 4));
-            a1.u = *reinterpret_cast<const u32x4_t *>(lds_k + (32 + k_rd_row) * KP + (x << 4));
-            s0 = Mma<T>::mfma(frag_as<T>(a0), frag_as<T>(qf[ks]), s0);
-            s1 = Mma<T>::mfma(frag_as<T>(a1), frag_as<T>(qf[ks]), s1);
+            for (int ks = 0; ks < QK_AHEAD; ++ks) {
+                a0[ks].u = *reinterpret_cast<const u32x4_t *>(lds_k + k_rd_off[ks]);
+                a1[ks].u = *reinterpret_cast<const u32x4_t *>(lds_k + k_rd_off[ks] + 32 * ROW_BYTES);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks) {
+                if (ks + QK_AHEAD < 8) {
+                    a0[ks + QK_AHEAD].u = *reinterpret_cast<const u32x4_t *>(lds_k + k_rd_off[ks + QK_AHEAD]);
+                    a1[ks + QK_AHEAD].u = *reinterpret_cast<const u32x4_t *>(lds_k + k_rd_off[ks + QK_AHEAD] + 32 * ROW_BYTES);
+                }
+                s0 = Mma<T>::mfma(frag_as<T>(a0[ks]), frag_as<T>(qf[ks]), s0);
+                s1 = Mma<T>::mfma(frag_as<T>(a1[ks]), frag_as<T>(qf[ks]), s1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
-
         if (MODE != MODE_DENSE) __builtin_amdgcn_s_setprio(0);
+        __builtin_amdgcn_s_waitcnt(0x0f70);      // vmcnt(0): this wave's part of V(it) is in LDS
+        __syncthreads();
+        if (it + 1 < ntiles) copy_tile(nxt, k_base, k_row, std::false_type{}, gt_nxt, lds_k);
+
         // ---- mask -----------------------------------------------------------
         // element (blk, r) of this lane is tile-local key tk = tkc + 4*g with the compile-time
         // part tkc = 32*blk + 8*(r/4) + r%4.  keep <=> tk <= hi && (tk > wlo || tk < slim).
@@ -398,16 +439,15 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
         const float alpha = grow ? __builtin_amdgcn_exp2f(m_i - m_use) : 1.0f;
         m_i = m_new;
         float psum = 0.f;
-        float pv[32];
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            pv[r] = __builtin_amdgcn_exp2f(fmaf(s0[r], p.scale_log2, -m_use));
-            pv[16 + r] = __builtin_amdgcn_exp2f(fmaf(s1[r], p.scale_log2, -m_use));
-        }
         Frag pfr[4];
+        {
+            float pv[16];
 #pragma unroll
-        for (int s = 0; s < 4; ++s) { cvt8<T>(&pv[8 * s], pfr[s]); psum += pair_sum<T>(pfr[s]); }
-        l_i = l_i * alpha + psum;
+            for (int r = 0; r < 16; ++r) pv[r] = __builtin_amdgcn_exp2f(fmaf(s0[r], p.scale_log2, -m_use));
+            cvt8<T>(&pv[0], pfr[0]);
+            cvt8<T>(&pv[8], pfr[1]);
+            psum += pair_sum<T>(pfr[0]) + pair_sum<T>(pfr[1]);
+        }
         if (__any(alpha != 1.0f)) {
 #pragma unroll
             for (int i = 0; i < 4; ++i)
@@ -416,25 +456,43 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
         }
 
         if (MODE != MODE_DENSE) __builtin_amdgcn_s_setprio(2);
-        // ---- O^T += V^T . P^T -------------------------------------------------
+        // ---- O^T += V^T . P^T; the exponentials of keys 32..63 run under the MFMAs of keys 0..31,
+        // the V^T fragments of key group s+1 are fetched under the MFMAs of group s ------------
+        {
+            Frag vf[4][4];
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            const Frag &pf = pfr[s];
+            for (int s = 0; s < 4; ++s)
 #pragma unroll
-            for (int db = 0; db < 4; ++db) {
-                Frag vf;
+                for (int db = 0; db < 4; ++db)
 #pragma unroll
-                for (int jj = 0; jj < 2; ++jj) {
-                    const int row = 16 * s + 8 * jj + 4 * g + v_rd_rsub;
-                    const int chunk = (4 * db + v_rd_chunk);
-                    vf.s4[jj] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                        (__attribute__((address_space(3))) short4_t *)(lds_v + row * VP + (chunk << 4) + v_rd_byte));
-                }
-                oacc[db] = Mma<T>::mfma(frag_as<T>(vf), frag_as<T>(pf), oacc[db]);
+                    for (int jj = 0; jj < 2; ++jj)
+                        vf[s][db].s4[jj] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                            (__attribute__((address_space(3))) short4_t *)(lds_v + v_rd_off[db] + (16 * s + 8 * jj) * ROW_BYTES));
+            {
+                float pv[16];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) pv[r] = __builtin_amdgcn_exp2f(fmaf(s1[r], p.scale_log2, -m_use));
+                cvt8<T>(&pv[0], pfr[2]);
+                cvt8<T>(&pv[8], pfr[3]);
+                psum += pair_sum<T>(pfr[2]) + pair_sum<T>(pfr[3]);
+            }
+            l_i = l_i * alpha + psum;
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+#pragma unroll
+                for (int db = 0; db < 4; ++db)
+                    oacc[db] = Mma<T>::mfma(frag_as<T>(vf[s][db]), frag_as<T>(pfr[s]), oacc[db]);
+            __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                if (i < 8) __builtin_amdgcn_sched_group_barrier(VALU_MASK, VALU_PER_MFMA, 0);
+                if (i < 12) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
             }
         }
         if (MODE != MODE_DENSE) __builtin_amdgcn_s_setprio(0);
         cur = nxt;
+        gt_cur = gt_nxt;
     }
 
     // ---- epilogue: O = O^T / l, transposed through LDS so that every global store is 16 bytes
@@ -444,7 +502,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
         const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
         constexpr int OP = ROW_BYTES + 8;                 // pitch: 8-byte lane writes spread over all banks
         __syncthreads();                                  // K/V tiles no longer needed
-        char *ot = lds_k + wave * 32 * OP;                // 32 rows per wave (8448 B <= half of lds_k)
+        char *ot = wave ? lds_v : lds_k;                  // 32 rows per wave (8448 B)
         const bool live = qrow < seqlen;
 #pragma unroll
         for (int db = 0; db < 4; ++db)
@@ -482,6 +540,8 @@ int check_tensors(const minf_qkvo *t) {
         if (((uintptr_t)ptrs[i]) & 15) return MINF_ERR_ALIGNMENT;
         for (int j = 0; j < 3; ++j)
             if (strides[i][j] < 0 || (strides[i][j] & 7)) return MINF_ERR_ALIGNMENT;
+        // 64 rows x token stride is formed in 32 bits inside the tile copies
+        if (strides[i][2] > (1 << 23)) return MINF_ERR_UNSUPPORTED;
     }
     return MINF_OK;
 }
