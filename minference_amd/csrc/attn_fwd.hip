@@ -27,9 +27,9 @@
 //   wait own K(it) copies; barrier (all of K(it) visible, everyone done with V(it-1))
 //   issue V(it) copy; S^T = K.Q^T with the K fragments read two k-steps ahead of their MFMAs
 //   wait own V(it) copies; barrier (all of V(it) visible, everyone done with K(it))
-//   issue K(it+1) copy; row max; exponentials of keys 0..31
-//   O^T += V^T.P^T with the exponentials of keys 32..63 placed behind the first eight MFMAs and
-//   the V^T fragments of key group s+1 read under the MFMAs of group s
+//   read the V^T fragments of keys 0..15; issue K(it+1) copy; row max; exponentials of keys 0..15
+//   O^T += V^T.P^T with the exponentials and the V^T fragment reads of key group s+1 (16 keys)
+//   placed behind the MFMAs of group s
 // The compiler's own schedule read every fragment right before its MFMA (full LDS latency exposed
 // sixteen times per tile); the order above is pinned with sched_barrier / sched_group_barrier.
 //
@@ -65,9 +65,9 @@ constexpr int HD = 128;       // head_dim
 constexpr int NTHREADS = 128; // 2 wavefronts
 constexpr int ROW_BYTES = HD * 2;
 // Scheduling constants (measured on MI355X): K fragments are read QK_AHEAD k-steps ahead of their
-// MFMAs; VALU_PER_MFMA softmax instructions are placed behind each of the first eight PV MFMAs.
+// MFMAs; VALU_PER_MFMA softmax instructions are placed behind each of the first twelve PV MFMAs.
 constexpr int QK_AHEAD = 2;
-constexpr int VALU_PER_MFMA = 5;
+constexpr int VALU_PER_MFMA = 6;
 constexpr int VALU_MASK = 0x402;             // sched_group_barrier classes: VALU | transcendental
 
 struct AttnParams {
@@ -228,7 +228,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
 
     const int tid = (int)threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: keep it in an SGPR
     const int l32 = lane & 31;
     const int g = lane >> 5;
 
@@ -352,6 +352,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
     for (int it = 0; it < ntiles; ++it) {
         __builtin_amdgcn_s_waitcnt(0x0f70);      // vmcnt(0): this wave's part of K(it) is in LDS
         __syncthreads();
+        Frag a0[8], a1[8];
         copy_tile(cur, v_base, v_row, std::true_type{}, gt_cur, lds_v);
         nxt = tile_at<MODE>(p, ridx, m, nblk, min(it + 1, ntiles - 1));
         gt_nxt = gather_ids(nxt);
@@ -364,7 +365,6 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
         {
             // K fragments are fetched QK_AHEAD k-steps before the MFMAs that consume them; the
             // scheduling fences keep the compiler from sinking the reads back to their use
-            Frag a0[8], a1[8];
 #pragma unroll
             for (int ks = 0; ks < QK_AHEAD; ++ks) {
                 a0[ks].u = *reinterpret_cast<const u32x4_t *>(lds_k + k_rd_off[ks]);
@@ -385,6 +385,16 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
         if (MODE != MODE_DENSE) __builtin_amdgcn_s_setprio(0);
         __builtin_amdgcn_s_waitcnt(0x0f70);      // vmcnt(0): this wave's part of V(it) is in LDS
         __syncthreads();
+        // V^T fragments of the first 16 keys: their LDS latency passes under the copy issue and the
+        // row max below
+        Frag vf[4][4];
+#pragma unroll
+        for (int db = 0; db < 4; ++db)
+#pragma unroll
+            for (int jj = 0; jj < 2; ++jj)
+                vf[0][db].s4[jj] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (__attribute__((address_space(3))) short4_t *)(lds_v + v_rd_off[db] + (8 * jj) * ROW_BYTES));
+        __builtin_amdgcn_sched_barrier(0);
         if (it + 1 < ntiles) copy_tile(nxt, k_base, k_row, std::false_type{}, gt_nxt, lds_k);
 
         // ---- mask -----------------------------------------------------------
@@ -426,11 +436,17 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
         }
 
         // ---- online softmax (exp2 domain) -------------------------------------
-        float mx = s0[0];
+        float mx;
+        {
+            float m4[4];                 // four independent chains instead of one of 32 links
 #pragma unroll
-        for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s0[r]);
+            for (int c = 0; c < 4; ++c) {
+                m4[c] = fmaxf(s0[4 * c], s1[4 * c]);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s1[r]);
+                for (int e = 1; e < 4; ++e) m4[c] = fmaxf(m4[c], fmaxf(s0[4 * c + e], s1[4 * c + e]));
+            }
+            mx = fmaxf(fmaxf(m4[0], m4[1]), fmaxf(m4[2], m4[3]));
+        }
         { const unsigned u = __float_as_uint(mx); auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false); mx = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1])); }
         const float cand = mx * p.scale_log2;
         const bool grow = cand > m_i + 8.0f;
@@ -440,14 +456,16 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
         m_i = m_new;
         float psum = 0.f;
         Frag pfr[4];
-        {
-            float pv[16];
+        // probabilities of key group q (16 keys): registers 8*(q%2) .. +7 of s0 (q < 2) / s1
+        auto probs = [&](int q) {
+            const f32x16_t &sx = q < 2 ? s0 : s1;
+            float pv[8];
 #pragma unroll
-            for (int r = 0; r < 16; ++r) pv[r] = __builtin_amdgcn_exp2f(fmaf(s0[r], p.scale_log2, -m_use));
-            cvt8<T>(&pv[0], pfr[0]);
-            cvt8<T>(&pv[8], pfr[1]);
-            psum += pair_sum<T>(pfr[0]) + pair_sum<T>(pfr[1]);
-        }
+            for (int r = 0; r < 8; ++r) pv[r] = __builtin_amdgcn_exp2f(fmaf(sx[8 * (q & 1) + r], p.scale_log2, -m_use));
+            cvt8<T>(&pv[0], pfr[q]);
+            psum += pair_sum<T>(pfr[q]);
+        };
+        probs(0);
         if (__any(alpha != 1.0f)) {
 #pragma unroll
             for (int i = 0; i < 4; ++i)
@@ -456,37 +474,30 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
         }
 
         if (MODE != MODE_DENSE) __builtin_amdgcn_s_setprio(2);
-        // ---- O^T += V^T . P^T; the exponentials of keys 32..63 run under the MFMAs of keys 0..31,
-        // the V^T fragments of key group s+1 are fetched under the MFMAs of group s ------------
+        // ---- O^T += V^T . P^T; the exponentials of key group q+1 run under the MFMAs of group q,
+        // the V^T fragments of group q+1 are fetched under them as well ------------------------
         {
-            Frag vf[4][4];
 #pragma unroll
-            for (int s = 0; s < 4; ++s)
+            for (int s = 1; s < 4; ++s)
 #pragma unroll
                 for (int db = 0; db < 4; ++db)
 #pragma unroll
                     for (int jj = 0; jj < 2; ++jj)
                         vf[s][db].s4[jj] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
                             (__attribute__((address_space(3))) short4_t *)(lds_v + v_rd_off[db] + (16 * s + 8 * jj) * ROW_BYTES));
-            {
-                float pv[16];
-#pragma unroll
-                for (int r = 0; r < 16; ++r) pv[r] = __builtin_amdgcn_exp2f(fmaf(s1[r], p.scale_log2, -m_use));
-                cvt8<T>(&pv[0], pfr[2]);
-                cvt8<T>(&pv[8], pfr[3]);
-                psum += pair_sum<T>(pfr[2]) + pair_sum<T>(pfr[3]);
-            }
+            probs(1);
+            probs(2);
+            probs(3);
             l_i = l_i * alpha + psum;
 #pragma unroll
             for (int s = 0; s < 4; ++s)
 #pragma unroll
                 for (int db = 0; db < 4; ++db)
                     oacc[db] = Mma<T>::mfma(frag_as<T>(vf[s][db]), frag_as<T>(pfr[s]), oacc[db]);
-            __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                if (i < 8) __builtin_amdgcn_sched_group_barrier(VALU_MASK, VALU_PER_MFMA, 0);
+                if (i < 12) __builtin_amdgcn_sched_group_barrier(VALU_MASK, VALU_PER_MFMA, 0);
                 if (i < 12) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
             }
         }
