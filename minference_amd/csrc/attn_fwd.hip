@@ -41,7 +41,7 @@
 //    below 2^8, far inside fp32/bf16 range), so most tiles skip the O^T rescale;
 //  * the cross-half max uses v_permlane32_swap, the row sums v_dot2 on the rounded probabilities
 //    (the same values the second MFMA consumes);
-//  * s_setprio raises the wave while it issues MFMAs (not in dense mode);
+//  * s_setprio raises the wave while it issues MFMAs;
 //  * the epilogue transposes O^T through LDS so each global store is 16 B of one 256-byte row.
 #include "minf_common.h"
 #include <math.h>
@@ -300,11 +300,24 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
             }
             return;
         }
+        // three straight-line variants (a per-row select would turn into sixteen tiny branches)
+        if (gathered) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int r = 32 * wave + 4 * j + cp_r;          // tile row
+                const int tk = max(0, min(__shfl(idv, r), seqlen - 1));
+                const int c = is_v ? (cp_c ^ ((r & 3) << 2)) : (cp_c ^ (r & 15));
+                const char *gp = base + tk * rowstride + c * 16;
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
+                                                 (__attribute__((address_space(3))) void *)(ldsbuf + (32 * wave + 4 * j) * ROW_BYTES),
+                                                 16, 0, 0);
+            }
+            return;
+        }
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            const int r = 32 * wave + 4 * j + cp_r;          // tile row
-            const int tok = gathered ? __shfl(idv, r) : t.start + r;
-            const int tk = max(0, min(tok, seqlen - 1));
+            const int r = 32 * wave + 4 * j + cp_r;
+            const int tk = max(0, min(t.start + r, seqlen - 1));
             const int c = is_v ? (cp_c ^ ((r & 3) << 2)) : (cp_c ^ (r & 15));
             const char *gp = base + tk * rowstride + c * 16;
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
@@ -357,7 +370,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
         nxt = tile_at<MODE>(p, ridx, m, nblk, min(it + 1, ntiles - 1));
         gt_nxt = gather_ids(nxt);
 
-        if (MODE != MODE_DENSE) __builtin_amdgcn_s_setprio(2);
+        __builtin_amdgcn_s_setprio(2);
         // ---- S^T = K . Q^T --------------------------------------------------
         f32x16_t s0, s1;
 #pragma unroll
@@ -382,7 +395,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
-        if (MODE != MODE_DENSE) __builtin_amdgcn_s_setprio(0);
+        __builtin_amdgcn_s_setprio(0);
         __builtin_amdgcn_s_waitcnt(0x0f70);      // vmcnt(0): this wave's part of V(it) is in LDS
         __syncthreads();
         // V^T fragments of the first 16 keys: their LDS latency passes under the copy issue and the
@@ -473,7 +486,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
                 for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
         }
 
-        if (MODE != MODE_DENSE) __builtin_amdgcn_s_setprio(2);
+        __builtin_amdgcn_s_setprio(2);
         // ---- O^T += V^T . P^T; the exponentials of key group q+1 run under the MFMAs of group q,
         // the V^T fragments of group q+1 are fetched under them as well ------------------------
         {
@@ -501,7 +514,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
                 if (i < 12) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
             }
         }
-        if (MODE != MODE_DENSE) __builtin_amdgcn_s_setprio(0);
+        __builtin_amdgcn_s_setprio(0);
         cur = nxt;
         gt_cur = gt_nxt;
     }
