@@ -181,7 +181,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU only: this build has no multi-GPU path "
-              "(heads shard across GPUs with no exchange; see DESIGN.md). Use --gpus 1.", file=sys.stderr)
+              "(every stage is per head, so heads would shard across GPUs with no exchange). Use --gpus 1.", file=sys.stderr)
         sys.exit(2)
 
     import torch
