@@ -73,11 +73,20 @@ __global__ __launch_bounds__(TK_THREADS) void topk_kernel(const TopkProblem p0, 
             const unsigned u = order_key(xv);
             if ((u & mask) == prefix) atomicAdd(&hist[(((u >> shift) & 255u) << 5) + (lane & 31)], 1u);
         };
-        for (int i = tid; i < nvec; i += TK_THREADS) {       // 16-byte loads over the aligned part
+        // 16-byte loads over the aligned part, four in flight per thread
+        int i = tid;
+        for (; i + 3 * TK_THREADS < nvec; i += 4 * TK_THREADS) {
+            float4 q[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) q[u] = reinterpret_cast<const float4 *>(x)[i + u * TK_THREADS];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) { tally(q[u].x); tally(q[u].y); tally(q[u].z); tally(q[u].w); }
+        }
+        for (; i < nvec; i += TK_THREADS) {
             const float4 q = reinterpret_cast<const float4 *>(x)[i];
             tally(q.x); tally(q.y); tally(q.z); tally(q.w);
         }
-        for (int i = nvec * 4 + tid; i < n; i += TK_THREADS) tally(x[i]);
+        for (int j = nvec * 4 + tid; j < n; j += TK_THREADS) tally(x[j]);
         __syncthreads();
         if (tid < 256) {                 // fold the 32 copies of bin `tid` (rotated: one bank per thread)
             unsigned sum = 0;
