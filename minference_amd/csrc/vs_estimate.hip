@@ -11,7 +11,7 @@
 // registers serve as A or B operand, so swapping the operands transposes the
 // score tile for free):
 //   stats  : S^T = K.Q^T  -> lane <-> query row: running max / sum-of-exp in
-//            registers, one (max, sum) pair per row per 1024-key chunk;
+//            registers, one (max, sum) pair per row per 2048-key chunk;
 //   reduce : combine the chunk pairs into M_i = max_i + log2(sum_i);
 //   scores : S = Q.K^T    -> lane <-> key: p = exp2(s - M_row); column sums are
 //            in-lane adds (+ one cross-half shuffle); for the diagonal sums each wave parks
@@ -32,7 +32,7 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
 typedef __attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned u32x4_t;
 
 constexpr int LQ = 64;          // query rows held per head (last_q <= LQ)
-constexpr int KC = 1024;        // keys per workgroup
+constexpr int KC = 2048;        // keys per workgroup
 constexpr int EST_THREADS = 256;
 constexpr int WIN = KC + LQ;    // diagonal window of one chunk
 constexpr int HD = 128;
@@ -218,7 +218,7 @@ __global__ __launch_bounds__(LQ) void est_reduce_kernel(const EstParams p) {
 // private per-wave window with plain read-modify-write (one wave, in-order LDS: no race).
 constexpr int TP = 33;                       // tile row pitch (floats)
 constexpr int TROWS = 94;                    // 32 rows of a half block, 31 zero rows above, 31 below
-constexpr int WWIN = KC / 4 + LQ;            // per-wave diagonal window (256 keys + 64)
+constexpr int WWIN = KC / 4 + LQ;            // per-wave diagonal window (a quarter of the chunk + 64)
 
 // (min 2 waves per SIMD: caps the kernel at 256 registers; it is latency bound and one resident
 // wave per SIMD ran 1.4x slower)
