@@ -319,9 +319,15 @@ __global__ __launch_bounds__(IDX_WAVES *MINF_WAVE) void vs_index_fast_kernel(
     int nb = 0, ncol = 0;
     bool live = start_m < seqlen;
 
+    // loads that do not depend on each other, issued together (the kernel is bound by chains of
+    // dependent loads, not by bandwidth)
+    const int o_first = sl[0], o_last = sl[nnz_s - 1];
+    const int tab_blocks = hdr[0], tab_runs = hdr[1], tab_v = hdr[2];
+    const bool whole_list = o_first <= end_m - 64;      // nothing skipped, nothing clipped
+
     int s0 = nnz_s;
     if (live) {
-        int lo = 0, hi = nnz_s;
+        int lo = 0, hi = whole_list ? 0 : nnz_s;        // first entry with an offset below end_m
         while (lo < hi) {
             int mid = (lo + hi) >> 1;
             if (sl[mid] >= end_m) lo = mid + 1; else hi = mid;
@@ -337,7 +343,7 @@ __global__ __launch_bounds__(IDX_WAVES *MINF_WAVE) void vs_index_fast_kernel(
         int vp = 0;
         int g = -1;                  // list entry from which the tables apply
         int e_lim = INT_MIN;         // end of the last explicitly built range
-        if (s0 == 0 && end_m - sl[0] >= 64) {
+        if (whole_list) {
             g = 0;
         } else {
             const int n = nnz_s - s0;
@@ -424,12 +430,13 @@ __global__ __launch_bounds__(IDX_WAVES *MINF_WAVE) void vs_index_fast_kernel(
             }
         }
         if (g >= 0) {
-            const int shift = end_m - hdr[2];
-            const int k0 = cpre[g], r0 = crun[g];
-            const int nblk = hdr[0] - k0, nruns = hdr[1];
+            const int shift = end_m - tab_v;
+            const int k0 = g == 0 ? 0 : cpre[g], r0 = g == 0 ? 0 : crun[g];   // entry 0 starts range 0
+            const int nblk = tab_blocks - k0, nruns = tab_runs;
             for (int k = lane; k < nblk; k += MINF_WAVE) bo_row[nb + k] = cpos[k0 + k] + shift;
             nb += nblk;
-            const int t_end = end_m - sl[nnz_s - 1];      // t of the last entry (not clipped here)
+            const int t_end = end_m - o_last;             // t of the last entry (not clipped here)
+            const int first_a = run_a[r0];                // start of the first remaining range
             while (vp < nnz_v) {
                 const int x = (vp + lane < nnz_v) ? vert[vp + lane] : INT_MAX;
                 const bool ok = x < t_end;
@@ -437,12 +444,16 @@ __global__ __launch_bounds__(IDX_WAVES *MINF_WAVE) void vs_index_fast_kernel(
                 bool emit = false;
                 if (ok && x >= e_lim) {
                     const int xv = x - shift;
-                    int lo = r0, hi = nruns;                  // first range >= r0 that ends after xv
-                    while (lo < hi) {
-                        int mid = (lo + hi) >> 1;
-                        if (run_e[mid] > xv) hi = mid; else lo = mid + 1;
+                    if (xv < first_a) {                       // below every remaining range: no search
+                        emit = true;
+                    } else {
+                        int lo = r0, hi = nruns;              // first range >= r0 that ends after xv
+                        while (lo < hi) {
+                            int mid = (lo + hi) >> 1;
+                            if (run_e[mid] > xv) hi = mid; else lo = mid + 1;
+                        }
+                        emit = !(lo < nruns && run_a[lo] <= xv);
                     }
-                    emit = !(lo < nruns && run_a[lo] <= xv);
                 }
                 const uint64_t em = __ballot(emit);
                 if (emit) ci_row[ncol + __builtin_popcountll(em & lt)] = x;
