@@ -218,32 +218,61 @@ __global__ __launch_bounds__(TKW_WAVES * 64) void topk_wave_kernel(const TopkPro
         const int i = j * 64 + lane;
         key[j] = i < n ? order_key(x[i]) : 0u;      // padding sorts below every real score
     }
+    // Rows with a masked (-inf) tail, e.g. block-causal score rows: when at least k entries are above
+    // -inf, the threshold is too, and register groups that hold nothing above -inf can be skipped
+    // in every pass and in the emit (they add nothing to a count of keys >= cand > key(-inf), and
+    // for cand <= key(-inf) the live groups alone already reach k).
+    constexpr unsigned KEY_FLOOR = 0x007fffffu;          // order_key(-inf)
+    constexpr int GROUP = ITEMS >= 8 ? 8 : ITEMS;
+    int nfin = 0, jmax = 0;
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) {
+        const int c = __builtin_popcountll(__ballot(key[j] > KEY_FLOOR));
+        nfin += c;
+        if (c) jmax = j + 1;
+    }
+    if (nfin < k) jmax = ITEMS;
     unsigned T = 0;
     for (int bit = 31; bit >= 0; --bit) {
         const unsigned cand = T | (1u << bit);
         int cnt = 0;
 #pragma unroll
-        for (int j = 0; j < ITEMS; ++j) cnt += __builtin_popcountll(__ballot(key[j] >= cand));
+        for (int jb = 0; jb < ITEMS; jb += GROUP) {
+            if (jb < jmax) {
+#pragma unroll
+                for (int j = jb; j < jb + GROUP; ++j) cnt += __builtin_popcountll(__ballot(key[j] >= cand));
+            }
+        }
         if (cnt >= k) T = cand;
     }
     int cgt = 0;
 #pragma unroll
-    for (int j = 0; j < ITEMS; ++j) cgt += __builtin_popcountll(__ballot(key[j] > T));
+    for (int jb = 0; jb < ITEMS; jb += GROUP) {
+        if (jb < jmax) {
+#pragma unroll
+            for (int j = jb; j < jb + GROUP; ++j) cgt += __builtin_popcountll(__ballot(key[j] > T));
+        }
+    }
     const int r = k - cgt;                           // entries equal to T that are taken, lowest index first
     int gt_before = 0, eq_before = 0;
     const uint64_t lt = minf_lanemask_lt();
 #pragma unroll
-    for (int j = 0; j < ITEMS; ++j) {
-        const int i = j * 64 + lane;
-        const bool gt = key[j] > T, eq = key[j] == T;
-        const uint64_t mg = __ballot(gt), me = __ballot(eq);
-        const int e_here = eq_before + __builtin_popcountll(me & lt);
-        if (gt || (eq && e_here < r)) {
-            const int pos = gt_before + __builtin_popcountll(mg & lt) + min(e_here, r);
-            o[pos] = reverse_base >= 0 ? reverse_base - i : i;
+    for (int jb = 0; jb < ITEMS; jb += GROUP) {
+        if (jb < jmax) {
+#pragma unroll
+            for (int j = jb; j < jb + GROUP; ++j) {
+                const int i = j * 64 + lane;
+                const bool gt = key[j] > T, eq = key[j] == T;
+                const uint64_t mg = __ballot(gt), me = __ballot(eq);
+                const int e_here = eq_before + __builtin_popcountll(me & lt);
+                if (gt || (eq && e_here < r)) {
+                    const int pos = gt_before + __builtin_popcountll(mg & lt) + min(e_here, r);
+                    o[pos] = reverse_base >= 0 ? reverse_base - i : i;
+                }
+                gt_before += __builtin_popcountll(mg);
+                eq_before += __builtin_popcountll(me);
+            }
         }
-        gt_before += __builtin_popcountll(mg);
-        eq_before += __builtin_popcountll(me);
     }
 }
 
