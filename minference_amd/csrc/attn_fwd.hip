@@ -3,7 +3,8 @@
 // A-shape ranges, dense causal).
 //
 // Work split: one workgroup (2 wavefronts) per (batch, query head, 64-row
-// block); each wavefront owns 32 query rows.  Everything is computed in the
+// block); each wavefront owns 32 query rows.  Dense and A-shape / tri-shape launches use the
+// paired variant: 4 wavefronts over two neighbouring row blocks that share every K/V tile copy.  Everything is computed in the
 // TRANSPOSED orientation so that softmax statistics are per lane:
 //
 //   S^T[token][qrow] = K_tile . Q^T      v_mfma_f32_32x32x16 (A = K from LDS, B = Q in VGPRs)
@@ -62,7 +63,7 @@ enum { MODE_VS = 0, MODE_BS = 1, MODE_ASHAPE = 2, MODE_DENSE = 3 };
 constexpr int BM = 64;        // query rows per workgroup
 constexpr int BN = 64;        // keys per tile
 constexpr int HD = 128;       // head_dim
-constexpr int NTHREADS = 128; // 2 wavefronts
+constexpr int NTHREADS = 128; // 2 wavefronts per 64-row block (x2 in the paired variant)
 constexpr int ROW_BYTES = HD * 2;
 // Scheduling constants (measured on MI355X): K fragments are read QK_AHEAD k-steps ahead of their
 // MFMAs; VALU_PER_MFMA softmax instructions are placed behind each of the first twelve PV MFMAs.
@@ -201,8 +202,45 @@ __device__ __forceinline__ Tile tile_at(const AttnParams &p, long long ridx, int
     return t;
 }
 
-template <typename T, int MODE>
-__global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams p) {
+// Paired variant (dense causal and A-shape / tri-shape, whose tile lists are analytic): one
+// workgroup of 4 waves covers the row blocks mA = 2*mp and mB = mA + 1.  Their tile lists differ
+// by at most the ends, so the workgroup walks the union once and every K/V tile is copied into LDS
+// once for 128 query rows; a half skips the tiles that are not on its own list.
+template <int MODE>
+__device__ __forceinline__ int pair_tile_count(const AttnParams &p, int mA, int mB, int &nblk) {
+    if (MODE == MODE_DENSE || mB * BM + BM - 1 >= p.dense_from) {
+        nblk = mB + 1;
+        return nblk;
+    }
+    int lo_key = mA * BM - p.n_local + 1;
+    int t_lo = lo_key > 0 ? (lo_key >> 6) : 0;
+    int sink_tiles = (p.n_init + BN - 1) >> 6;
+    nblk = min(sink_tiles, t_lo);
+    return nblk + (mB - t_lo + 1);
+}
+template <int MODE>
+__device__ __forceinline__ int pair_tile_start(const AttnParams &p, int mA, int mB, int nblk, int it) {
+    if (MODE == MODE_DENSE || mB * BM + BM - 1 >= p.dense_from) return it * BN;
+    int lo_key = mA * BM - p.n_local + 1;
+    int t_lo = lo_key > 0 ? (lo_key >> 6) : 0;
+    return (it < nblk ? it : t_lo + (it - nblk)) * BN;
+}
+// is the tile that starts at key `start` on the list of row block m ?
+template <int MODE>
+__device__ __forceinline__ bool tile_on_list(const AttnParams &p, int m, int start) {
+    const int ti = start >> 6;
+    if (ti > m) return false;
+    if (MODE == MODE_DENSE || m * BM + BM - 1 >= p.dense_from) return true;
+    int lo_key = m * BM - p.n_local + 1;
+    int t_lo = lo_key > 0 ? (lo_key >> 6) : 0;
+    return ti >= t_lo || ti < ((p.n_init + BN - 1) >> 6);
+}
+
+template <typename T, int MODE, bool PAIR>
+__global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_kernel(const AttnParams p) {
+    static_assert(!PAIR || MODE == MODE_DENSE || MODE == MODE_ASHAPE, "paired variant: analytic tile lists only");
+    constexpr int NT = PAIR ? 2 * NTHREADS : NTHREADS;      // threads per workgroup
+    constexpr int CROWS = PAIR ? 16 : 32;                   // tile rows copied by one wave
     // two separate LDS objects: the compiler then lets reads of one overtake copies into the other
     __shared__ __attribute__((aligned(16))) char lds_k[BN * ROW_BYTES];
     __shared__ __attribute__((aligned(16))) char lds_v[BN * ROW_BYTES];
@@ -220,15 +258,20 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
     const int hin = (int)(rest % group); rest /= group;
     // Dense causal work grows with the row block, so the heavy (late) blocks go first; the sparse
     // modes have near-constant work per row block and measure faster in ascending order.
-    const int mi = (int)(rest % p.rows); rest /= p.rows;
-    const int m = MODE == MODE_DENSE ? p.rows - 1 - mi : mi;
+    const int rows_wg = PAIR ? (p.rows + 1) >> 1 : p.rows;           // row-block slots per (batch, head)
+    const int mi = (int)(rest % rows_wg); rest /= rows_wg;
+    const int mslot = MODE == MODE_DENSE ? rows_wg - 1 - mi : mi;
     const int hkv = (int)(rest % p.hk);
     const int b = (int)(rest / p.hk);
     const int h = hkv * group + hin;
 
     const int tid = (int)threadIdx.x;
     const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: keep it in an SGPR
+    const int wave_wg = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: keep it in an SGPR
+    const int half = PAIR ? wave_wg >> 1 : 0;                        // which row block of the pair
+    const int wave = PAIR ? wave_wg & 1 : wave_wg;                   // wave inside the row block
+    const int m = PAIR ? 2 * mslot + half : mslot;
+    const int mA = PAIR ? 2 * mslot : mslot, mB = PAIR ? min(mA + 1, p.rows - 1) : mslot;
     const int l32 = lane & 31;
     const int g = lane >> 5;
 
@@ -237,26 +280,29 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
     const int qrow = row0 + wave * 32 + l32;          // this lane's query row
     char *o_base = p.o + ((long long)b * p.os[0] + (long long)h * p.os[1]) * 2;
 
-    if (row0 >= seqlen) {
-        // row block past the sequence: zeros (16 B per lane-step)
-        for (int i = tid; i < BM * 16; i += NTHREADS) {
-            int r = row0 + (i >> 4);
-            if (r < p.n) *reinterpret_cast<u32x4_t *>(o_base + (long long)r * p.os[2] * 2 + (i & 15) * 16) = u32x4_t{0u, 0u, 0u, 0u};
-        }
-        return;
+    // row block past the sequence: zeros (16 B per lane-step); in the paired variant the other
+    // half may still have work, so this half stays for the copies and barriers without tiles
+    const bool have_rows = m < p.rows && row0 < seqlen;
+    if (!have_rows) {
+        if (m < p.rows)
+            for (int i = tid & (NTHREADS - 1); i < BM * 16; i += NTHREADS) {
+                int r = row0 + (i >> 4);
+                if (r < p.n) *reinterpret_cast<u32x4_t *>(o_base + (long long)r * p.os[2] * 2 + (i & 15) * 16) = u32x4_t{0u, 0u, 0u, 0u};
+            }
+        if (!PAIR || mA * BM >= seqlen) return;      // (wave-uniform; for a pair: both halves are past)
     }
 
     const char *q_base = p.q + ((long long)b * p.qs[0] + (long long)h * p.qs[1]) * 2;
     const char *k_base = p.k + ((long long)b * p.ks[0] + (long long)hkv * p.ks[1]) * 2;
     const char *v_base = p.v + ((long long)b * p.vs[0] + (long long)hkv * p.vs[1]) * 2;
     const long long k_row = p.ks[2] * 2, v_row = p.vs[2] * 2;
-    const long long ridx = ((long long)b * p.hq + h) * p.rows + m;
+    const long long ridx = ((long long)b * p.hq + h) * p.rows + min(m, p.rows - 1);
 
     // ---- Q fragments (B operand of S^T): row qrow, d = 16*ks + 8*g + 0..7 ----
     Frag qf[8];
     {
         const bool ok = qrow < seqlen;
-        const char *qp = q_base + (long long)(ok ? qrow : row0) * p.qs[2] * 2 + g * 16;
+        const char *qp = q_base + (long long)(ok ? qrow : min(row0, seqlen - 1)) * p.qs[2] * 2 + g * 16;
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) {
             qf[ks].u = *reinterpret_cast<const u32x4_t *>(qp + ks * 32);
@@ -265,12 +311,23 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
     }
 
     int nblk = 0;
-    const int ntiles = tile_count<MODE>(p, ridx, m, nblk);
+    const int ntiles = PAIR ? pair_tile_count<MODE>(p, mA, mB, nblk) : tile_count<MODE>(p, ridx, m, nblk);
+    auto tile_of = [&](int it) -> Tile {
+        if constexpr (PAIR) {
+            Tile t;
+            t.gathered = 0;
+            t.nvalid = BN;
+            t.start = pair_tile_start<MODE>(p, mA, mB, nblk, it);
+            return t;
+        } else {
+            return tile_at<MODE>(p, ridx, m, nblk, it);
+        }
+    };
 
     // ---- global -> LDS copies without a register round trip (global_load_lds_dwordx4): every lane
     // fetches 16 bytes from its own global address and the wave's 64 x 16 B land contiguously in
     // LDS at a wave-uniform base (lane i -> base + 16*i), i.e. one instruction fills 4 tile rows;
-    // wave w owns rows 32*w .. 32*w+31 (8 instructions per matrix).  The 16-byte chunks of a row
+    // wave w owns rows 32*w .. 32*w+31 (8 instructions per matrix; 16 rows, 4 instructions when paired).  The 16-byte chunks of a row
     // are permuted for conflict-free reads (K: chunk ^ row%16, V: chunk ^ 4*(row%4)); the
     // permutation is applied on the global side: lane (row, c') loads global chunk c' ^ swz(row).
     // Rows that do not exist (past seqlen, or padding of a gathered tile) are read from a clamped,
@@ -290,12 +347,12 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
         if (!gathered && t.start >= 0 && t.start + BN <= seqlen) {
             const char *tb = base + (long long)t.start * rowstride;      // wave-uniform
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const int r = 32 * wave + 4 * j + cp_r;
+            for (int j = 0; j < CROWS / 4; ++j) {
+                const int r = CROWS * wave_wg + 4 * j + cp_r;
                 const int c = is_v ? (cp_c ^ ((r & 3) << 2)) : (cp_c ^ (r & 15));
                 const char *gp = tb + (unsigned)(r * (int)rowstride + c * 16);
                 __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
-                                                 (__attribute__((address_space(3))) void *)(ldsbuf + (32 * wave + 4 * j) * ROW_BYTES),
+                                                 (__attribute__((address_space(3))) void *)(ldsbuf + (CROWS * wave_wg + 4 * j) * ROW_BYTES),
                                                  16, 0, 0);
             }
             return;
@@ -303,25 +360,25 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
         // three straight-line variants (a per-row select would turn into sixteen tiny branches)
         if (gathered) {
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const int r = 32 * wave + 4 * j + cp_r;          // tile row
+            for (int j = 0; j < CROWS / 4; ++j) {
+                const int r = CROWS * wave_wg + 4 * j + cp_r;          // tile row
                 const int tk = max(0, min(__shfl(idv, r), seqlen - 1));
                 const int c = is_v ? (cp_c ^ ((r & 3) << 2)) : (cp_c ^ (r & 15));
                 const char *gp = base + tk * rowstride + c * 16;
                 __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
-                                                 (__attribute__((address_space(3))) void *)(ldsbuf + (32 * wave + 4 * j) * ROW_BYTES),
+                                                 (__attribute__((address_space(3))) void *)(ldsbuf + (CROWS * wave_wg + 4 * j) * ROW_BYTES),
                                                  16, 0, 0);
             }
             return;
         }
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const int r = 32 * wave + 4 * j + cp_r;
+        for (int j = 0; j < CROWS / 4; ++j) {
+            const int r = CROWS * wave_wg + 4 * j + cp_r;
             const int tk = max(0, min(t.start + r, seqlen - 1));
             const int c = is_v ? (cp_c ^ ((r & 3) << 2)) : (cp_c ^ (r & 15));
             const char *gp = base + tk * rowstride + c * 16;
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
-                                             (__attribute__((address_space(3))) void *)(ldsbuf + (32 * wave + 4 * j) * ROW_BYTES),
+                                             (__attribute__((address_space(3))) void *)(ldsbuf + (CROWS * wave_wg + 4 * j) * ROW_BYTES),
                                              16, 0, 0);
         }
     };
@@ -357,7 +414,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
     Tile cur, nxt;
     int gt_cur = 0, gt_nxt = 0;
     if (ntiles > 0) {
-        cur = tile_at<MODE>(p, ridx, m, nblk, 0);
+        cur = tile_of(0);
         gt_cur = gather_ids(cur);
         copy_tile(cur, k_base, k_row, std::false_type{}, gt_cur, lds_k);
     }
@@ -367,12 +424,15 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
         __syncthreads();
         Frag a0[8], a1[8];
         copy_tile(cur, v_base, v_row, std::true_type{}, gt_cur, lds_v);
-        nxt = tile_at<MODE>(p, ridx, m, nblk, min(it + 1, ntiles - 1));
+        nxt = tile_of(min(it + 1, ntiles - 1));
         gt_nxt = gather_ids(nxt);
 
+        // paired variant: is this tile on the list of this wave's row block ?
+        const bool active = !PAIR || (have_rows && tile_on_list<MODE>(p, m, cur.start));
+        f32x16_t s0, s1;
+        if (active) {
         __builtin_amdgcn_s_setprio(2);
         // ---- S^T = K . Q^T --------------------------------------------------
-        f32x16_t s0, s1;
 #pragma unroll
         for (int r = 0; r < 16; ++r) { s0[r] = 0.f; s1[r] = 0.f; }
         {
@@ -396,11 +456,13 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
             }
         }
         __builtin_amdgcn_s_setprio(0);
+        }
         __builtin_amdgcn_s_waitcnt(0x0f70);      // vmcnt(0): this wave's part of V(it) is in LDS
         __syncthreads();
         // V^T fragments of the first 16 keys: their LDS latency passes under the copy issue and the
         // row max below
         Frag vf[4][4];
+        if (active) {
 #pragma unroll
         for (int db = 0; db < 4; ++db)
 #pragma unroll
@@ -408,7 +470,9 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
                 vf[0][db].s4[jj] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
                     (__attribute__((address_space(3))) short4_t *)(lds_v + v_rd_off[db] + (8 * jj) * ROW_BYTES));
         __builtin_amdgcn_sched_barrier(0);
+        }
         if (it + 1 < ntiles) copy_tile(nxt, k_base, k_row, std::false_type{}, gt_nxt, lds_k);
+        if (active) {
 
         // ---- mask -----------------------------------------------------------
         // element (blk, r) of this lane is tile-local key tk = tkc + 4*g with the compile-time
@@ -515,6 +579,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
             }
         }
         __builtin_amdgcn_s_setprio(0);
+        }
         cur = nxt;
         gt_cur = gt_nxt;
     }
@@ -524,9 +589,10 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
     {
         float l_tot = l_i + __shfl_xor(l_i, 32);
         const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
-        constexpr int OP = ROW_BYTES + 8;                 // pitch: 8-byte lane writes spread over all banks
+        // pitch: 8-byte lane writes spread over all banks (four waves only fit without the pad)
+        constexpr int OP = PAIR ? ROW_BYTES : ROW_BYTES + 8;
         __syncthreads();                                  // K/V tiles no longer needed
-        char *ot = wave ? lds_v : lds_k;                  // 32 rows per wave (8448 B)
+        char *ot = PAIR ? (half ? lds_v : lds_k) + wave * 32 * OP : (wave ? lds_v : lds_k);   // 32 rows per wave
         const bool live = qrow < seqlen;
 #pragma unroll
         for (int db = 0; db < 4; ++db)
@@ -544,7 +610,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_fwd_kernel(const AttnParams 
             const int r = 4 * i + (lane >> 4);
             const int grow = row0 + wave * 32 + r;
             const u32x4_t val = *reinterpret_cast<const u32x4_t *>(ot + r * OP + (lane & 15) * 16);
-            if (grow < p.n) *reinterpret_cast<u32x4_t *>(o_base + (long long)grow * p.os[2] * 2 + (lane & 15) * 16) = val;
+            if (grow < p.n && have_rows) *reinterpret_cast<u32x4_t *>(o_base + (long long)grow * p.os[2] * 2 + (lane & 15) * 16) = val;
         }
     }
 }
@@ -586,16 +652,19 @@ void fill_params(AttnParams &p, const minf_qkvo *t) {
     p.total_wg = (long long)t->batch * t->heads_q * p.rows;
 }
 
-template <int MODE> int launch(const AttnParams &p, int dtype, void *stream) {
+template <int MODE> int launch(AttnParams p, int dtype, void *stream) {
     if (p.total_wg == 0) return MINF_OK;
+    constexpr bool PAIR = MODE == MODE_DENSE || MODE == MODE_ASHAPE;
+    if (PAIR) p.total_wg = (long long)p.batch * p.hq * ((p.rows + 1) / 2);
     const long long per_xcd = (p.total_wg + 7) >> 3;
     const long long grid = per_xcd * 8;
     if (grid > 0x7fffffffLL) return MINF_ERR_UNSUPPORTED;
+    const dim3 block(PAIR ? 2 * NTHREADS : NTHREADS);
     if (dtype == MINF_BF16)
-        hipLaunchKernelGGL((attn_fwd_kernel<__bf16, MODE>), dim3((unsigned)grid), dim3(NTHREADS), 0,
+        hipLaunchKernelGGL((attn_fwd_kernel<__bf16, MODE, PAIR>), dim3((unsigned)grid), block, 0,
                            (hipStream_t)stream, p);
     else
-        hipLaunchKernelGGL((attn_fwd_kernel<_Float16, MODE>), dim3((unsigned)grid), dim3(NTHREADS), 0,
+        hipLaunchKernelGGL((attn_fwd_kernel<_Float16, MODE, PAIR>), dim3((unsigned)grid), block, 0,
                            (hipStream_t)stream, p);
     return minf_launch_status();
 }
