@@ -4,8 +4,8 @@
 //
 // Work split: one workgroup (2 wavefronts) per (batch, query head, 64-row
 // block); each wavefront owns 32 query rows.  Dense and A-shape / tri-shape launches use the
-// paired variant: 4 wavefronts over two neighbouring row blocks that share every K/V tile copy.  Everything is computed in the
-// TRANSPOSED orientation so that softmax statistics are per lane:
+// paired variant: 4 wavefronts over two neighbouring row blocks that share every K/V tile copy.
+// Everything is computed in the TRANSPOSED orientation so that softmax statistics are per lane:
 //
 //   S^T[token][qrow] = K_tile . Q^T      v_mfma_f32_32x32x16 (A = K from LDS, B = Q in VGPRs)
 //   O^T[d][qrow]    += V_tile^T . P^T    (A = V^T via ds_read_b64_tr_b16, B = P straight from
