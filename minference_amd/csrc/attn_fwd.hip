@@ -150,7 +150,9 @@ struct Tile {
     int start;          // first token (contiguous) / first list position (gathered)
     int gathered;       // 0/1
     int nvalid;         // gathered: number of valid list entries in this tile
+    int on_a, on_b;     // paired block-sparse walk: is the tile on the list of row block A / B
 };
+constexpr int BS_PAIR_MAX = 512;   // longest block list the paired block-sparse walk keeps in LDS
 
 template <int MODE>
 __device__ __forceinline__ int tile_count(const AttnParams &p, long long ridx, int m, int &nblk) {
@@ -238,7 +240,7 @@ __device__ __forceinline__ bool tile_on_list(const AttnParams &p, int m, int sta
 
 template <typename T, int MODE, bool PAIR>
 __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_kernel(const AttnParams p) {
-    static_assert(!PAIR || MODE == MODE_DENSE || MODE == MODE_ASHAPE, "paired variant: analytic tile lists only");
+    static_assert(!PAIR || MODE != MODE_VS, "paired variant: no vertical-slash lists");
     constexpr int NT = PAIR ? 2 * NTHREADS : NTHREADS;      // threads per workgroup
     constexpr int CROWS = PAIR ? 16 : 32;                   // tile rows copied by one wave
     // two separate LDS objects: the compiler then lets reads of one overtake copies into the other
@@ -311,12 +313,48 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
     }
 
     int nblk = 0;
-    const int ntiles = PAIR ? pair_tile_count<MODE>(p, mA, mB, nblk) : tile_count<MODE>(p, ridx, m, nblk);
-    auto tile_of = [&](int it) -> Tile {
-        if constexpr (PAIR) {
+    // Paired block-sparse: both row blocks' lists (ascending block ids) are parked in LDS and walked
+    // as one merged sequence; a block that is on both lists is copied and visited once.
+    __shared__ int lds_list[PAIR && MODE == MODE_BS ? 2 * BS_PAIR_MAX : 1];
+    int bs_na = 0, bs_nb = 0, bs_ia = 0, bs_ib = 0;
+    if constexpr (PAIR && MODE == MODE_BS) {
+        bs_na = min(mA + 1, p.max_blocks);
+        bs_nb = (2 * mslot + 1 < p.rows && (2 * mslot + 1) * BM < seqlen) ? min(mA + 2, p.max_blocks) : 0;
+        const long long rbase = ((long long)b * p.hq + h) * p.bidx_rows;
+        for (int i = tid; i < bs_na; i += NT) lds_list[i] = p.bidx[(rbase + mA) * p.max_blocks + i];
+        for (int i = tid; i < bs_nb; i += NT) lds_list[BS_PAIR_MAX + i] = p.bidx[(rbase + mA + 1) * p.max_blocks + i];
+        __syncthreads();
+    }
+    auto bs_merge_next = [&]() -> Tile {      // one step of the merged walk (wave-uniform)
+        Tile t;
+        t.gathered = 0;
+        t.nvalid = BN;
+        const int xa = bs_ia < bs_na ? __builtin_amdgcn_readfirstlane(lds_list[min(bs_ia, BS_PAIR_MAX - 1)]) : 0x7fffffff;
+        const int xb = bs_ib < bs_nb ? __builtin_amdgcn_readfirstlane(lds_list[BS_PAIR_MAX + min(bs_ib, BS_PAIR_MAX - 1)]) : 0x7fffffff;
+        const int x = min(xa, xb);
+        t.on_a = xa == x && bs_ia < bs_na;
+        t.on_b = xb == x && bs_ib < bs_nb;
+        bs_ia += t.on_a;
+        bs_ib += t.on_b;
+        t.start = x * BN;
+        return t;
+    };
+    // the merged walk ends when both lists are used up (its length is not known in advance)
+    int ntiles = 0;
+    if constexpr (!(PAIR && MODE == MODE_BS))
+        ntiles = PAIR ? pair_tile_count<MODE>(p, mA, mB, nblk) : tile_count<MODE>(p, ridx, m, nblk);
+    auto more_tiles = [&](int it) -> bool {   // is there a tile number `it` ?
+        if constexpr (PAIR && MODE == MODE_BS) return bs_ia < bs_na || bs_ib < bs_nb;
+        else return it < ntiles;
+    };
+    auto tile_of = [&](int it) -> Tile {      // called with it = 0, 1, 2, ... in order
+        if constexpr (PAIR && MODE == MODE_BS) {
+            return bs_merge_next();
+        } else if constexpr (PAIR) {
             Tile t;
             t.gathered = 0;
             t.nvalid = BN;
+            t.on_a = t.on_b = 1;
             t.start = pair_tile_start<MODE>(p, mA, mB, nblk, it);
             return t;
         } else {
@@ -413,22 +451,26 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
     //   issue K(it+1) copy; softmax; O^T += V^T.P^T
     Tile cur, nxt;
     int gt_cur = 0, gt_nxt = 0;
-    if (ntiles > 0) {
+    bool have_cur = more_tiles(0);
+    if (have_cur) {
         cur = tile_of(0);
         gt_cur = gather_ids(cur);
         copy_tile(cur, k_base, k_row, std::false_type{}, gt_cur, lds_k);
     }
 
-    for (int it = 0; it < ntiles; ++it) {
+    for (int it = 0; have_cur; ++it) {
         __builtin_amdgcn_s_waitcnt(0x0f70);      // vmcnt(0): this wave's part of K(it) is in LDS
         __syncthreads();
         Frag a0[8], a1[8];
         copy_tile(cur, v_base, v_row, std::true_type{}, gt_cur, lds_v);
-        nxt = tile_of(min(it + 1, ntiles - 1));
+        const bool have_nxt = more_tiles(it + 1);
+        nxt = have_nxt ? tile_of(it + 1) : cur;
         gt_nxt = gather_ids(nxt);
 
         // paired variant: is this tile on the list of this wave's row block ?
-        const bool active = !PAIR || (have_rows && tile_on_list<MODE>(p, m, cur.start));
+        bool active = true;
+        if constexpr (PAIR && MODE == MODE_BS) active = have_rows && (half ? cur.on_b : cur.on_a);
+        else if constexpr (PAIR) active = have_rows && tile_on_list<MODE>(p, m, cur.start);
         f32x16_t s0, s1;
         if (active) {
         __builtin_amdgcn_s_setprio(2);
@@ -471,7 +513,7 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
                     (__attribute__((address_space(3))) short4_t *)(lds_v + v_rd_off[db] + (8 * jj) * ROW_BYTES));
         __builtin_amdgcn_sched_barrier(0);
         }
-        if (it + 1 < ntiles) copy_tile(nxt, k_base, k_row, std::false_type{}, gt_nxt, lds_k);
+        if (have_nxt) copy_tile(nxt, k_base, k_row, std::false_type{}, gt_nxt, lds_k);
         if (active) {
 
         // ---- mask -----------------------------------------------------------
@@ -582,6 +624,7 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
         }
         cur = nxt;
         gt_cur = gt_nxt;
+        have_cur = have_nxt;
     }
 
     // ---- epilogue: O = O^T / l, transposed through LDS so that every global store is 16 bytes
@@ -654,18 +697,23 @@ void fill_params(AttnParams &p, const minf_qkvo *t) {
 
 template <int MODE> int launch(AttnParams p, int dtype, void *stream) {
     if (p.total_wg == 0) return MINF_OK;
-    constexpr bool PAIR = MODE == MODE_DENSE || MODE == MODE_ASHAPE;
-    if (PAIR) p.total_wg = (long long)p.batch * p.hq * ((p.rows + 1) / 2);
+    constexpr bool CAN_PAIR = MODE != MODE_VS;
+    const bool pair = CAN_PAIR && (MODE != MODE_BS || p.max_blocks <= BS_PAIR_MAX);
+    if (pair) p.total_wg = (long long)p.batch * p.hq * ((p.rows + 1) / 2);
     const long long per_xcd = (p.total_wg + 7) >> 3;
     const long long grid = per_xcd * 8;
     if (grid > 0x7fffffffLL) return MINF_ERR_UNSUPPORTED;
-    const dim3 block(PAIR ? 2 * NTHREADS : NTHREADS);
-    if (dtype == MINF_BF16)
-        hipLaunchKernelGGL((attn_fwd_kernel<__bf16, MODE, PAIR>), dim3((unsigned)grid), block, 0,
-                           (hipStream_t)stream, p);
-    else
-        hipLaunchKernelGGL((attn_fwd_kernel<_Float16, MODE, PAIR>), dim3((unsigned)grid), block, 0,
-                           (hipStream_t)stream, p);
+    const dim3 block(pair ? 2 * NTHREADS : NTHREADS);
+    hipStream_t st = (hipStream_t)stream;
+    if constexpr (CAN_PAIR) {
+        if (pair) {
+            if (dtype == MINF_BF16) hipLaunchKernelGGL((attn_fwd_kernel<__bf16, MODE, true>), dim3((unsigned)grid), block, 0, st, p);
+            else hipLaunchKernelGGL((attn_fwd_kernel<_Float16, MODE, true>), dim3((unsigned)grid), block, 0, st, p);
+            return minf_launch_status();
+        }
+    }
+    if (dtype == MINF_BF16) hipLaunchKernelGGL((attn_fwd_kernel<__bf16, MODE, false>), dim3((unsigned)grid), block, 0, st, p);
+    else hipLaunchKernelGGL((attn_fwd_kernel<_Float16, MODE, false>), dim3((unsigned)grid), block, 0, st, p);
     return minf_launch_status();
 }
 

@@ -104,6 +104,32 @@ def test_block_sparse_from_index_vs_oracle(gpu, n, top_k, hq, hk):
     check(out, ref, "bs")
 
 
+@pytest.mark.parametrize("n,top_k,order", [(1984, 6, "shuffled"), (1984, 6, "sorted"), (1100, 3, "shuffled"),
+                                           (4160, 40, "sorted"), (1100, 600, "sorted")])
+def test_block_sparse_lists_that_differ_between_neighbouring_row_blocks(gpu, n, top_k, order):
+    """Two neighbouring row blocks are served by one workgroup that walks the union of their
+    lists: lists drawn independently per row block (little or no overlap, any order, an odd
+    number of row blocks) must give the same result as the mask built from each list alone."""
+    from minference_amd import block_sparse_attention_from_index
+    print(f"case bs-lists n={n} top_k={top_k} {order}", flush=True)
+    hq = 2
+    q, k, v = make(1, hq, 1, n, 23, torch.bfloat16)
+    rows = (n + 64 - (n & 63)) // 64
+    rng = np.random.default_rng(n + top_k)
+    bi = np.zeros((1, hq, rows, top_k), dtype=np.int32)
+    for h in range(hq):
+        for m in range(rows):
+            cnt = min(m + 1, top_k)
+            pick = rng.choice(m + 1, size=cnt, replace=False)
+            bi[0, h, m, :cnt] = np.sort(pick) if order == "sorted" else pick
+            bi[0, h, m, cnt:] = m            # never visited: only the first min(m+1, top_k) count
+    bi = torch.from_numpy(bi)
+    out = block_sparse_attention_from_index(q.to(gpu), k.to(gpu), v.to(gpu), bi.to(gpu))
+    ref = torch.stack([O.masked_attention(q[0, h], expand(k, hq)[0, h], expand(v, hq)[0, h],
+                                          O.bs_mask(bi[0, h].numpy(), n)) for h in range(hq)])[None]
+    check(out, ref, "bs-lists")
+
+
 def test_block_sparse_op_topk_covers_everything_equals_sdpa(gpu):
     from minference_amd import block_sparse_attention
     n = 900
