@@ -232,6 +232,58 @@ int minf_bs_block_index(const void *q, const void *k, const int64_t *q_stride,
                         int32_t *block_index, void *workspace, size_t workspace_bytes,
                         void *stream);
 
+/*
+ * Offline pattern search: the share of the exact causal softmax mass that candidate sparse
+ * patterns keep, averaged over the query rows >= row_begin.  Replaces the scoring part of
+ * search_pattern (reference minference/modules/minference_forward.py:129-227: the stream_llm,
+ * vertical_and_slash and block_sparse closures build N x N masks and multiply them into the
+ * N x N softmax, :156-161, :166-172, :187-194); here nothing of size N x N is materialised.
+ * Up to 8 candidates are scored in one sweep: bit t of every flag byte belongs to candidate t.
+ * Element (r, c), c <= r, counts for candidate t iff bit t is set in col_flags[c], in
+ * diag_flags[r - c] or in block_flags[r / 32][c / 32].
+ *   col_flags, diag_flags [batch*heads_q, flag_pitch] uint8, 4-byte aligned,
+ *       flag_pitch % 4 == 0 and flag_pitch >= n rounded up to 64 (padding bytes zero)
+ *   block_flags [batch*heads_q, ceil(n/32), block_pitch] uint8 or NULL, block_pitch >= ceil(n/32)
+ *   recall [batch*heads_q, 8] fp32: mean over rows r in [row_begin, n) of
+ *       sum_{c in candidate} softmax(q.k^T * sm_scale)[r, c]; NaN when n <= row_begin
+ *       (the reference's mean of an empty slice); bits nobody set give 0
+ *   workspace: minf_pattern_recall_workspace_bytes() bytes, 4-byte aligned
+ * Deterministic (fixed summation order).  fp32 softmax on 16-bit q, k (the reference rounds the
+ * probabilities to the input dtype before summing them).
+ */
+size_t minf_pattern_recall_workspace_bytes(int batch, int heads_q, int n);
+int minf_pattern_recall(const void *q, const void *k, const int64_t *q_stride,
+                        const int64_t *k_stride, int batch, int heads_q, int heads_kv, int n,
+                        int head_dim, int dtype, float sm_scale, const uint8_t *col_flags,
+                        const uint8_t *diag_flags, int64_t flag_pitch, const uint8_t *block_flags,
+                        int64_t block_pitch, int row_begin, float *recall, void *workspace,
+                        size_t workspace_bytes, void *stream);
+
+/*
+ * Builders of the flag arrays above (reference: the scatter of top-k indices into an N x N mask
+ * and the spdiags construction, minference_forward.py:141-155, :166-168, :186-189).
+ * minf_flags_set_indices ORs bit `bit` into flags[row, idx[row, i]] for i < k (entries outside
+ * [0, limit) are ignored); minf_flags_set_range ORs it into flags[row, begin..end) of every row.
+ * flags [rows, flag_pitch] uint8, 4-byte aligned, flag_pitch % 4 == 0; idx [rows, k] int32 with
+ * idx_stride elements between rows.
+ */
+int minf_flags_set_indices(const int32_t *idx, int rows, int k, int64_t idx_stride, int bit,
+                           uint8_t *flags, int64_t flag_pitch, int limit, void *stream);
+int minf_flags_set_range(int begin, int end, int rows, int bit, uint8_t *flags, int64_t flag_pitch,
+                         void *stream);
+
+/*
+ * Block index of the block_sparse candidate of the pattern search (reference
+ * minference_forward.py:175-186): like minf_bs_block_index with 32-token blocks,
+ * rows = ceil(n/32) (zero padding only up to the next multiple of 32) and no forced blocks.
+ *   block_index [batch, heads_q, rows, min(top_k, rows)] int32
+ */
+size_t minf_search_block_index_workspace_bytes(int batch, int heads_q, int heads_kv, int n);
+int minf_search_block_index(const void *q, const void *k, const int64_t *q_stride,
+                            const int64_t *k_stride, int batch, int heads_q, int heads_kv, int n,
+                            int head_dim, int dtype, int top_k, int32_t *block_index,
+                            void *workspace, size_t workspace_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

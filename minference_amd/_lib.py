@@ -37,6 +37,13 @@ SIGNATURES = {
     "minf_bs_block_index_rows": (c_int, [c_int]),
     "minf_bs_block_index_workspace_bytes": (ctypes.c_size_t, [c_int] * 4),
     "minf_bs_block_index": (c_int, [c_ptr, c_ptr, c_ptr, c_ptr] + [c_int] * 8 + [c_ptr, c_ptr, ctypes.c_size_t, c_ptr]),
+    "minf_pattern_recall_workspace_bytes": (ctypes.c_size_t, [c_int] * 3),
+    "minf_pattern_recall": (c_int, [c_ptr, c_ptr, c_ptr, c_ptr] + [c_int] * 6 + [c_f32, c_ptr, c_ptr, c_i64, c_ptr, c_i64,
+                                                                                   c_int, c_ptr, c_ptr, ctypes.c_size_t, c_ptr]),
+    "minf_flags_set_indices": (c_int, [c_ptr, c_int, c_int, c_i64, c_int, c_ptr, c_i64, c_int, c_ptr]),
+    "minf_flags_set_range": (c_int, [c_int, c_int, c_int, c_int, c_ptr, c_i64, c_ptr]),
+    "minf_search_block_index_workspace_bytes": (ctypes.c_size_t, [c_int] * 4),
+    "minf_search_block_index": (c_int, [c_ptr, c_ptr, c_ptr, c_ptr] + [c_int] * 7 + [c_ptr, c_ptr, ctypes.c_size_t, c_ptr]),
 }
 
 

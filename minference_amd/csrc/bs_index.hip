@@ -35,6 +35,7 @@ struct PoolParams {
     long long xs[3];
     float *out;               // [batch*heads, rows, 128] fp32
     int heads, n, rows;
+    int blk;                  // tokens per block: 64 or 32
 };
 
 template <typename T> __device__ __forceinline__ float to_f32(unsigned short bits);
@@ -60,8 +61,8 @@ template <typename T> __global__ __launch_bounds__(256) void bs_pool_kernel(cons
     for (int e = 0; e < 8; ++e) acc[e] = 0.f;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        const int tok = blk * BLK + r4 + 16 * j;
-        if (tok < p.n) {
+        const int tok = blk * p.blk + r4 + 16 * j;
+        if (16 * j < p.blk && tok < p.n) {
             const u32x4_t raw = *reinterpret_cast<const u32x4_t *>(base + (long long)tok * p.xs[2] * 2 + c * 16);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -77,7 +78,7 @@ template <typename T> __global__ __launch_bounds__(256) void bs_pool_kernel(cons
         float s = 0.f;
 #pragma unroll
         for (int r = 0; r < 16; ++r) s += red[r][tid];
-        p.out[((long long)bh * p.rows + blk) * HD + tid] = s * (1.0f / BLK);
+        p.out[((long long)bh * p.rows + blk) * HD + tid] = s / (float)p.blk;
     }
 }
 
@@ -141,23 +142,21 @@ __global__ __launch_bounds__(256) void bs_scores_kernel(const ScoreParams p) {
 inline int padded_rows(int n) { return (n + (BLK - (n & (BLK - 1)))) / BLK; }
 inline int score_pitch(int rows) { return (rows + 3) & ~3; }
 inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+inline size_t workspace_for(int batch, int heads_q, int heads_kv, int rows) {
+    return align256((size_t)batch * heads_q * rows * HD * 4) + align256((size_t)batch * heads_kv * rows * HD * 4) +
+           align256((size_t)batch * heads_q * rows * score_pitch(rows) * 4);
+}
 
 }  // namespace
 
 extern "C" int minf_bs_block_index_rows(int n) { return n < 0 ? 0 : padded_rows(n); }
 
-extern "C" size_t minf_bs_block_index_workspace_bytes(int batch, int heads_q, int heads_kv, int n) {
-    if (batch <= 0 || heads_q <= 0 || heads_kv <= 0 || n <= 0) return 0;
-    const size_t rows = (size_t)padded_rows(n);
-    return align256((size_t)batch * heads_q * rows * HD * 4) + align256((size_t)batch * heads_kv * rows * HD * 4) +
-           align256((size_t)batch * heads_q * rows * score_pitch((int)rows) * 4);
-}
+namespace {
 
-extern "C" int minf_bs_block_index(const void *q, const void *k, const int64_t *q_stride,
-                                   const int64_t *k_stride, int batch, int heads_q, int heads_kv,
-                                   int n, int head_dim, int dtype, int top_k, int force_diag_first,
-                                   int32_t *block_index, void *workspace, size_t workspace_bytes,
-                                   void *stream) {
+int block_index_impl(const void *q, const void *k, const int64_t *q_stride, const int64_t *k_stride, int batch,
+                     int heads_q, int heads_kv, int n, int head_dim, int dtype, int blk, int rows, int top_k,
+                     int force_diag_first, int32_t *block_index, void *workspace, size_t workspace_bytes,
+                     void *stream) {
     if (!q || !k || !q_stride || !k_stride || !block_index) return MINF_ERR_INVALID_ARG;
     if (batch < 0 || heads_q <= 0 || heads_kv <= 0 || n <= 0 || top_k <= 0) return MINF_ERR_INVALID_ARG;
     if (heads_q % heads_kv != 0) return MINF_ERR_INVALID_ARG;
@@ -167,9 +166,8 @@ extern "C" int minf_bs_block_index(const void *q, const void *k, const int64_t *
     for (int i = 0; i < 3; ++i)
         if ((q_stride[i] | k_stride[i]) & 7) return MINF_ERR_ALIGNMENT;
     if (batch == 0) return MINF_OK;
-    const size_t need = minf_bs_block_index_workspace_bytes(batch, heads_q, heads_kv, n);
+    const size_t need = workspace_for(batch, heads_q, heads_kv, rows);
     if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 15)) return MINF_ERR_WORKSPACE;
-    const int rows = padded_rows(n);
     const int pitch = score_pitch(rows);
     if ((long long)batch * heads_q * rows > 0x7fffffffLL || (long long)batch * heads_q > 65535) return MINF_ERR_UNSUPPORTED;
 
@@ -181,8 +179,8 @@ extern "C" int minf_bs_block_index(const void *q, const void *k, const int64_t *
     float *scores = (float *)ws;
     hipStream_t st = (hipStream_t)stream;
 
-    PoolParams pq{(const char *)q, {q_stride[0], q_stride[1], q_stride[2]}, qp, heads_q, n, rows};
-    PoolParams pk{(const char *)k, {k_stride[0], k_stride[1], k_stride[2]}, kp, heads_kv, n, rows};
+    PoolParams pq{(const char *)q, {q_stride[0], q_stride[1], q_stride[2]}, qp, heads_q, n, rows, blk};
+    PoolParams pk{(const char *)k, {k_stride[0], k_stride[1], k_stride[2]}, kp, heads_kv, n, rows, blk};
     if (dtype == MINF_BF16) {
         hipLaunchKernelGGL(bs_pool_kernel<__bf16>, dim3(rows, batch * heads_q), dim3(256), 0, st, pq);
         hipLaunchKernelGGL(bs_pool_kernel<__bf16>, dim3(rows, batch * heads_kv), dim3(256), 0, st, pk);
@@ -201,4 +199,34 @@ extern "C" int minf_bs_block_index(const void *q, const void *k, const int64_t *
 
     const int kk = top_k < rows ? top_k : rows;
     return minf_topk_indices(scores, batch * heads_q * rows, rows, pitch, kk, block_index, kk, -1, stream);
+}
+
+}  // namespace
+
+extern "C" size_t minf_bs_block_index_workspace_bytes(int batch, int heads_q, int heads_kv, int n) {
+    if (batch <= 0 || heads_q <= 0 || heads_kv <= 0 || n <= 0) return 0;
+    return workspace_for(batch, heads_q, heads_kv, padded_rows(n));
+}
+
+extern "C" int minf_bs_block_index(const void *q, const void *k, const int64_t *q_stride,
+                                   const int64_t *k_stride, int batch, int heads_q, int heads_kv,
+                                   int n, int head_dim, int dtype, int top_k, int force_diag_first,
+                                   int32_t *block_index, void *workspace, size_t workspace_bytes,
+                                   void *stream) {
+    return block_index_impl(q, k, q_stride, k_stride, batch, heads_q, heads_kv, n, head_dim, dtype, BLK,
+                            n > 0 ? padded_rows(n) : 0, top_k, force_diag_first, block_index, workspace,
+                            workspace_bytes, stream);
+}
+
+extern "C" size_t minf_search_block_index_workspace_bytes(int batch, int heads_q, int heads_kv, int n) {
+    if (batch <= 0 || heads_q <= 0 || heads_kv <= 0 || n <= 0) return 0;
+    return workspace_for(batch, heads_q, heads_kv, (n + 31) / 32);
+}
+
+extern "C" int minf_search_block_index(const void *q, const void *k, const int64_t *q_stride,
+                                       const int64_t *k_stride, int batch, int heads_q, int heads_kv,
+                                       int n, int head_dim, int dtype, int top_k, int32_t *block_index,
+                                       void *workspace, size_t workspace_bytes, void *stream) {
+    return block_index_impl(q, k, q_stride, k_stride, batch, heads_q, heads_kv, n, head_dim, dtype, 32,
+                            n > 0 ? (n + 31) / 32 : 0, top_k, 0, block_index, workspace, workspace_bytes, stream);
 }

@@ -13,6 +13,8 @@ Every function cites the reference lines it restates.  Parity status:
   torch's scaled_dot_product_attention, brute force on tiny inputs)
 * ``bs_block_index`` / ``bs_mask``    pinned (properties, top_k>=rows -> causal SDPA)
 * ``ashape_mask``         pinned (closed form vs per-element loop, n_local>=N -> causal SDPA)
+* ``search_candidate_mask`` / ``search_pattern_scores``  pinned (Q=0 closed forms counted by
+  explicit loops, all-kept candidates -> 1, brute force on tiny inputs)
 * ``torch.topk`` tie order and Triton's bf16 rounding points are implementation
   defined in the reference (not in its source): "parity unpinned" for those;
   tests compare top-k *sets* away from ties and outputs within tolerance.
@@ -347,3 +349,89 @@ def streaming_forward(q, k, v, n_init, n_local):
         for h in range(H):
             out[b, h] = masked_attention(q[b, h], k[b, h], v[b, h], m)
     return out
+
+
+# --------------------------------------------------------------------------
+# f-4  offline pattern search   minference/modules/minference_forward.py:129-227
+# --------------------------------------------------------------------------
+SEARCH_ROW_BEGIN = 2500                                     # :161,:172,:194  [..., 2500:]
+SEARCH_CANDIDATES = (                                       # :209-215
+    ("stream_llm", 100, 800),
+    ("vertical_and_slash", 30, 800), ("vertical_and_slash", 100, 750),
+    ("vertical_and_slash", 500, 700), ("vertical_and_slash", 3500, 100),
+    ("block_sparse", 8, 1),
+)
+
+
+def search_candidate_mask(q, k, ty, v_size, s_size):
+    """Element mask [N,N] (bool, already causal) that search_pattern scores for one candidate of
+    one head; q,k [N,D].  fp32 arithmetic, ties -> lowest index.
+    stream_llm (:164-173): offsets 0..s_size plus the first v_size columns.
+    vertical_and_slash (:133-162): the v_size best columns of the last-64-query estimate (first
+    30 forced) plus the s_size best single diagonals (offsets 0..29 forced).
+    block_sparse (:175-195): 32x32 blocks, zero-padded mean pooling, unscaled pooled scores,
+    the block_num // v_size best key blocks of every query block row."""
+    n, d = q.shape
+    r = torch.arange(n)[:, None]
+    c = torch.arange(n)[None, :]
+    off = r - c
+    causal = off >= 0
+    if ty == "stream_llm":
+        return (causal & (off <= s_size)) | (causal & (c < v_size))
+    if ty == "vertical_and_slash":
+        vertical, slash = estimate_scores(q[None, None], k[None, None], 64)
+        vertical, slash = vertical[0, 0].clone(), slash[0, 0].clone()
+        vertical[:30] = torch.inf
+        slash[-30:] = torch.inf
+        cols = topk_lowest_index(vertical, min(v_size, n))
+        offs = (n - 1) - topk_lowest_index(slash, min(s_size, n))
+        colkeep = torch.zeros(n, dtype=torch.bool); colkeep[cols] = True
+        offkeep = torch.zeros(n, dtype=torch.bool); offkeep[offs] = True
+        return causal & (colkeep[None, :] | offkeep[off.clamp(min=0)])
+    if ty == "block_sparse":
+        nb = (n - 1) // 32 + 1
+        pad = nb * 32 - n
+        bq = torch.nn.functional.pad(q.float(), [0, 0, 0, pad]).reshape(nb, 32, d).mean(1)
+        bk = torch.nn.functional.pad(k.float(), [0, 0, 0, pad]).reshape(nb, 32, d).mean(1)
+        sc = bq @ bk.T
+        ar = torch.arange(nb)
+        sc = torch.where(ar[:, None] >= ar[None, :], sc, torch.tensor(-torch.inf))
+        keep = nb // v_size
+        bm = torch.zeros(nb, nb, dtype=torch.bool)
+        if keep > 0:
+            idx = topk_lowest_index(sc, keep)
+            bm[ar[:, None].expand_as(idx), idx] = True
+        full = bm.repeat_interleave(32, 0).repeat_interleave(32, 1)[:n, :n]
+        return causal & full
+    raise ValueError(ty)
+
+
+def search_pattern_scores(q, k, candidates=SEARCH_CANDIDATES, row_begin=SEARCH_ROW_BEGIN):
+    """:197-219: for every candidate, the mean over query rows >= row_begin of the softmax mass
+    that falls inside the candidate's mask.  q,k [N,D] of one head -> list of floats (nan when
+    N <= row_begin, like the mean of an empty slice)."""
+    n, d = q.shape
+    s = (q.float() @ k.float().T) / math.sqrt(d)
+    s = torch.where(torch.arange(n)[:, None] >= torch.arange(n)[None, :], s, torch.tensor(-torch.inf))
+    attn = torch.softmax(s, dim=-1, dtype=torch.float32)
+    out = []
+    for ty, v_size, s_size in candidates:
+        m = search_candidate_mask(q, k, ty, v_size, s_size)
+        out.append((attn * m)[row_begin:].sum(-1).mean().item())
+    return out
+
+
+def search_pattern(q, k, candidates=SEARCH_CANDIDATES, row_begin=SEARCH_ROW_BEGIN):
+    """:205-227: best candidate by score (first wins ties, score must exceed 0), relabelled like
+    the reference: stream_llm -> vertical_and_slash with its own sizes, block_sparse ->
+    vertical_and_slash (1000, 6096).  -> (type, v, s, score)."""
+    scores = search_pattern_scores(q, k, candidates, row_begin)
+    best_ty, best_v, best_s, best = "", 0, 0, 0.0
+    for (ty, v_size, s_size), sc in zip(candidates, scores):
+        if sc > best:
+            best_ty, best_v, best_s, best = ty, v_size, s_size, sc
+    if best_ty == "stream_llm":
+        best_ty = "vertical_and_slash"
+    if best_ty == "block_sparse":
+        best_ty, best_v, best_s = "vertical_and_slash", 1000, 6096
+    return best_ty, best_v, best_s, best
