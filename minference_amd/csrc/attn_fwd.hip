@@ -3,8 +3,9 @@
 // A-shape ranges, dense causal).
 //
 // Work split: one workgroup (2 wavefronts) per (batch, query head, 64-row
-// block); each wavefront owns 32 query rows.  Dense and A-shape / tri-shape launches use the
-// paired variant: 4 wavefronts over two neighbouring row blocks that share every K/V tile copy.
+// block); each wavefront owns 32 query rows.  Dense, A-shape / tri-shape and block-sparse launches
+// use the paired variant: 4 wavefronts over two neighbouring row blocks that walk the union of
+// their tile lists and share every K/V tile copy.
 // Everything is computed in the TRANSPOSED orientation so that softmax statistics are per lane:
 //
 //   S^T[token][qrow] = K_tile . Q^T      v_mfma_f32_32x32x16 (A = K from LDS, B = Q in VGPRs)
@@ -157,8 +158,9 @@ constexpr int BS_PAIR_MAX = 512;   // longest block list the paired block-sparse
 template <int MODE>
 __device__ __forceinline__ int tile_count(const AttnParams &p, long long ridx, int m, int &nblk) {
     if constexpr (MODE == MODE_VS) {
-        nblk = as_const(p.bc)[ridx];
-        return nblk + ((as_const(p.cc)[ridx] + BN - 1) >> 6);
+        // counts are clamped to the list widths: a bad count must not turn into a read past the row
+        nblk = max(0, min(as_const(p.bc)[ridx], p.nnz_s));
+        return nblk + ((max(0, min(as_const(p.cc)[ridx], p.nnz_v)) + BN - 1) >> 6);
     } else if constexpr (MODE == MODE_BS) {
         nblk = min(m + 1, p.max_blocks);
         return nblk;
@@ -190,7 +192,7 @@ __device__ __forceinline__ Tile tile_at(const AttnParams &p, long long ridx, int
         } else {
             t.gathered = 1;
             t.start = (it - nblk) * BN;
-            t.nvalid = min(BN, as_const(p.cc)[ridx] - t.start);
+            t.nvalid = min(BN, min(as_const(p.cc)[ridx], p.nnz_v) - t.start);
         }
     } else if constexpr (MODE == MODE_BS) {
         t.start = as_const(p.bidx)[((ridx / p.rows) * p.bidx_rows + m) * p.max_blocks + it] * BN;
@@ -204,10 +206,11 @@ __device__ __forceinline__ Tile tile_at(const AttnParams &p, long long ridx, int
     return t;
 }
 
-// Paired variant (dense causal and A-shape / tri-shape, whose tile lists are analytic): one
-// workgroup of 4 waves covers the row blocks mA = 2*mp and mB = mA + 1.  Their tile lists differ
-// by at most the ends, so the workgroup walks the union once and every K/V tile is copied into LDS
-// once for 128 query rows; a half skips the tiles that are not on its own list.
+// Paired variant: one workgroup of 4 waves covers the row blocks mA = 2*mp and mB = mA + 1.  It
+// walks the union of their two tile lists once, so every K/V tile is copied into LDS once for 128
+// query rows; a half skips the tiles that are not on its own list.  For dense causal and A-shape /
+// tri-shape the lists are analytic and differ by at most the ends (the three helpers below); for
+// block-sparse the two lists are merged on the fly inside the kernel.
 template <int MODE>
 __device__ __forceinline__ int pair_tile_count(const AttnParams &p, int mA, int mB, int &nblk) {
     if (MODE == MODE_DENSE || mB * BM + BM - 1 >= p.dense_from) {
@@ -697,7 +700,10 @@ void fill_params(AttnParams &p, const minf_qkvo *t) {
 
 template <int MODE> int launch(AttnParams p, int dtype, void *stream) {
     if (p.total_wg == 0) return MINF_OK;
+    // vertical-slash lists (blocks + gathered columns per row block) run on the 2-wave kernel,
+    // everything else on the paired one -- except block lists too long for the paired walk's LDS copy
     constexpr bool CAN_PAIR = MODE != MODE_VS;
+    constexpr bool CAN_SINGLE = MODE == MODE_VS || MODE == MODE_BS;
     const bool pair = CAN_PAIR && (MODE != MODE_BS || p.max_blocks <= BS_PAIR_MAX);
     if (pair) p.total_wg = (long long)p.batch * p.hq * ((p.rows + 1) / 2);
     const long long per_xcd = (p.total_wg + 7) >> 3;
@@ -712,9 +718,12 @@ template <int MODE> int launch(AttnParams p, int dtype, void *stream) {
             return minf_launch_status();
         }
     }
-    if (dtype == MINF_BF16) hipLaunchKernelGGL((attn_fwd_kernel<__bf16, MODE, false>), dim3((unsigned)grid), block, 0, st, p);
-    else hipLaunchKernelGGL((attn_fwd_kernel<_Float16, MODE, false>), dim3((unsigned)grid), block, 0, st, p);
-    return minf_launch_status();
+    if constexpr (CAN_SINGLE) {
+        if (dtype == MINF_BF16) hipLaunchKernelGGL((attn_fwd_kernel<__bf16, MODE, false>), dim3((unsigned)grid), block, 0, st, p);
+        else hipLaunchKernelGGL((attn_fwd_kernel<_Float16, MODE, false>), dim3((unsigned)grid), block, 0, st, p);
+        return minf_launch_status();
+    }
+    return MINF_ERR_UNSUPPORTED;      // not reached: every mode has one of the two variants
 }
 
 }  // namespace

@@ -64,6 +64,45 @@ def test_argument_validation_needs_no_gpu(lib):
     assert lib.minf_vs_estimate_workspace_bytes(0, 32, 131072) == 0
 
 
+def test_argument_validation_of_the_index_estimate_and_search_entry_points(lib):
+    from minference_amd import _lib
+    i3 = (_lib.c_i64 * 3)(128 * 64 * 4, 128 * 64, 128)
+    bad = (_lib.c_i64 * 3)(128 * 64 * 4, 128 * 64, 100)
+    P = 4096                                                     # any 16-byte aligned non-null address; never dereferenced
+    # estimate: workspace too small / misaligned strides / last_q out of range
+    assert lib.minf_vs_estimate(P, P, i3, i3, 1, 4, 4, 64, 128, 0, 0.1, 64, 30, 100, P, P, P, 16, None) == -4
+    assert lib.minf_vs_estimate(P, P, bad, i3, 1, 4, 4, 64, 128, 0, 0.1, 64, 30, 100, P, P, P, 1 << 30, None) == -3
+    assert lib.minf_vs_estimate(P, P, i3, i3, 1, 4, 4, 64, 128, 0, 0.1, 65, 30, 100, P, P, P, 1 << 30, None) == -1
+    assert lib.minf_vs_estimate(P, P, i3, i3, 1, 4, 4, 64, 64, 0, 0.1, 64, 30, 100, P, P, P, 1 << 30, None) == -2
+    # block index: head counts, head_dim, workspace
+    assert lib.minf_bs_block_index(P, P, i3, i3, 1, 4, 3, 64, 128, 0, 10, 0, P, P, 1 << 30, None) == -1
+    assert lib.minf_bs_block_index(P, P, i3, i3, 1, 4, 4, 64, 256, 0, 10, 0, P, P, 1 << 30, None) == -2
+    assert lib.minf_bs_block_index(P, P, i3, i3, 1, 4, 4, 64, 128, 0, 10, 0, P, P, 8, None) == -4
+    assert lib.minf_search_block_index(P, P, i3, i3, 1, 4, 4, 64, 128, 0, 0, P, P, 1 << 30, None) == -1   # top_k 0
+    assert lib.minf_bs_block_index_rows(64) == 2 and lib.minf_bs_block_index_rows(65) == 2
+    # vertical-slash attention: row count must be ceil(n/64), list widths positive
+    t = _lib.QKVO()
+    t.q = t.k = t.v = t.o = P
+    t.batch, t.heads_q, t.heads_kv, t.n, t.head_dim, t.dtype = 1, 4, 4, 130, 128, 0
+    for name in ("q_stride", "k_stride", "v_stride", "o_stride"):
+        getattr(t, name)[:] = [128 * 130 * 4, 128 * 130, 128]
+    assert lib.minf_vs_attn_fwd(ctypes.byref(t), P, P, P, P, 2, 8, 8, None) == -1         # rows must be 3
+    assert lib.minf_vs_attn_fwd(ctypes.byref(t), P, P, P, P, 3, 0, 8, None) == -1         # nnz_s < 1
+    assert lib.minf_vs_attn_fwd(ctypes.byref(t), None, P, P, P, 3, 8, 8, None) == -1
+    assert lib.minf_bs_attn_fwd(ctypes.byref(t), P, 2, 4, None) == -1                     # too few rows
+    assert lib.minf_ashape_attn_fwd(ctypes.byref(t), 4, 0, None) == -1                    # n_local < 1
+    assert lib.minf_trishape_attn_fwd(ctypes.byref(t), 4, 8, -1, None) == -1
+    # pattern search: flag pitch rules, candidate bit range, workspace
+    assert lib.minf_pattern_recall(P, P, i3, i3, 1, 4, 4, 130, 128, 0, 0.1, P, P, 128, None, 0, 0, P, P, 1 << 20, None) == -1   # pitch < 192
+    assert lib.minf_pattern_recall(P, P, i3, i3, 1, 4, 4, 130, 128, 0, 0.1, P, P, 192, None, 0, 0, P, P, 8, None) == -4
+    assert lib.minf_pattern_recall(P, P, i3, i3, 1, 4, 4, 130, 128, 0, 0.1, P, P, 192, P, 2, 0, P, P, 1 << 20, None) == -1      # block pitch < 5
+    assert lib.minf_pattern_recall_workspace_bytes(1, 4, 130) == 4 * 3 * 8 * 4
+    assert lib.minf_flags_set_indices(P, 4, 10, 10, 8, P, 192, 130, None) == -1           # bit 8
+    assert lib.minf_flags_set_indices(P, 4, 10, 10, 0, P, 190, 130, None) == -1           # pitch % 4
+    assert lib.minf_flags_set_range(0, 200, 4, 0, P, 192, None) == -1                     # end > pitch
+    assert lib.minf_flags_set_range(10, 10, 4, 0, P, 192, None) == 0                      # empty range: nothing to do
+
+
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     from minference_amd import _lib
     monkeypatch.setattr(_lib, "_lib", None)
