@@ -77,11 +77,12 @@ int minf_vs_index_build(const int32_t *seqlens, const int32_t *vertical_idx,
  * Same result as minf_vs_index_build, faster: a per-head pass first tabulates the part of the
  * reference's range merge that does not depend on the row block (ranges and blocks of a slash
  * list only move with the row block once no entry is skipped or clipped), then every row block
- * copies its blocks from the table and tests its verticals against the tabulated ranges.
- * workspace: minf_vs_index_workspace_bytes(batch, heads, nnz_s) bytes of device memory, 4-byte
- * aligned, overwritten.  Same reference lines, same bit-exactness and error behaviour.
+ * copies its blocks from the table and tests its verticals against a per-head coverage bitmap of
+ * the tabulated ranges.
+ * workspace: minf_vs_index_workspace_bytes(batch, heads, nnz_s, rows) bytes of device memory,
+ * 4-byte aligned, overwritten.  Same reference lines, same bit-exactness and error behaviour.
  */
-size_t minf_vs_index_workspace_bytes(int batch, int heads, int nnz_s);
+size_t minf_vs_index_workspace_bytes(int batch, int heads, int nnz_s, int rows);
 int minf_vs_index_build_ws(const int32_t *seqlens, const int32_t *vertical_idx,
                            const int32_t *slash_idx, int32_t *block_count,
                            int32_t *block_offset, int32_t *column_count,

@@ -22,7 +22,7 @@ SIGNATURES = {
     "minf_version": (c_int, []),
     "minf_status_string": (ctypes.c_char_p, [c_int]),
     "minf_vs_index_build": (c_int, [c_ptr] * 7 + [c_int] * 6 + [c_ptr, c_ptr]),
-    "minf_vs_index_workspace_bytes": (ctypes.c_size_t, [c_int] * 3),
+    "minf_vs_index_workspace_bytes": (ctypes.c_size_t, [c_int] * 4),
     "minf_vs_index_build_ws": (c_int, [c_ptr] * 7 + [c_int] * 6 + [c_ptr, c_ptr, ctypes.c_size_t, c_ptr]),
     "minf_vs_attn_fwd": (c_int, [c_ptr] * 5 + [c_int] * 3 + [c_ptr]),
     "minf_bs_attn_fwd": (c_int, [c_ptr, c_ptr, c_int, c_int, c_ptr]),

@@ -40,6 +40,27 @@ __device__ __forceinline__ void zero_range(int32_t *p, int from, int to, int lan
     if (lane < tail) q[n4 * 4 + lane] = 0;
 }
 
+// dst[i] = src[i] + shift for i < n with 16-byte stores: dst is brought to a 16-byte boundary with
+// single stores first (src then sits at any 4-byte phase; its 16-byte loads need no alignment)
+__device__ __forceinline__ void copy_shifted(int32_t *dst, const int32_t *src, int n, int shift, int lane) {
+    if (n <= 0) return;
+    int head = (int)(((16u - (unsigned)((uintptr_t)dst & 15u)) & 15u) >> 2);
+    if (head > n) head = n;
+    if (lane < head) dst[lane] = src[lane] + shift;
+    dst += head;
+    src += head;
+    n -= head;
+    const int n4 = n >> 2;
+    for (int i = lane; i < n4; i += MINF_WAVE) {
+        int4 v;
+        __builtin_memcpy(&v, src + 4 * i, 16);
+        v.x += shift; v.y += shift; v.z += shift; v.w += shift;
+        reinterpret_cast<int4 *>(dst)[i] = v;
+    }
+    const int tail = n & 3;
+    if (lane < tail) dst[n4 * 4 + lane] = src[n4 * 4 + lane] + shift;
+}
+
 // Range starts of one chunk of 64 entries.  `t` ascends along the lanes (padding lanes repeat the
 // last entry); the state carried in from the previous chunk is the current range start `cur_a`,
 // the running range end `carried_e` and the previous entry `carried_t`.  Entry i starts a new
@@ -222,14 +243,19 @@ __global__ __launch_bounds__(IDX_WAVES *MINF_WAVE) void vs_index_kernel(
 // not inside one of the remaining tabulated ranges, is not below the end of the last range of the
 // explicit part, and is below the last entry's t - the reference's merge rule restated per element.
 #define IDX_TAB_HDR 4
-__device__ __forceinline__ long long idx_tab_ints(int nnz_s) { return IDX_TAB_HDR + 5ll * nnz_s; }
+// per head: header, five tables of nnz_s ints, then a coverage bitmap of the virtual row (one bit
+// per key position, set inside the tabulated ranges) of bm_words 32-bit words
+__host__ __device__ __forceinline__ long long idx_bm_words(int rows) { return ((long long)rows * 64 + 64 + 31) / 32 + 1; }
+__host__ __device__ __forceinline__ long long idx_tab_ints(int nnz_s, int rows) {
+    return IDX_TAB_HDR + 5ll * nnz_s + idx_bm_words(rows);
+}
 
 __global__ __launch_bounds__(MINF_WAVE) void vs_index_prep_kernel(const int32_t *__restrict__ slash,
-                                                                  int32_t *__restrict__ tables, int nnz_s) {
+                                                                  int32_t *__restrict__ tables, int nnz_s, int rows) {
     const int lane = minf_lane();
     const long long bh = blockIdx.x;
     const int32_t *sl = slash + bh * (long long)nnz_s;
-    int32_t *hdr = tables + bh * idx_tab_ints(nnz_s);
+    int32_t *hdr = tables + bh * idx_tab_ints(nnz_s, rows);
     int32_t *cpos = hdr + IDX_TAB_HDR, *cpre = cpos + nnz_s, *crun = cpre + nnz_s;
     int32_t *run_a = crun + nnz_s, *run_e = run_a + nnz_s;
     const int V = sl[0] + 64;
@@ -237,11 +263,17 @@ __global__ __launch_bounds__(MINF_WAVE) void vs_index_prep_kernel(const int32_t 
     int nb = 0, nr = 0;
     int carried_e = 0, carried_t = 0, cur_a = 0;
     const int nchunks = (nnz_s + MINF_WAVE - 1) / MINF_WAVE;
+    // the walk is one chain of chunks; the list entries of the next two chunks are fetched ahead so
+    // that no chunk waits for a load
+    int o_next = sl[min(lane, nnz_s - 1)], o_next2 = sl[min(MINF_WAVE + lane, nnz_s - 1)];
     for (int c = 0; c < nchunks; ++c) {
         const int base = c * MINF_WAVE;
         const int cnt = min(MINF_WAVE, nnz_s - base);
         const bool valid = lane < cnt;
-        int t = valid ? max(V - sl[base + lane], 64) : 0;
+        const int o_cur = o_next;
+        o_next = o_next2;
+        o_next2 = sl[min(base + 3 * MINF_WAVE + lane - MINF_WAVE, nnz_s - 1)];
+        int t = valid ? max(V - o_cur, 64) : 0;
         const int tlast = minf_readlane(t, cnt - 1);
         if (!valid) t = tlast;
         if (c == 0) {
@@ -281,8 +313,39 @@ __global__ __launch_bounds__(MINF_WAVE) void vs_index_prep_kernel(const int32_t 
         hdr[0] = nb;
         hdr[1] = nr;
         hdr[2] = V;
-        hdr[3] = 0;
+        // the bitmap covers positions [0, 32 * bm_words); a list whose largest offset lies far
+        // outside the context does not fit and the row blocks fall back to searching the ranges
+        hdr[3] = (long long)V <= 32 * (idx_bm_words(rows) - 1) ? 1 : 0;
     }
+}
+
+// Coverage bitmap of a head's virtual row: bit p of the bitmap is set iff position p lies inside one
+// of the tabulated ranges [run_a[r], run_e[r]).  One thread per 32-bit word: a binary search finds
+// the first range that ends after the word's first position; ranges are at least 64 long, so at
+// most two of them touch a word.
+__global__ __launch_bounds__(256) void vs_index_bitmap_kernel(int32_t *__restrict__ tables, int nnz_s, int rows) {
+    const long long bh = blockIdx.y;
+    int32_t *hdr = tables + bh * idx_tab_ints(nnz_s, rows);
+    if (!hdr[3]) return;
+    const int32_t *run_a = hdr + IDX_TAB_HDR + 3ll * nnz_s, *run_e = run_a + nnz_s;
+    uint32_t *bm = reinterpret_cast<uint32_t *>(hdr + IDX_TAB_HDR + 5ll * nnz_s);
+    const long long w = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (w >= idx_bm_words(rows)) return;
+    const int nr = hdr[1];
+    const long long p0 = 32 * w, p1 = p0 + 32;
+    int lo = 0, hi = nr;                       // first range with run_e > p0
+    while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (run_e[mid] > p0) hi = mid; else lo = mid + 1;
+    }
+    uint32_t bits = 0;
+    for (int r = lo; r < nr; ++r) {
+        const long long a = run_a[r], e = run_e[r];
+        if (a >= p1) break;
+        const int from = (int)(max(a, p0) - p0), to = (int)(min(e, p1) - p0);      // [from, to) inside the word
+        if (to > from) bits |= (to - from >= 32 ? 0xffffffffu : ((1u << (to - from)) - 1u)) << from;
+    }
+    bm[w] = bits;
 }
 
 __global__ __launch_bounds__(IDX_WAVES *MINF_WAVE) void vs_index_fast_kernel(
@@ -307,9 +370,10 @@ __global__ __launch_bounds__(IDX_WAVES *MINF_WAVE) void vs_index_fast_kernel(
     int32_t *ci_row = column_index + ro * (long long)nnz_v;
     const int32_t *vert = vertical + bh * (long long)nnz_v;
     const int32_t *sl = slash + bh * (long long)nnz_s;
-    const int32_t *hdr = tables + bh * idx_tab_ints(nnz_s);
+    const int32_t *hdr = tables + bh * idx_tab_ints(nnz_s, rows);
     const int32_t *cpos = hdr + IDX_TAB_HDR, *cpre = cpos + nnz_s, *crun = cpre + nnz_s;
     const int32_t *run_a = crun + nnz_s, *run_e = run_a + nnz_s;
+    const uint32_t *bm = reinterpret_cast<const uint32_t *>(run_e + nnz_s);
 
     const int seqlen = seqlens[b];
     const int start_m = m * 64;
@@ -322,17 +386,31 @@ __global__ __launch_bounds__(IDX_WAVES *MINF_WAVE) void vs_index_fast_kernel(
     // loads that do not depend on each other, issued together (the kernel is bound by chains of
     // dependent loads, not by bandwidth)
     const int o_first = sl[0], o_last = sl[nnz_s - 1];
-    const int tab_blocks = hdr[0], tab_runs = hdr[1], tab_v = hdr[2];
+    const int tab_blocks = hdr[0], tab_runs = hdr[1], tab_v = hdr[2], bm_ok = hdr[3];
     const bool whole_list = o_first <= end_m - 64;      // nothing skipped, nothing clipped
 
     int s0 = nnz_s;
     if (live) {
-        int lo = 0, hi = whole_list ? 0 : nnz_s;        // first entry with an offset below end_m
-        while (lo < hi) {
-            int mid = (lo + hi) >> 1;
-            if (sl[mid] >= end_m) lo = mid + 1; else hi = mid;
+        // first entry with an offset below end_m = number of entries >= end_m (descending list):
+        // 64 samples one stride apart locate the segment, the lanes then count inside it -- two
+        // rounds of independent loads instead of a 13-step chain of dependent ones
+        s0 = 0;
+        if (!whole_list) {
+            const int stride = (nnz_s + MINF_WAVE - 1) / MINF_WAVE;
+            const int si = min(lane * stride, nnz_s - 1);
+            const bool above = lane * stride < nnz_s && sl[si] >= end_m;
+            const int nseg = __builtin_popcountll(__ballot(above));       // samples 0..nseg-1 are >= end_m
+            if (nseg > 0) {
+                const int seg = (nseg - 1) * stride;                      // entries [0, seg] are >= end_m
+                int cnt = 0;
+                for (int i0 = 0; i0 < stride; i0 += MINF_WAVE) {        // same trip count in every lane
+                    const int idx = seg + i0 + lane;
+                    const bool ab = i0 + lane < stride && idx < nnz_s && sl[idx] >= end_m;
+                    cnt += __builtin_popcountll(__ballot(ab));
+                }
+                s0 = seg + cnt;
+            }
         }
-        s0 = lo;
         if (s0 >= nnz_s) {           // the reference would read past the list here
             live = false;
             if (error_flag && lane == 0) *error_flag = 1;
@@ -433,33 +511,46 @@ __global__ __launch_bounds__(IDX_WAVES *MINF_WAVE) void vs_index_fast_kernel(
             const int shift = end_m - tab_v;
             const int k0 = g == 0 ? 0 : cpre[g], r0 = g == 0 ? 0 : crun[g];   // entry 0 starts range 0
             const int nblk = tab_blocks - k0, nruns = tab_runs;
-            for (int k = lane; k < nblk; k += MINF_WAVE) bo_row[nb + k] = cpos[k0 + k] + shift;
+            copy_shifted(bo_row + nb, cpos + k0, nblk, shift, lane);
             nb += nblk;
             const int t_end = end_m - o_last;             // t of the last entry (not clipped here)
             const int first_a = run_a[r0];                // start of the first remaining range
+            // four batches of 64 verticals per round: their loads and their coverage look-ups are
+            // independent, only the ordered emit is sequential
             while (vp < nnz_v) {
-                const int x = (vp + lane < nnz_v) ? vert[vp + lane] : INT_MAX;
-                const bool ok = x < t_end;
-                const int k = __builtin_popcountll(__ballot(ok));
-                bool emit = false;
-                if (ok && x >= e_lim) {
-                    const int xv = x - shift;
-                    if (xv < first_a) {                       // below every remaining range: no search
-                        emit = true;
-                    } else {
-                        int lo = r0, hi = nruns;              // first range >= r0 that ends after xv
-                        while (lo < hi) {
-                            int mid = (lo + hi) >> 1;
-                            if (run_e[mid] > xv) hi = mid; else lo = mid + 1;
+                int x[4];
+                bool emit[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) x[u] = (vp + u * MINF_WAVE + lane < nnz_v) ? vert[vp + u * MINF_WAVE + lane] : INT_MAX;
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    emit[u] = false;
+                    if (x[u] < t_end && x[u] >= e_lim) {
+                        const int xv = x[u] - shift;
+                        if (xv < first_a) {                   // below every remaining range
+                            emit[u] = true;
+                        } else if (bm_ok) {                   // xv < tab_v: inside the bitmap
+                            emit[u] = !((bm[xv >> 5] >> (xv & 31)) & 1u);
+                        } else {
+                            int lo = r0, hi = nruns;          // first range >= r0 that ends after xv
+                            while (lo < hi) {
+                                int mid = (lo + hi) >> 1;
+                                if (run_e[mid] > xv) hi = mid; else lo = mid + 1;
+                            }
+                            emit[u] = !(lo < nruns && run_a[lo] <= xv);
                         }
-                        emit = !(lo < nruns && run_a[lo] <= xv);
                     }
                 }
-                const uint64_t em = __ballot(emit);
-                if (emit) ci_row[ncol + __builtin_popcountll(em & lt)] = x;
-                ncol += __builtin_popcountll(em);
-                vp += k;
-                if (k < MINF_WAVE) break;
+                bool more = true;
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const uint64_t em = __ballot(emit[u]);
+                    if (emit[u]) ci_row[ncol + __builtin_popcountll(em & lt)] = x[u];
+                    ncol += __builtin_popcountll(em);
+                    more = more && __builtin_popcountll(__ballot(x[u] < t_end)) == MINF_WAVE;
+                }
+                vp += 4 * MINF_WAVE;
+                if (!more) break;                             // verticals ascend: nothing further is below t_end
             }
         }
     }
@@ -498,9 +589,9 @@ extern "C" int minf_vs_index_build(const int32_t *seqlens, const int32_t *vertic
 }
 
 
-extern "C" size_t minf_vs_index_workspace_bytes(int batch, int heads, int nnz_s) {
-    if (batch <= 0 || heads <= 0 || nnz_s <= 0) return 0;
-    return (size_t)batch * heads * (IDX_TAB_HDR + 5 * (size_t)nnz_s) * sizeof(int32_t);
+extern "C" size_t minf_vs_index_workspace_bytes(int batch, int heads, int nnz_s, int rows) {
+    if (batch <= 0 || heads <= 0 || nnz_s <= 0 || rows < 0) return 0;
+    return (size_t)batch * heads * (size_t)idx_tab_ints(nnz_s, rows) * sizeof(int32_t);
 }
 
 extern "C" int minf_vs_index_build_ws(const int32_t *seqlens, const int32_t *vertical_idx,
@@ -515,14 +606,19 @@ extern "C" int minf_vs_index_build_ws(const int32_t *seqlens, const int32_t *ver
     if (batch < 0 || heads < 0 || rows < 0 || nnz_v < 1 || nnz_s < 1) return MINF_ERR_INVALID_ARG;
     const long long total = (long long)batch * heads * rows;
     if (total == 0) return MINF_OK;
-    if (!workspace || workspace_bytes < minf_vs_index_workspace_bytes(batch, heads, nnz_s) ||
+    if (!workspace || workspace_bytes < minf_vs_index_workspace_bytes(batch, heads, nnz_s, rows) ||
         ((uintptr_t)workspace & 3))
         return MINF_ERR_WORKSPACE;
     const long long nblk = (total + IDX_WAVES - 1) / IDX_WAVES;
     if (nblk > 0x7fffffffLL || (long long)batch * heads > 0x7fffffffLL) return MINF_ERR_UNSUPPORTED;
     hipLaunchKernelGGL(vs_index_prep_kernel, dim3((unsigned)(batch * heads)), dim3(MINF_WAVE), 0,
-                       (hipStream_t)stream, slash_idx, (int32_t *)workspace, nnz_s);
+                       (hipStream_t)stream, slash_idx, (int32_t *)workspace, nnz_s, rows);
     int status = minf_launch_status();
+    if (status != MINF_OK) return status;
+    if ((long long)batch * heads > 65535) return MINF_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(vs_index_bitmap_kernel, dim3((unsigned)((idx_bm_words(rows) + 255) / 256), (unsigned)(batch * heads)),
+                       dim3(256), 0, (hipStream_t)stream, (int32_t *)workspace, nnz_s, rows);
+    status = minf_launch_status();
     if (status != MINF_OK) return status;
     hipLaunchKernelGGL(vs_index_fast_kernel, dim3((unsigned)nblk), dim3(IDX_WAVES * MINF_WAVE), 0,
                        (hipStream_t)stream, seqlens, vertical_idx, slash_idx, (const int32_t *)workspace,

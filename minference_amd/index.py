@@ -47,7 +47,7 @@ def convert_vertical_slash_indexes(seqlens, vertical_indexes, slash_indexes, con
         raise ValueError("batch/head sizes of seqlens, vertical_indexes, slash_indexes differ")
     rows = (int(context_size) + 63) // 64
     dev = v.device
-    alloc = torch.zeros if False else torch.empty   # the kernel writes every element itself
+    alloc = torch.empty                              # the kernel writes every element itself
     block_count = alloc((B, H, rows), dtype=torch.int32, device=dev)
     block_offset = alloc((B, H, rows, S), dtype=torch.int32, device=dev)
     column_count = alloc((B, H, rows), dtype=torch.int32, device=dev)
@@ -63,7 +63,7 @@ def convert_vertical_slash_indexes(seqlens, vertical_indexes, slash_indexes, con
             error_flag.data_ptr() if error_flag is not None else None)
     with torch.cuda.device(dev):
         if use_tables:
-            ws_bytes = lib.minf_vs_index_workspace_bytes(B, H, S)
+            ws_bytes = lib.minf_vs_index_workspace_bytes(B, H, S, rows)
             ws = torch.empty(max(ws_bytes, 4), dtype=torch.uint8, device=dev)
             st = lib.minf_vs_index_build_ws(*args, ws.data_ptr(), ws_bytes, _lib.stream_ptr(dev))
         else:
