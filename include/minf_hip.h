@@ -202,6 +202,17 @@ int minf_topk_indices(const float *scores, int rows, int n, int64_t row_stride, 
                       int32_t *out, int64_t out_stride, int reverse_base, void *stream);
 
 /*
+ * minf_topk_indices for block-causal score rows of at most 4096 entries (the block scores of
+ * block-sparse attention, reference minference/ops/block_sparse_flash_attention.py:161-166):
+ * row r belongs to query block m = r % rows_per_head, entries above the diagonal are -inf by
+ * construction and only the first 32 * (m / 32 + 1) entries of a row need to be stored; the rest
+ * is never read and counts as -inf.  Same selection and order as minf_topk_indices on the fully
+ * stored rows.  n > 4096 returns MINF_ERR_UNSUPPORTED.
+ */
+int minf_topk_indices_block_causal(const float *scores, int rows, int n, int64_t row_stride, int k,
+                                   int32_t *out, int64_t out_stride, int rows_per_head, void *stream);
+
+/*
  * Two selections of minf_topk_indices in one launch (same rows / n / row_stride; separate k,
  * output and reverse_base): the vertical and the slash top-k of a layer
  * (reference minference/modules/minference_forward.py:607 and :612).

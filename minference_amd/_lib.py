@@ -33,6 +33,7 @@ SIGNATURES = {
     "minf_vs_estimate": (c_int, [c_ptr, c_ptr, c_ptr, c_ptr] + [c_int] * 6 + [c_f32] + [c_int] * 3
                          + [c_ptr, c_ptr, c_ptr, ctypes.c_size_t, c_ptr]),
     "minf_topk_indices": (c_int, [c_ptr, c_int, c_int, c_i64, c_int, c_ptr, c_i64, c_int, c_ptr]),
+    "minf_topk_indices_block_causal": (c_int, [c_ptr, c_int, c_int, c_i64, c_int, c_ptr, c_i64, c_int, c_ptr]),
     "minf_topk_indices_pair": (c_int, [c_ptr, c_int, c_ptr, c_i64, c_int] * 2 + [c_int, c_int, c_i64, c_ptr]),
     "minf_bs_block_index_rows": (c_int, [c_int]),
     "minf_bs_block_index_workspace_bytes": (ctypes.c_size_t, [c_int] * 4),

@@ -20,6 +20,8 @@
 
 extern "C" int minf_topk_indices(const float *scores, int rows, int n, int64_t row_stride, int k,
                                  int32_t *out, int64_t out_stride, int reverse_base, void *stream);
+extern "C" int minf_topk_indices_block_causal(const float *scores, int rows, int n, int64_t row_stride, int k,
+                                              int32_t *out, int64_t out_stride, int rows_per_head, void *stream);
 
 namespace {
 
@@ -87,6 +89,7 @@ struct ScoreParams {
     float *scores;            // [batch*heads_q, rows, pitch]
     int heads_q, heads_kv, rows, pitch, force;
     int mtiles, ntiles;
+    int skip_masked;
 };
 
 // lane l supplies row l%32 and, for MFMA step (s, j), contraction index 8*s + 4*(l/32) + j:
@@ -113,6 +116,9 @@ __global__ __launch_bounds__(256) void bs_scores_kernel(const ScoreParams p) {
     load_operand(qbase, m0 + l32, p.rows, g, aq);             // A operand: query blocks -> accumulator rows
     for (int nt = wave; nt < p.ntiles; nt += 4) {
         const int n0 = nt * 32;
+        // tiles wholly above the diagonal hold only -inf: when the selection that follows knows
+        // that (rows of at most 4096 scores), they are neither computed nor stored
+        if (p.skip_masked && n0 > m0 + 31) continue;
         f32x16_t acc;
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[r] = 0.f;
@@ -191,13 +197,16 @@ int block_index_impl(const void *q, const void *k, const int64_t *q_stride, cons
     int status = minf_launch_status();
     if (status != MINF_OK) return status;
 
+    const bool causal_topk = rows <= 64 * 64;      // one wave per row: reads only the stored prefix of a row
     ScoreParams sp{qp, kp, scores, heads_q, heads_kv, rows, pitch, force_diag_first ? 1 : 0,
-                   (rows + 31) / 32, (pitch + 31) / 32};
+                   (rows + 31) / 32, (pitch + 31) / 32, causal_topk ? 1 : 0};
     hipLaunchKernelGGL(bs_scores_kernel, dim3(sp.mtiles, batch * heads_q), dim3(256), 0, st, sp);
     status = minf_launch_status();
     if (status != MINF_OK) return status;
 
     const int kk = top_k < rows ? top_k : rows;
+    if (causal_topk)
+        return minf_topk_indices_block_causal(scores, batch * heads_q * rows, rows, pitch, kk, block_index, kk, rows, stream);
     return minf_topk_indices(scores, batch * heads_q * rows, rows, pitch, kk, block_index, kk, -1, stream);
 }
 

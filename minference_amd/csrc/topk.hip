@@ -33,6 +33,9 @@ struct TopkProblem {
     int32_t *out;
     long long out_stride;
     int reverse_base;
+    // block-causal score rows (wave kernel only): row r belongs to query block m = r % causal_rows and
+    // only its first 32 * (m / 32 + 1) entries are stored; the rest counts as -inf.  0 = plain rows
+    int causal_rows;
 };
 
 // blockIdx.y selects one of two problems over rows of the same length n (vertical and slash
@@ -194,12 +197,15 @@ __global__ __launch_bounds__(TK_THREADS) void topk_kernel(const TopkProblem p0, 
 
 // Short rows (n <= 64 * ITEMS <= 4096, e.g. the block scores of block-sparse attention): one
 // wavefront per row, the row held in registers (lane l owns indices l, l+64, ...).  The k-th
-// largest key is found bit by bit: T = the largest value with count(key >= T) >= k, 32 counting
-// passes of one compare + ballot popcount per element (no LDS, no barriers); the emit is the same
-// ordered ballot-prefix write as in the wide kernel, so both kernels select identical sets.
+// largest key is found bit by bit: T = the largest value with count(key >= T) >= k, one counting
+// pass per bit below the bits all live keys share, stopping as soon as a count hits k exactly
+// (no LDS, no barriers); the emit is the same ordered ballot-prefix write as in the wide kernel, so
+// both kernels select identical sets.
 constexpr int TKW_WAVES = 4;
+// (the second launch bound is the number of resident waves per SIMD the register budget must allow:
+// the kernel is latency bound, and left alone the 64-item variant took 141 registers = 3 waves)
 template <int ITEMS>
-__global__ __launch_bounds__(TKW_WAVES * 64) void topk_wave_kernel(const TopkProblem p0, const TopkProblem p1,
+__global__ __launch_bounds__(TKW_WAVES * 64, ITEMS >= 64 ? 3 : (ITEMS >= 40 ? 5 : 8)) void topk_wave_kernel(const TopkProblem p0, const TopkProblem p1,
                                                                    int n, int rows) {
     const TopkProblem &pr = blockIdx.y == 0 ? p0 : p1;
     const int lane = (int)threadIdx.x & 63, wave = (int)threadIdx.x >> 6;
@@ -212,17 +218,19 @@ __global__ __launch_bounds__(TKW_WAVES * 64) void topk_wave_kernel(const TopkPro
         for (int i = lane; i < n; i += 64) o[i] = reverse_base >= 0 ? reverse_base - i : i;
         return;
     }
+    constexpr unsigned KEY_FLOOR = 0x007fffffu;          // order_key(-inf)
+    const int stored = pr.causal_rows > 0 ? min(n, 32 * ((row % pr.causal_rows) / 32 + 1)) : n;
     unsigned key[ITEMS];
 #pragma unroll
     for (int j = 0; j < ITEMS; ++j) {
         const int i = j * 64 + lane;
-        key[j] = i < n ? order_key(x[i]) : 0u;      // padding sorts below every real score
+        // padding sorts below every real score; entries that are not stored are -inf
+        key[j] = i < stored ? order_key(x[i]) : (i < n ? KEY_FLOOR : 0u);
     }
     // Rows with a masked (-inf) tail, e.g. block-causal score rows: when at least k entries are above
     // -inf, the threshold is too, and register groups that hold nothing above -inf can be skipped
     // in every pass and in the emit (they add nothing to a count of keys >= cand > key(-inf), and
     // for cand <= key(-inf) the live groups alone already reach k).
-    constexpr unsigned KEY_FLOOR = 0x007fffffu;          // order_key(-inf)
     constexpr int GROUP = ITEMS >= 8 ? 8 : ITEMS;
     int nfin = 0, jmax = 0;
 #pragma unroll
@@ -231,19 +239,47 @@ __global__ __launch_bounds__(TKW_WAVES * 64) void topk_wave_kernel(const TopkPro
         nfin += c;
         if (c) jmax = j + 1;
     }
-    if (nfin < k) jmax = ITEMS;
-    unsigned T = 0;
-    for (int bit = 31; bit >= 0; --bit) {
+    const bool with_floor = nfin < k;                // masked / padding entries take part in the selection
+    if (with_floor) jmax = ITEMS;
+    // Keys that can be the threshold lie between the smallest and the largest live key: the bits
+    // those two share are bits of T, the search starts below them.
+    unsigned kmax = 0u, kmin = 0xffffffffu;
+#pragma unroll
+    for (int jb = 0; jb < ITEMS; jb += GROUP) {
+        if (jb < jmax) {
+#pragma unroll
+            for (int j = jb; j < jb + GROUP; ++j) {
+                kmax = max(kmax, key[j]);
+                kmin = min(kmin, (with_floor || key[j] > KEY_FLOOR) ? key[j] : 0xffffffffu);
+            }
+        }
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+        kmax = max(kmax, (unsigned)__shfl_xor((int)kmax, d));
+        kmin = min(kmin, (unsigned)__shfl_xor((int)kmin, d));
+    }
+    const unsigned diff = kmax ^ kmin;
+    const int top_bit = diff ? 31 - __builtin_clz(diff) : -1;            // highest bit in which live keys differ
+    unsigned T = top_bit >= 0 ? (top_bit == 31 ? 0u : (kmax >> (top_bit + 1)) << (top_bit + 1)) : kmax;
+    for (int bit = top_bit; bit >= 0; --bit) {
         const unsigned cand = T | (1u << bit);
-        int cnt = 0;
+        // every lane counts its own keys (compare + add with carry), the lane counts (< 128) are
+        // summed through seven ballots of their bits
+        int c = 0;
 #pragma unroll
         for (int jb = 0; jb < ITEMS; jb += GROUP) {
             if (jb < jmax) {
 #pragma unroll
-                for (int j = jb; j < jb + GROUP; ++j) cnt += __builtin_popcountll(__ballot(key[j] >= cand));
+                for (int j = jb; j < jb + GROUP; ++j) c += key[j] >= cand ? 1 : 0;
             }
         }
+        int cnt = 0;
+#pragma unroll
+        for (int b = 0; b < (ITEMS >= 64 ? 7 : (ITEMS >= 32 ? 6 : (ITEMS >= 16 ? 5 : 3))); ++b)
+            cnt += __builtin_popcountll(__ballot((c >> b) & 1)) << b;
         if (cnt >= k) T = cand;
+        if (cnt == k) break;                         // exactly k keys are >= T: nothing left to decide
     }
     int cgt = 0;
 #pragma unroll
@@ -282,6 +318,8 @@ void launch_topk(const TopkProblem &pa, const TopkProblem &pb, int problems, int
         hipLaunchKernelGGL(topk_wave_kernel<4>, grid_w, dim3(TKW_WAVES * 64), 0, st, pa, pb, n, rows);
     else if (n <= 64 * 16)
         hipLaunchKernelGGL(topk_wave_kernel<16>, grid_w, dim3(TKW_WAVES * 64), 0, st, pa, pb, n, rows);
+    else if (n <= 64 * 40)
+        hipLaunchKernelGGL(topk_wave_kernel<40>, grid_w, dim3(TKW_WAVES * 64), 0, st, pa, pb, n, rows);
     else if (n <= 64 * 64)
         hipLaunchKernelGGL(topk_wave_kernel<64>, grid_w, dim3(TKW_WAVES * 64), 0, st, pa, pb, n, rows);
     else
@@ -295,7 +333,18 @@ extern "C" int minf_topk_indices(const float *scores, int rows, int n, int64_t r
     if (!scores || !out || rows < 0 || n <= 0 || k <= 0) return MINF_ERR_INVALID_ARG;
     if (row_stride < n || out_stride < (k < n ? k : n)) return MINF_ERR_INVALID_ARG;
     if (rows == 0) return MINF_OK;
-    TopkProblem p{scores, (long long)row_stride, k, out, (long long)out_stride, reverse_base};
+    TopkProblem p{scores, (long long)row_stride, k, out, (long long)out_stride, reverse_base, 0};
+    launch_topk(p, p, 1, rows, n, (hipStream_t)stream);
+    return minf_launch_status();
+}
+
+extern "C" int minf_topk_indices_block_causal(const float *scores, int rows, int n, int64_t row_stride, int k,
+                                              int32_t *out, int64_t out_stride, int rows_per_head, void *stream) {
+    if (!scores || !out || rows < 0 || n <= 0 || k <= 0 || rows_per_head <= 0) return MINF_ERR_INVALID_ARG;
+    if (row_stride < n || out_stride < (k < n ? k : n)) return MINF_ERR_INVALID_ARG;
+    if (n > 64 * 64) return MINF_ERR_UNSUPPORTED;      // only the one-wave-per-row kernel knows about stored prefixes
+    if (rows == 0) return MINF_OK;
+    TopkProblem p{scores, (long long)row_stride, k, out, (long long)out_stride, -1, rows_per_head};
     launch_topk(p, p, 1, rows, n, (hipStream_t)stream);
     return minf_launch_status();
 }
@@ -309,8 +358,8 @@ extern "C" int minf_topk_indices_pair(const float *scores_a, int k_a, int32_t *o
     if (row_stride < n || out_stride_a < (k_a < n ? k_a : n) || out_stride_b < (k_b < n ? k_b : n))
         return MINF_ERR_INVALID_ARG;
     if (rows == 0) return MINF_OK;
-    TopkProblem pa{scores_a, (long long)row_stride, k_a, out_a, (long long)out_stride_a, reverse_base_a};
-    TopkProblem pb{scores_b, (long long)row_stride, k_b, out_b, (long long)out_stride_b, reverse_base_b};
+    TopkProblem pa{scores_a, (long long)row_stride, k_a, out_a, (long long)out_stride_a, reverse_base_a, 0};
+    TopkProblem pb{scores_b, (long long)row_stride, k_b, out_b, (long long)out_stride_b, reverse_base_b, 0};
     launch_topk(pa, pb, 2, rows, n, (hipStream_t)stream);
     return minf_launch_status();
 }
