@@ -45,6 +45,21 @@ def test_random_lists(gpu, heads, n, nv, ns, seed):
     assert_same(run_gpu([n], v, s, n, gpu), ref)
 
 
+@pytest.mark.parametrize("n,smax,ns,nv", [(1024, 9000, 300, 60), (4096, 4160, 129, 500), (2000, 200000, 64, 1000)])
+def test_offsets_beyond_the_context(gpu, n, smax, ns, nv):
+    """Slash offsets far larger than the context (every row block skips most of the list): the
+    per-head table then spans more positions than the coverage bitmap holds, and the row blocks
+    fall back to searching the tabulated ranges.  Same tensors as the oracle either way."""
+    rng = np.random.default_rng(n + ns)
+    for h_seed in range(3):
+        big = rng.choice(np.arange(64, smax), size=ns - 40, replace=False)
+        sl = np.sort(np.concatenate([np.arange(40), big]))[::-1].astype(np.int32)
+        vl = np.sort(rng.choice(n, size=min(nv, n), replace=False)).astype(np.int32)
+        v, s = vl[None, None, :].copy(), sl[None, None, :].copy()
+        ref = O.vs_index_build([n], v, s, n)
+        assert_same(run_gpu([n], v, s, n, gpu), ref)
+
+
 @pytest.mark.parametrize("mode", [0, 1, 2, 3])
 def test_structured_lists_all_rows(gpu, mode):
     """Slash lists that stress the table-driven path: clusters with gaps just below / above the
