@@ -4,7 +4,8 @@ Counterpart of ``minference_prefill_kernel`` / ``minference_prefill_forward``
 (reference minference/modules/minference_forward.py:594-674) with the same
 ``prefill_kwargs`` dictionary: ``layer_idx`` and ``attn_forward_config`` with
 ``best_pattern`` (list over layers of ``{"<head>": [type, vertical_size,
-slash_size, score]}``), ``starting_layer`` and ``minference_ratio``.  Heads are
+slash_size, score]}``), ``starting_layer``, ``minference_ratio`` and the search mode
+(``is_search``, ``config_path``, with ``num_hidden_layers`` in ``prefill_kwargs``).  Heads are
 grouped by (pattern, sizes) and every group is one batched launch sequence
 instead of the reference's Python loop over heads.  K/V may have fewer heads
 than Q (no repeat_kv needed).
@@ -12,6 +13,7 @@ than Q (no repeat_kv needed).
 from __future__ import annotations
 
 import json
+import os
 
 import torch
 
@@ -78,15 +80,40 @@ def minference_prefill_kernel(q, k, v, pattern, vertical_size, slash_size):
     raise KeyError(pattern)
 
 
+def _search_layer(query_states, key_states, value_states, prefill_kwargs):
+    """Search mode (minference_forward.py:644-673): the layer's per-head patterns are searched
+    and appended to the JSON list at ``config_path`` (one ``{head: [type, v, s, score]}`` object
+    per layer, in layer order), and the layer's output is dense causal attention.  A file that
+    already holds ``num_hidden_layers`` layers raises, like the reference; layers the file
+    already holds are not searched again."""
+    from .search import search_patterns
+    config = prefill_kwargs["attn_forward_config"]
+    layer_idx = prefill_kwargs["layer_idx"]
+    config_path = config.get("config_path", None)
+    config_list = []
+    if config_path and os.path.isfile(config_path):
+        with open(config_path) as f:
+            config_list = json.load(f)
+        if len(config_list) == prefill_kwargs.get("num_hidden_layers", -1):
+            raise RuntimeError(f"Search already completed; see {config_path}.")
+    if layer_idx >= len(config_list):
+        new_config = search_patterns(query_states, key_states)
+        if config_path:
+            config_list.append(new_config)
+            with open(config_path, "w") as f:
+                json.dump(config_list, f, indent=2)
+    return dense_causal_attention(query_states, key_states, value_states)
+
+
 def minference_prefill_forward(query_states, key_states, value_states, prefill_kwargs):
     """Sparse prefill attention of one layer: [B,Hq,N,D] x [B,Hk,N,D] -> [B,Hq,N,D]."""
     config = prefill_kwargs["attn_forward_config"]
     layer_idx = prefill_kwargs["layer_idx"]
     starting_layer = config.get("starting_layer", 0)
-    if config.get("is_search", False):
-        raise NotImplementedError("offline pattern search is not part of this package")
     B, H, N, D = query_states.shape
     group = H // key_states.shape[1]
+    if config.get("is_search", False):
+        return _search_layer(query_states, key_states, value_states, prefill_kwargs)
     if layer_idx < starting_layer:
         return dense_causal_attention(query_states, key_states, value_states)
     plan = _head_plan(config, layer_idx, H)

@@ -127,3 +127,30 @@ def test_deterministic(gpu):
     a = pattern_recall(q.to(gpu), k.to(gpu), row_begin=500)
     b = pattern_recall(q.to(gpu), k.to(gpu), row_begin=500)
     assert torch.equal(a, b)
+
+
+def test_search_mode_of_the_dispatcher_writes_the_pattern_file(gpu, tmp_path):
+    """minference_forward.py:644-673: with is_search every layer's heads are searched, the result
+    is appended to config_path, the layer's output is dense causal attention; the finished file
+    drives the sparse dispatcher."""
+    import json
+    from minference_amd import dense_causal_attention, minference_prefill_forward
+    n = 2900
+    q, k = heads(n, 4, 2, 17)
+    v = torch.randn(1, 2, n, 128, generator=torch.Generator().manual_seed(3)).bfloat16()
+    qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
+    path = tmp_path / "best_pattern.json"
+    cfg = {"is_search": True, "config_path": str(path)}
+    dense = dense_causal_attention(qg, kg, vg)
+    for layer in range(2):
+        out = minference_prefill_forward(qg, kg, vg, {"layer_idx": layer, "num_hidden_layers": 2, "attn_forward_config": cfg})
+        assert torch.equal(out, dense)
+    table = json.loads(path.read_text())
+    assert len(table) == 2 and sorted(table[0]) == ["0", "1", "2", "3"]
+    for h in range(4):
+        want = O.search_pattern(q[0, h].float(), k[0, h // 2].float())
+        assert tuple(table[1][str(h)][:3]) == want[:3]
+    with pytest.raises(RuntimeError, match="Search already completed"):
+        minference_prefill_forward(qg, kg, vg, {"layer_idx": 0, "num_hidden_layers": 2, "attn_forward_config": cfg})
+    sparse = minference_prefill_forward(qg, kg, vg, {"layer_idx": 1, "attn_forward_config": {"best_pattern": table}})
+    assert sparse.shape == dense.shape and torch.isfinite(sparse.float()).all()

@@ -43,11 +43,16 @@ def test_kv_head_selection_for_gqa_groups():
     assert prefill._kv_for_heads(k, [2, 7], 1).flatten().tolist() == [2, 7]
 
 
-def test_is_search_is_rejected():
-    with pytest.raises(NotImplementedError):
-        prefill.minference_prefill_forward(torch.zeros(1, 1, 64, 128), torch.zeros(1, 1, 64, 128),
-                                           torch.zeros(1, 1, 64, 128),
-                                           {"layer_idx": 0, "attn_forward_config": {"is_search": True}})
+def test_search_mode_has_no_cpu_path_and_respects_a_finished_file(tmp_path):
+    cfg_path = tmp_path / "patterns.json"
+    kw = {"layer_idx": 0, "num_hidden_layers": 2,
+          "attn_forward_config": {"is_search": True, "config_path": str(cfg_path)}}
+    z = torch.zeros(1, 1, 64, 128)
+    with pytest.raises(RuntimeError):                     # CPU tensors: the search kernels need the GPU
+        prefill.minference_prefill_forward(z, z, z, kw)
+    cfg_path.write_text('[{"0": ["vertical_and_slash", 30, 800, 0.9]}, {"0": ["vertical_and_slash", 30, 800, 0.9]}]')
+    with pytest.raises(RuntimeError, match="Search already completed"):
+        prefill.minference_prefill_forward(z, z, z, kw)
 
 
 def test_shipped_pattern_files_have_the_expected_format():
