@@ -16,6 +16,7 @@ from .estimate import estimate_vertical_slash, topk_indices, vertical_slash_scor
 from .prefill import (load_best_pattern, minference_prefill_forward, minference_prefill_kernel,
                       vertical_slash_prefill)
 from .search import pattern_recall, search_pattern, search_patterns
+from .patch import MInference, MInferenceConfig
 
 __all__ = [
     "estimate_vertical_slash", "vertical_slash_scores", "topk_indices", "vertical_slash_prefill",
@@ -23,6 +24,6 @@ __all__ = [
     "vertical_slash_sparse_attention", "block_sparse_attention", "streaming_forward",
     "convert_vertical_slash_indexes", "vertical_slash_attention_from_index",
     "block_sparse_attention_from_index", "dense_causal_attention", "tri_shape_forward",
-    "pattern_recall", "search_pattern", "search_patterns",
+    "pattern_recall", "search_pattern", "search_patterns", "MInference", "MInferenceConfig",
 ]
 __version__ = "0.1.0"

@@ -1,0 +1,135 @@
+"""``MInference(attn_type, model_name, ...)(model)`` -- the reference's patch entry point for
+Hugging Face models, on this package's kernels.
+
+Counterpart of ``MInference`` / ``MInferenceConfig`` (reference minference/models_patch.py:18-160,
+minference/minference_configuration.py:7-100) and of the attention forward the patch installs
+(minference/modules/forward.py:22-234, which hands ``[B, H, N, D]`` q/k/v to
+``prefill_forwards[attn_type]``).  The reference replaces ``forward`` methods of a particular
+transformers release; here the hook is transformers' own attention-function registry
+(``AttentionInterface``): an attention function named ``"minference_amd"`` is registered and the
+model is switched to it, so every decoder architecture whose attention module goes through that
+registry (Llama, Qwen2, Mistral, ...) is covered without touching its code.  The function
+receives K/V with their own (fewer) heads -- no ``repeat_kv`` copy is ever made.
+
+Scope: the prefill of one unpadded sequence (what the reference's prefill path assumes as well).
+Decode steps and chunks that attend to a longer cache (``key length != query length``) are passed
+to transformers' SDPA function unchanged.  KV-cache compression (``kv_type``), CPU KV offload and
+the reference's other attention types belong to other paths of the reference and raise.
+"""
+from __future__ import annotations
+
+import json
+
+SUPPORTED_ATTN_TYPES = ("minference", "dense", "a_shape", "tri_shape", "hf")
+INTERFACE_NAME = "minference_amd"
+_registered = False
+
+
+class MInferenceConfig:
+    """Same constructor arguments as the reference's configuration object
+    (minference_configuration.py:43-55); unsupported choices raise instead of being ignored."""
+
+    def __init__(self, attn_type="minference", model_name=None, config_path=None, starting_layer=-1,
+                 kv_cache_cpu=False, kv_type="dense", is_search=False, attn_kwargs=None, **kwargs):
+        if attn_type not in SUPPORTED_ATTN_TYPES:
+            raise NotImplementedError(
+                f"attn_type {attn_type!r}: this package implements {SUPPORTED_ATTN_TYPES} "
+                "(the dynamic sparse prefill path and its dense / A-shape / tri-shape relatives)")
+        if kv_type != "dense" or kv_cache_cpu:
+            raise NotImplementedError("KV-cache compression and CPU offload are not part of the prefill path")
+        if kwargs:
+            raise TypeError(f"unknown arguments {sorted(kwargs)}")
+        self.attn_type = attn_type
+        self.model_name = model_name
+        self.config_path = config_path
+        self.starting_layer = starting_layer
+        self.is_search = is_search
+        self.attn_kwargs = dict(attn_kwargs or {})
+
+
+def _attention(module, query, key, value, attention_mask, dropout=0.0, scaling=None, **kwargs):
+    """The registered attention function: [B,H,N,D] q, [B,Hk,N,D] k/v -> ([B,N,H,D], None)."""
+    from .ops import dense_causal_attention, streaming_forward, tri_shape_forward
+    from .prefill import minference_prefill_forward
+    state = getattr(module.config, "minference_amd", None)
+    n = query.shape[2]
+    if state is None or n == 1 or key.shape[2] != n or not query.is_cuda:
+        from transformers.integrations.sdpa_attention import sdpa_attention_forward
+        return sdpa_attention_forward(module, query, key, value, attention_mask, dropout=dropout,
+                                      scaling=scaling, **kwargs)
+    d = query.shape[-1]
+    if scaling is not None and abs(scaling * d ** 0.5 - 1.0) > 1e-6:
+        query = query * (scaling * d ** 0.5)              # the kernels scale by 1/sqrt(head_dim)
+    ty = state["attn_type"]
+    kw = state["attn_kwargs"]
+    if ty == "minference":
+        out = minference_prefill_forward(query, key, value, {
+            "layer_idx": module.layer_idx, "num_hidden_layers": module.config.num_hidden_layers,
+            "attn_forward_config": kw})
+    elif ty == "dense":
+        out = dense_causal_attention(query, key, value)
+    elif ty == "a_shape":
+        out = streaming_forward(query, key, value, kw["n_init"], kw["n_local"])
+    else:
+        out = tri_shape_forward(query, key, value, kw["n_init"], kw["n_local"], kw["n_last"])
+    return out.transpose(1, 2), None
+
+
+def _register():
+    global _registered
+    if not _registered:
+        from transformers import AttentionInterface
+        AttentionInterface.register(INTERFACE_NAME, _attention)
+        _registered = True
+
+
+class MInference:
+    """``MInference("minference", model_name, config_path=...)(model)`` returns the model with its
+    attention switched to this package (models_patch.py:18-52).
+
+    * ``"minference"``: per-head patterns from the ``best_pattern`` JSON at ``config_path``
+      (``is_search=True``: search them instead, layer by layer, and write the file;
+      ``attn_kwargs`` may carry ``minference_ratio``); layers below ``starting_layer`` run dense.
+      Without a file every head uses vertical_and_slash (1000, 6096).
+    * ``"dense"``: dense causal attention on the same tile engine.
+    * ``"a_shape"`` / ``"tri_shape"``: ``n_init`` (128), ``n_local`` (3968) and ``n_last`` (100)
+      from ``attn_kwargs`` (defaults of models_patch.py:134-143).
+    * ``"hf"``: the model is returned unchanged.
+    """
+
+    def __init__(self, attn_type="minference", model_name=None, config_path=None, starting_layer=-1,
+                 kv_cache_cpu=False, kv_type="dense", is_search=False, attn_kwargs=None, **kwargs):
+        self.config = MInferenceConfig(attn_type=attn_type, model_name=model_name, config_path=config_path,
+                                       starting_layer=starting_layer, kv_cache_cpu=kv_cache_cpu,
+                                       kv_type=kv_type, is_search=is_search, attn_kwargs=attn_kwargs, **kwargs)
+
+    def __call__(self, model):
+        return self.patch_model(model)
+
+    def patch_model(self, model):
+        c = self.config
+        if c.attn_type == "hf":
+            return model
+        kw = dict(c.attn_kwargs)
+        if c.attn_type == "minference":
+            kw.setdefault("starting_layer", c.starting_layer)
+            kw["is_search"] = bool(c.is_search)
+            kw["config_path"] = c.config_path
+            if not c.is_search and "best_pattern" not in kw:
+                if c.config_path:
+                    with open(c.config_path) as f:
+                        kw["best_pattern"] = json.load(f)
+                else:
+                    kw["best_pattern"] = None            # every head: vertical_and_slash (1000, 6096)
+            if c.is_search and not c.config_path:
+                raise ValueError("is_search needs a config_path to write the patterns to")
+        elif c.attn_type in ("a_shape", "tri_shape"):
+            kw.setdefault("n_local", 3968)
+            kw.setdefault("n_init", 128)
+            kw.setdefault("n_last", 100)
+        _register()
+        model.config.starting_layer = c.starting_layer       # models_patch.py:112-114
+        model.config.config_path = c.config_path
+        model.config.minference_amd = {"attn_type": c.attn_type, "attn_kwargs": kw}
+        model.set_attn_implementation(INTERFACE_NAME)
+        return model

@@ -1,0 +1,97 @@
+"""``MInference(...)(model)`` on a Hugging Face Llama (random init, transformers' own modelling
+code): the patch routes the prefill attention of every layer through this package.  Patterns that
+keep every causal key must reproduce the unpatched model (bf16 tolerance on the logits), sparse
+patterns must change them, generation (prefill + decode steps) must still work, and the search
+mode must write a pattern file the patch can load again."""
+import json
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def tiny_llama(gpu, layers=2):
+    from transformers import LlamaConfig, LlamaForCausalLM
+    torch.manual_seed(0)
+    cfg = LlamaConfig(vocab_size=320, hidden_size=512, intermediate_size=1024, num_hidden_layers=layers,
+                      num_attention_heads=4, num_key_value_heads=2, head_dim=128, max_position_embeddings=8192,
+                      rope_theta=500000.0)
+    return LlamaForCausalLM(cfg).to(gpu).to(torch.bfloat16).eval()
+
+
+def logits_of(model, ids):
+    with torch.no_grad():
+        return model(ids).logits.float()
+
+
+def close(a, b, what):
+    err = (a - b).abs()
+    scale = b.abs().max().item()
+    print(f"{what}: max-abs {err.max().item():.3e} of scale {scale:.3e}", flush=True)
+    assert err.max().item() <= 3e-2 * scale + 1e-2, what       # bf16 model, two layers
+
+
+def test_patterns_that_keep_everything_reproduce_the_unpatched_model(gpu, tmp_path):
+    from minference_amd import MInference
+    n = 700
+    ids = torch.randint(0, 320, (1, n), generator=torch.Generator().manual_seed(1)).to(gpu)
+    model = tiny_llama(gpu)
+    base = logits_of(model, ids)
+
+    dense = MInference("dense")(model)
+    assert dense.config._attn_implementation == "minference_amd"
+    close(logits_of(dense, ids), base, "dense")
+
+    # per-head table: a window wider than the sequence for some heads, vertical-slash with every
+    # diagonal for the others; layer 0 below starting_layer runs dense
+    table = [{str(h): (["stream_llm", 4, 4096, 1.0] if h % 2 else ["vertical_and_slash", 30, 100000, 1.0])
+              for h in range(4)} for _ in range(2)]
+    path = tmp_path / "patterns.json"
+    path.write_text(json.dumps(table))
+    mi = MInference("minference", "tiny-llama", config_path=str(path), starting_layer=1)(model)
+    close(logits_of(mi, ids), base, "minference (all-keeping patterns)")
+
+    tri = MInference("tri_shape", attn_kwargs={"n_init": 8, "n_local": 4096, "n_last": 64})(model)
+    close(logits_of(tri, ids), base, "tri_shape (window wider than the sequence)")
+
+
+def test_sparse_patterns_are_really_applied(gpu):
+    from minference_amd import MInference
+    n = 1500
+    ids = torch.randint(0, 320, (1, n), generator=torch.Generator().manual_seed(2)).to(gpu)
+    model = tiny_llama(gpu)
+    base = logits_of(model, ids)
+    a = MInference("a_shape", attn_kwargs={"n_init": 4, "n_local": 64})(model)
+    out = logits_of(a, ids)
+    assert torch.isfinite(out).all()
+    # rows inside the first window see every key: identical there, different far behind it
+    close(out[:, :60], base[:, :60], "a_shape, first rows")
+    assert (out[:, -200:] - base[:, -200:]).abs().max() > 5e-2
+
+
+def test_generate_runs_prefill_sparse_and_decode_through_transformers(gpu):
+    from minference_amd import MInference
+    n = 300
+    ids = torch.randint(0, 320, (1, n), generator=torch.Generator().manual_seed(3)).to(gpu)
+    model = tiny_llama(gpu)
+    want = model.generate(ids, max_new_tokens=4, do_sample=False)
+    got = MInference("dense")(model).generate(ids, max_new_tokens=4, do_sample=False)
+    assert got.shape == want.shape == (1, n + 4)
+    assert torch.equal(got[:, :n], ids)
+
+
+def test_search_mode_writes_a_table_the_patch_loads(gpu, tmp_path):
+    from minference_amd import MInference
+    n = 2900                                  # the search averages over rows >= 2500
+    ids = torch.randint(0, 320, (1, n), generator=torch.Generator().manual_seed(4)).to(gpu)
+    model = tiny_llama(gpu)
+    base = logits_of(model, ids)
+    path = tmp_path / "found.json"
+    searching = MInference("minference", config_path=str(path), is_search=True)(model)
+    close(logits_of(searching, ids), base, "search mode output is dense")
+    table = json.loads(path.read_text())
+    assert len(table) == 2 and all(sorted(layer) == ["0", "1", "2", "3"] for layer in table)
+    assert all(entry[0] == "vertical_and_slash" for layer in table for entry in layer.values())
+    sparse = MInference("minference", config_path=str(path))(model)
+    assert torch.isfinite(logits_of(sparse, ids)).all()

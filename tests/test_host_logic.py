@@ -99,3 +99,20 @@ def test_planted_layer_is_deterministic_and_structured():
     pos = (k[0, 0, :, -3].float() * 16384 + k[0, 0, :, -2].float() * 128 + k[0, 0, :, -1].float())
     assert torch.equal(pos, torch.arange(2048).float())
     assert len(meta["heavy"]) == 2 and len(meta["heavy"][0]) == 32
+
+
+def test_patch_configuration_rejects_what_is_not_built():
+    from minference_amd import MInference
+    for bad in ("inf_llm", "flexprefill", "vllm_minference", "dilated1"):
+        with pytest.raises(NotImplementedError):
+            MInference(bad)
+    with pytest.raises(NotImplementedError):
+        MInference("minference", kv_type="snapkv")
+    with pytest.raises(NotImplementedError):
+        MInference("minference", kv_cache_cpu=True)
+    with pytest.raises(TypeError):
+        MInference("minference", not_an_argument=1)
+    m = MInference("a_shape", attn_kwargs={"n_local": 100})
+    assert m.config.attn_type == "a_shape" and m.config.attn_kwargs == {"n_local": 100}
+    sentinel = object()
+    assert MInference("hf")(sentinel) is sentinel                     # "hf": model unchanged
