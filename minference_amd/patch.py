@@ -20,7 +20,7 @@ from __future__ import annotations
 
 import json
 
-SUPPORTED_ATTN_TYPES = ("minference", "dense", "a_shape", "tri_shape", "hf")
+SUPPORTED_ATTN_TYPES = ("minference", "tri_mix_minference", "tri_mix", "dense", "a_shape", "tri_shape", "hf")
 INTERFACE_NAME = "minference_amd"
 _registered = False
 
@@ -50,7 +50,7 @@ class MInferenceConfig:
 def _attention(module, query, key, value, attention_mask, dropout=0.0, scaling=None, **kwargs):
     """The registered attention function: [B,H,N,D] q, [B,Hk,N,D] k/v -> ([B,N,H,D], None)."""
     from .ops import dense_causal_attention, streaming_forward, tri_shape_forward
-    from .prefill import minference_prefill_forward
+    from .prefill import minference_prefill_forward, tri_mix_forward, tri_mix_minference_forward
     state = getattr(module.config, "minference_amd", None)
     n = query.shape[2]
     if state is None or n == 1 or key.shape[2] != n or not query.is_cuda:
@@ -62,8 +62,10 @@ def _attention(module, query, key, value, attention_mask, dropout=0.0, scaling=N
         query = query * (scaling * d ** 0.5)              # the kernels scale by 1/sqrt(head_dim)
     ty = state["attn_type"]
     kw = state["attn_kwargs"]
-    if ty == "minference":
-        out = minference_prefill_forward(query, key, value, {
+    if ty in ("minference", "tri_mix_minference", "tri_mix"):
+        fn = {"minference": minference_prefill_forward, "tri_mix_minference": tri_mix_minference_forward,
+              "tri_mix": tri_mix_forward}[ty]
+        out = fn(query, key, value, {
             "layer_idx": module.layer_idx, "num_hidden_layers": module.config.num_hidden_layers,
             "attn_forward_config": kw})
     elif ty == "dense":
@@ -91,6 +93,8 @@ class MInference:
       (``is_search=True``: search them instead, layer by layer, and write the file;
       ``attn_kwargs`` may carry ``minference_ratio``); layers below ``starting_layer`` run dense.
       Without a file every head uses vertical_and_slash (1000, 6096).
+    * ``"tri_mix_minference"`` / ``"tri_mix"``: the per-head patterns (resp. dense attention) below
+      ``attn_kwargs["starting_layer"]`` (16), tri-shape (n_init 8, n_local 512, n_last 128) from there on.
     * ``"dense"``: dense causal attention on the same tile engine.
     * ``"a_shape"`` / ``"tri_shape"``: ``n_init`` (128), ``n_local`` (3968) and ``n_last`` (100)
       from ``attn_kwargs`` (defaults of models_patch.py:134-143).
@@ -123,6 +127,18 @@ class MInference:
                     kw["best_pattern"] = None            # every head: vertical_and_slash (1000, 6096)
             if c.is_search and not c.config_path:
                 raise ValueError("is_search needs a config_path to write the patterns to")
+        elif c.attn_type in ("tri_mix_minference", "tri_mix"):
+            # models_patch.py:116-127: tri-shape (8 + 512, last 128 rows dense) from layer 16 on
+            if c.attn_type == "tri_mix_minference" and "best_pattern" not in kw:
+                if c.config_path:
+                    with open(c.config_path) as f:
+                        kw["best_pattern"] = json.load(f)
+                else:
+                    kw["best_pattern"] = None
+            kw.setdefault("n_local", 512)
+            kw.setdefault("n_init", 8)
+            kw.setdefault("n_last", 128)
+            kw.setdefault("starting_layer", 16)
         elif c.attn_type in ("a_shape", "tri_shape"):
             kw.setdefault("n_local", 3968)
             kw.setdefault("n_init", 128)

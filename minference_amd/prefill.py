@@ -19,7 +19,7 @@ import torch
 
 from .estimate import estimate_vertical_slash
 from .index import convert_vertical_slash_indexes
-from .ops import (block_sparse_attention, dense_causal_attention, streaming_forward,
+from .ops import (block_sparse_attention, dense_causal_attention, streaming_forward, tri_shape_forward,
                   vertical_slash_attention_from_index)
 
 DEFAULT_PATTERN = ("vertical_and_slash", 1000, 6096, 1)   # minference_forward.py:621
@@ -127,3 +127,29 @@ def minference_prefill_forward(query_states, key_states, value_states, prefill_k
         vh = _kv_for_heads(value_states, heads, group)
         output[:, heads] = minference_prefill_kernel(qh, kh, vh, ty, vs, ss)
     return output
+
+
+def tri_shape_kernel(query_states, key_states, value_states, prefill_kwargs):
+    """Tri-shape attention with n_init / n_local / n_last taken from ``attn_forward_config``
+    (the dispatcher-level wrapper the reference's tri_mix module calls, modules/tri_mix.py:35-37)."""
+    cfg = prefill_kwargs["attn_forward_config"]
+    return tri_shape_forward(query_states, key_states, value_states, cfg["n_init"], cfg["n_local"],
+                             cfg.get("n_last", 100))
+
+
+def tri_mix_forward(query_states, key_states, value_states, prefill_kwargs):
+    """modules/tri_mix.py:19-39: dense causal attention below ``starting_layer``, tri-shape from there on."""
+    if prefill_kwargs["layer_idx"] < prefill_kwargs["attn_forward_config"].get("starting_layer", 0):
+        return dense_causal_attention(query_states, key_states, value_states)
+    return tri_shape_kernel(query_states, key_states, value_states, prefill_kwargs)
+
+
+def tri_mix_minference_forward(query_states, key_states, value_states, prefill_kwargs):
+    """modules/tri_mix.py:42-53: the per-head sparse patterns below ``starting_layer``, tri-shape from
+    there on."""
+    cfg = prefill_kwargs["attn_forward_config"]
+    if prefill_kwargs["layer_idx"] < cfg.get("starting_layer", 0):
+        inner = dict(prefill_kwargs)
+        inner["attn_forward_config"] = dict(cfg, starting_layer=0)
+        return minference_prefill_forward(query_states, key_states, value_states, inner)
+    return tri_shape_kernel(query_states, key_states, value_states, prefill_kwargs)

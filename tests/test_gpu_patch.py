@@ -56,6 +56,30 @@ def test_patterns_that_keep_everything_reproduce_the_unpatched_model(gpu, tmp_pa
     close(logits_of(tri, ids), base, "tri_shape (window wider than the sequence)")
 
 
+def test_tri_mix_switches_method_at_the_starting_layer(gpu):
+    from minference_amd import MInference, dense_causal_attention, tri_mix_forward, tri_mix_minference_forward, tri_shape_forward
+    from minference_amd import minference_prefill_forward
+    n = 1300
+    g = torch.Generator().manual_seed(9)
+    q = torch.randn(1, 4, n, 128, generator=g).bfloat16().to(gpu)
+    k = torch.randn(1, 2, n, 128, generator=g).bfloat16().to(gpu)
+    v = torch.randn(1, 2, n, 128, generator=g).bfloat16().to(gpu)
+    cfg = {"starting_layer": 1, "n_init": 8, "n_local": 128, "n_last": 64,
+           "best_pattern": [{str(h): ["stream_llm", 16, 200, 1.0] for h in range(4)}] * 2}
+    tri = tri_shape_forward(q, k, v, 8, 128, 64)
+    assert torch.equal(tri_mix_forward(q, k, v, {"layer_idx": 0, "attn_forward_config": cfg}), dense_causal_attention(q, k, v))
+    assert torch.equal(tri_mix_forward(q, k, v, {"layer_idx": 1, "attn_forward_config": cfg}), tri)
+    sparse0 = minference_prefill_forward(q, k, v, {"layer_idx": 0, "attn_forward_config": dict(cfg, starting_layer=0)})
+    assert torch.equal(tri_mix_minference_forward(q, k, v, {"layer_idx": 0, "attn_forward_config": cfg}), sparse0)
+    assert torch.equal(tri_mix_minference_forward(q, k, v, {"layer_idx": 1, "attn_forward_config": cfg}), tri)
+    # through the patch: everything wide enough to keep all keys -> the unpatched model
+    ids = torch.randint(0, 320, (1, 500), generator=torch.Generator().manual_seed(5)).to(gpu)
+    model = tiny_llama(gpu)
+    base = logits_of(model, ids)
+    mixed = MInference("tri_mix", attn_kwargs={"starting_layer": 1, "n_local": 4096})(model)
+    close(logits_of(mixed, ids), base, "tri_mix (window wider than the sequence)")
+
+
 def test_sparse_patterns_are_really_applied(gpu):
     from minference_amd import MInference
     n = 1500
