@@ -14,7 +14,8 @@ from .ops import (block_sparse_attention, block_sparse_attention_from_index, den
 
 from .estimate import estimate_vertical_slash, topk_indices, vertical_slash_scores
 from .prefill import (load_best_pattern, minference_prefill_forward, minference_prefill_kernel,
-                      tri_mix_forward, tri_mix_minference_forward, vertical_slash_prefill)
+                      dilated_forward, static_vertical_slash_forward, tri_mix_forward,
+                      tri_mix_minference_forward, vertical_slash_prefill)
 from .search import pattern_recall, search_pattern, search_patterns
 from .patch import MInference, MInferenceConfig
 
@@ -25,6 +26,6 @@ __all__ = [
     "convert_vertical_slash_indexes", "vertical_slash_attention_from_index",
     "block_sparse_attention_from_index", "dense_causal_attention", "tri_shape_forward",
     "pattern_recall", "search_pattern", "search_patterns", "MInference", "MInferenceConfig",
-    "tri_mix_forward", "tri_mix_minference_forward",
+    "tri_mix_forward", "tri_mix_minference_forward", "dilated_forward", "static_vertical_slash_forward",
 ]
 __version__ = "0.1.0"

@@ -20,7 +20,8 @@ from __future__ import annotations
 
 import json
 
-SUPPORTED_ATTN_TYPES = ("minference", "tri_mix_minference", "tri_mix", "dense", "a_shape", "tri_shape", "hf")
+SUPPORTED_ATTN_TYPES = ("minference", "tri_mix_minference", "tri_mix", "static", "dilated1", "dilated2", "dense",
+                        "a_shape", "tri_shape", "hf")
 INTERFACE_NAME = "minference_amd"
 _registered = False
 
@@ -50,7 +51,8 @@ class MInferenceConfig:
 def _attention(module, query, key, value, attention_mask, dropout=0.0, scaling=None, **kwargs):
     """The registered attention function: [B,H,N,D] q, [B,Hk,N,D] k/v -> ([B,N,H,D], None)."""
     from .ops import dense_causal_attention, streaming_forward, tri_shape_forward
-    from .prefill import minference_prefill_forward, tri_mix_forward, tri_mix_minference_forward
+    from .prefill import (DEFAULT_PATTERN, dilated_forward, minference_prefill_forward,
+                          static_vertical_slash_forward, tri_mix_forward, tri_mix_minference_forward)
     state = getattr(module.config, "minference_amd", None)
     n = query.shape[2]
     if state is None or n == 1 or key.shape[2] != n or not query.is_cuda:
@@ -68,6 +70,15 @@ def _attention(module, query, key, value, attention_mask, dropout=0.0, scaling=N
         out = fn(query, key, value, {
             "layer_idx": module.layer_idx, "num_hidden_layers": module.config.num_hidden_layers,
             "attn_forward_config": kw})
+    elif ty in ("dilated1", "dilated2"):
+        out = dilated_forward(query, key, value, ty)
+    elif ty == "static":
+        # one (vertical_size, slash_size) per layer: the sizes of head 0 of the table, like a layer
+        # whose heads share a pattern (the reference estimates per head inside its head loop)
+        best = kw.get("best_pattern")
+        _, vs, ss, _ = (best[module.layer_idx].get("0", DEFAULT_PATTERN) if best else DEFAULT_PATTERN)
+        cache = state.setdefault("static_cache", {}).setdefault(module.layer_idx, {})
+        out = static_vertical_slash_forward(query, key, value, vs, ss, cache)
     elif ty == "dense":
         out = dense_causal_attention(query, key, value)
     elif ty == "a_shape":
@@ -95,6 +106,8 @@ class MInference:
       Without a file every head uses vertical_and_slash (1000, 6096).
     * ``"tri_mix_minference"`` / ``"tri_mix"``: the per-head patterns (resp. dense attention) below
       ``attn_kwargs["starting_layer"]`` (16), tri-shape (n_init 8, n_local 512, n_last 128) from there on.
+    * ``"static"``: vertical-slash indices estimated on the first prompt and reused afterwards;
+      ``"dilated1"`` / ``"dilated2"``: the fixed dilated-window baselines (minference_forward.py:365-379).
     * ``"dense"``: dense causal attention on the same tile engine.
     * ``"a_shape"`` / ``"tri_shape"``: ``n_init`` (128), ``n_local`` (3968) and ``n_last`` (100)
       from ``attn_kwargs`` (defaults of models_patch.py:134-143).
@@ -115,6 +128,9 @@ class MInference:
         if c.attn_type == "hf":
             return model
         kw = dict(c.attn_kwargs)
+        if c.attn_type == "static" and "best_pattern" not in kw and c.config_path:
+            with open(c.config_path) as f:
+                kw["best_pattern"] = json.load(f)
         if c.attn_type == "minference":
             kw.setdefault("starting_layer", c.starting_layer)
             kw["is_search"] = bool(c.is_search)

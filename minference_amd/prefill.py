@@ -20,7 +20,7 @@ import torch
 from .estimate import estimate_vertical_slash
 from .index import convert_vertical_slash_indexes
 from .ops import (block_sparse_attention, dense_causal_attention, streaming_forward, tri_shape_forward,
-                  vertical_slash_attention_from_index)
+                  vertical_slash_attention_from_index, vertical_slash_sparse_attention)
 
 DEFAULT_PATTERN = ("vertical_and_slash", 1000, 6096, 1)   # minference_forward.py:621
 
@@ -153,3 +153,37 @@ def tri_mix_minference_forward(query_states, key_states, value_states, prefill_k
         inner["attn_forward_config"] = dict(cfg, starting_layer=0)
         return minference_prefill_forward(query_states, key_states, value_states, inner)
     return tri_shape_kernel(query_states, key_states, value_states, prefill_kwargs)
+
+
+def dilated_forward(q, k, v, kind):
+    """The fixed "dilated" baselines of the reference (minference_forward.py:365-379): the first
+    min(1024, N) columns plus, for ``dilated1``, every second diagonal of the last 8192 offsets'
+    worth of positions, for ``dilated2`` the last 2048 diagonals and every second one of the 4096
+    before them -- expressed, as in the reference, through the vertical-slash operator."""
+    n = q.shape[2]
+    dev = q.device
+    vertical = torch.arange(0, min(1024, n), device=dev, dtype=torch.int32)[None, None, :]
+    pos = torch.arange(0, n, device=dev, dtype=torch.int32)
+    if kind == "dilated1":
+        pos = pos[-8192::2]
+    elif kind == "dilated2":
+        pos = torch.cat([pos[-2048:], pos[-6144:-2048:2]], 0)
+    else:
+        raise KeyError(kind)
+    slash = (n - 1) - pos[None, None, :]
+    B, H = q.shape[:2]
+    return vertical_slash_sparse_attention(q, k, v, vertical.expand(B, H, -1), slash.expand(B, H, -1))
+
+
+def static_vertical_slash_forward(q, k, v, vertical_size, slash_size, cache):
+    """The "static pattern" baseline (minference_forward.py:418-434, 476-477): the vertical and
+    slash indices are estimated on the first prompt a layer sees (forcing the first 30 columns and
+    the 30 nearest diagonals) and reused for every later one; ``cache`` is that layer's dictionary."""
+    from .estimate import topk_vertical_slash, vertical_slash_scores
+    if "vs" not in cache:
+        n = q.shape[2]
+        vsz, ssz = min(n, max(int(vertical_size), 30)), min(n, max(int(slash_size), 50))
+        vertical, slash = vertical_slash_scores(q, k, 64, 30, 30)
+        cache["vs"] = topk_vertical_slash(vertical, slash, vsz, ssz)
+    v_idx, s_idx = cache["vs"]
+    return vertical_slash_sparse_attention(q, k, v, v_idx, s_idx)

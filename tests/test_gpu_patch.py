@@ -80,6 +80,39 @@ def test_tri_mix_switches_method_at_the_starting_layer(gpu):
     close(logits_of(mixed, ids), base, "tri_mix (window wider than the sequence)")
 
 
+def test_dilated_and_static_baselines(gpu):
+    from oracle import oracle as O
+    from minference_amd import MInference, dilated_forward, static_vertical_slash_forward
+    n = 3000
+    g = torch.Generator().manual_seed(11)
+    q = torch.randn(1, 2, n, 128, generator=g).bfloat16()
+    k = torch.randn(1, 2, n, 128, generator=g).bfloat16()
+    v = torch.randn(1, 2, n, 128, generator=g).bfloat16()
+    for kind in ("dilated1", "dilated2"):
+        out = dilated_forward(q.to(gpu), k.to(gpu), v.to(gpu), kind).float().cpu()
+        pos = torch.arange(n)
+        pos = pos[-8192::2] if kind == "dilated1" else torch.cat([pos[-2048:], pos[-6144:-2048:2]])
+        v_idx = torch.arange(min(1024, n)).expand(1, 2, -1)
+        s_idx = ((n - 1) - pos).expand(1, 2, -1)
+        ref = O.vertical_slash_sparse_attention(q, k, v, v_idx, s_idx)
+        err = (out - ref).abs()
+        print(kind, err.max().item(), err.mean().item(), flush=True)
+        assert err.max() <= 2e-2 and err.mean() <= 1e-3
+    cache = {}
+    a = static_vertical_slash_forward(q.to(gpu), k.to(gpu), v.to(gpu), 100, 200, cache)
+    q2 = torch.randn(1, 2, n, 128, generator=g).bfloat16()
+    b = static_vertical_slash_forward(q2.to(gpu), k.to(gpu), v.to(gpu), 100, 200, cache)      # reuses the indices
+    v_idx, s_idx = cache["vs"]
+    ref = O.vertical_slash_sparse_attention(q2, k, v, v_idx.cpu(), s_idx.cpu())
+    assert (b.float().cpu() - ref).abs().max() <= 2e-2 and a.shape == b.shape
+    # through the patch (short prompt: the dilated patterns keep every key)
+    ids = torch.randint(0, 320, (1, 400), generator=torch.Generator().manual_seed(6)).to(gpu)
+    model = tiny_llama(gpu)
+    base = logits_of(model, ids)
+    close(logits_of(MInference("dilated2")(model), ids), base, "dilated2 on a short prompt")
+    assert torch.isfinite(logits_of(MInference("static")(model), ids)).all()
+
+
 def test_sparse_patterns_are_really_applied(gpu):
     from minference_amd import MInference
     n = 1500

@@ -103,7 +103,7 @@ def test_planted_layer_is_deterministic_and_structured():
 
 def test_patch_configuration_rejects_what_is_not_built():
     from minference_amd import MInference
-    for bad in ("inf_llm", "flexprefill", "vllm_minference", "dilated1"):
+    for bad in ("inf_llm", "flexprefill", "vllm_minference", "xattention"):
         with pytest.raises(NotImplementedError):
             MInference(bad)
     with pytest.raises(NotImplementedError):
