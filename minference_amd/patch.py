@@ -12,8 +12,8 @@ registry (Llama, Qwen2, Mistral, ...) is covered without touching its code.  The
 receives K/V with their own (fewer) heads -- no ``repeat_kv`` copy is ever made.
 
 Scope: the prefill of one unpadded sequence (what the reference's prefill path assumes as well).
-Decode steps and chunks that attend to a longer cache (``key length != query length``) are passed
-to transformers' SDPA function unchanged.  KV-cache compression (``kv_type``), CPU KV offload and
+Decode steps, chunks that attend to a longer cache (``key length != query length``) and calls that
+carry an explicit attention mask (padding, packing) are passed to transformers' SDPA function unchanged.  KV-cache compression (``kv_type``), CPU KV offload and
 the reference's other attention types belong to other paths of the reference and raise.
 """
 from __future__ import annotations
@@ -55,7 +55,8 @@ def _attention(module, query, key, value, attention_mask, dropout=0.0, scaling=N
                           static_vertical_slash_forward, tri_mix_forward, tri_mix_minference_forward)
     state = getattr(module.config, "minference_amd", None)
     n = query.shape[2]
-    if state is None or n == 1 or key.shape[2] != n or not query.is_cuda:
+    # an explicit mask means padding or packing: not the single-sequence prefill this path covers
+    if state is None or n == 1 or key.shape[2] != n or attention_mask is not None or not query.is_cuda:
         from transformers.integrations.sdpa_attention import sdpa_attention_forward
         return sdpa_attention_forward(module, query, key, value, attention_mask, dropout=dropout,
                                       scaling=scaling, **kwargs)
@@ -92,7 +93,12 @@ def _register():
     global _registered
     if not _registered:
         from transformers import AttentionInterface
+        from transformers.masking_utils import AttentionMaskInterface, sdpa_mask
         AttentionInterface.register(INTERFACE_NAME, _attention)
+        # masks are built as for SDPA: none at all for one unpadded causal sequence, a boolean 4-D
+        # mask when there is padding (without this registration transformers would build no mask
+        # for an attention function it does not know, padding or not)
+        AttentionMaskInterface.register(INTERFACE_NAME, sdpa_mask)
         _registered = True
 
 

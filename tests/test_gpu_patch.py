@@ -138,6 +138,18 @@ def test_generate_runs_prefill_sparse_and_decode_through_transformers(gpu):
     assert torch.equal(got[:, :n], ids)
 
 
+def test_padded_batches_fall_through_to_transformers(gpu):
+    from minference_amd import MInference
+    ids = torch.randint(0, 320, (2, 200), generator=torch.Generator().manual_seed(8)).to(gpu)
+    mask = torch.ones_like(ids)
+    mask[1, :37] = 0                                       # left padding in the second sequence
+    model = tiny_llama(gpu)
+    with torch.no_grad():
+        want = model(ids, attention_mask=mask).logits.float()
+        got = MInference("a_shape", attn_kwargs={"n_init": 1, "n_local": 8})(model)(ids, attention_mask=mask).logits.float()
+    close(got[:, 40:], want[:, 40:], "padded batch")      # identical path: the sparse pattern was not applied
+
+
 def test_search_mode_writes_a_table_the_patch_loads(gpu, tmp_path):
     from minference_amd import MInference
     n = 2900                                  # the search averages over rows >= 2500
