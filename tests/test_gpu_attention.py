@@ -325,3 +325,46 @@ def test_tri_shape_vs_oracle(gpu, n, n_init, n_local, n_last):
     mask = O.trishape_mask(n, n_init, n_local, n_last)
     ref = torch.stack([O.masked_attention(q[0, h], k[0, 0], v[0, 0], mask) for h in range(2)])[None]
     check(out, ref, "trishape")
+
+
+@pytest.mark.parametrize("seed", list(range(8)))
+def test_seeded_random_shapes_all_operators(gpu, seed):
+    """Random sequence lengths (any remainder modulo 64), head counts, list sizes and window sizes,
+    one case per operator and seed, against the fp32 masked-dense oracle."""
+    from minference_amd import (block_sparse_attention_from_index, streaming_forward, tri_shape_forward,
+                                vertical_slash_sparse_attention)
+    rng = np.random.default_rng(7000 + seed)
+    n = int(rng.integers(65, 1800))
+    hk = int(rng.choice([1, 2]))
+    hq = hk * int(rng.choice([1, 2, 4]))
+    dtype = torch.bfloat16 if seed % 2 == 0 else torch.float16
+    print(f"case random seed={seed} n={n} hq={hq} hk={hk} {dtype}", flush=True)
+    q, k, v = make(1, hq, hk, n, 900 + seed, dtype)
+    qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
+    ke, ve = expand(k, hq), expand(v, hq)
+
+    nv, ns = int(rng.integers(1, min(n, 300))), int(rng.integers(1, min(n, 300)))
+    vi, si = gen.vs_index_inputs(hq, n, nv, ns, seed=seed, force_v=min(2, nv), force_s=min(int(rng.integers(1, 5)), ns))
+    v_idx, s_idx = torch.from_numpy(vi.astype(np.int64)), torch.from_numpy(np.ascontiguousarray(si).astype(np.int64))
+    out = vertical_slash_sparse_attention(qg, kg, vg, v_idx.to(gpu), s_idx.to(gpu))
+    check(out, O.vertical_slash_sparse_attention(q, ke, ve, v_idx, s_idx), "random vs")
+
+    rows = (n + 64 - (n & 63)) // 64
+    top_k = int(rng.integers(1, 9))
+    bi = np.zeros((1, hq, rows, top_k), dtype=np.int32)
+    for h in range(hq):
+        for m in range(rows):
+            cnt = min(m + 1, top_k)
+            bi[0, h, m, :cnt] = np.sort(rng.choice(m + 1, size=cnt, replace=False))
+            bi[0, h, m, cnt:] = m
+    bi = torch.from_numpy(bi)
+    out = block_sparse_attention_from_index(qg, kg, vg, bi.to(gpu))
+    ref = torch.stack([O.masked_attention(q[0, h], ke[0, h], ve[0, h], O.bs_mask(bi[0, h].numpy(), n)) for h in range(hq)])[None]
+    check(out, ref, "random bs")
+
+    n_init, n_local = int(rng.integers(0, 200)), int(rng.integers(1, 700))
+    check(streaming_forward(qg, kg, vg, n_init, n_local), O.streaming_forward(q, ke, ve, n_init, n_local), "random a-shape")
+    n_last = int(rng.integers(1, 150))
+    nl = min(n_last, n - 1)
+    ref = torch.stack([O.masked_attention(q[0, h], ke[0, h], ve[0, h], O.trishape_mask(n, n_init, n_local, nl)) for h in range(hq)])[None]
+    check(tri_shape_forward(qg, kg, vg, n_init, n_local, n_last), ref, "random tri-shape")
