@@ -14,7 +14,6 @@ token chunks so no intermediate is larger than ``chunk x intermediate_size``.
 """
 from __future__ import annotations
 
-import math
 from dataclasses import dataclass
 
 import torch

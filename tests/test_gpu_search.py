@@ -3,7 +3,6 @@ C ABI) against the oracle's N x N restatement.  Tolerance: the scores are means 
 masses in [0, 1]; both sides compute in fp32 on identical 16-bit inputs, so they agree to 2e-3
 absolute (the slack covers a top-k boundary element whose two fp32 estimates differ in the last
 bits and fall on either side of the threshold)."""
-import math
 
 import numpy as np
 import pytest

@@ -1,7 +1,6 @@
 """Host-side logic that needs no GPU: per-head pattern planning of the dispatcher
 (reference minference/modules/minference_forward.py:594-674), argument checks of the
 operators, generators."""
-import json
 import os
 
 import numpy as np

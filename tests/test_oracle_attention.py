@@ -1,7 +1,6 @@
 """Pins the attention side of the oracle (masks + fp32 masked-dense softmax) through special
 cases that reduce to torch's scaled_dot_product_attention and per-element brute force."""
 import numpy as np
-import pytest
 import torch
 
 from oracle import oracle as O

@@ -5,7 +5,6 @@ per-element brute force on tiny inputs."""
 import math
 
 import numpy as np
-import pytest
 import torch
 
 from oracle import oracle as O
