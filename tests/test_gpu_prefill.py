@@ -95,6 +95,41 @@ def test_config2_full_size_sampled_row_blocks(gpu):
         assert err.max() <= 2e-2 and err.mean() <= 1e-3
 
 
+def test_one_million_tokens_sampled_row_blocks(gpu):
+    """The longest context the reference advertises (Llama-3-8B-1M): 1 048 576 tokens minus a ragged
+    tail, 2 query heads on one kv head, the whole GPU path with zero-filled index tensors; sampled
+    row blocks are checked like in the 131072-token test (index rows bit-exact against the reference
+    algorithm, attention rows against the fp32 masked-dense result)."""
+    import minference_amd as M
+    n, hq, hk = 1048576 - 11, 2, 1
+    q, k, v, _ = gen.planted_layer(n, hq, hk, seed=101, dtype=torch.bfloat16)
+    qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
+    v_idx, s_idx = M.estimate_vertical_slash(qg, kg, 1000, 6096)
+    seqlens = torch.full((1,), n, dtype=torch.int32, device=gpu)
+    bc, bo, cc, ci = M.convert_vertical_slash_indexes(seqlens, v_idx, s_idx, n, 64, 64)
+    out = M.vertical_slash_attention_from_index(qg, kg, vg, bc, bo, cc, ci, seqlens)
+    torch.cuda.synchronize()
+    rows = (n + 63) // 64
+    assert bc.shape == (1, hq, rows) and int(bc.max()) <= 6096 and int(cc.max()) <= 1000
+    vi_c, si_c = v_idx.cpu().numpy(), s_idx.cpu().numpy()
+    kf, vf = k[0, 0].float(), v[0, 0].float()
+    for h, m in [(0, 0), (1, rows - 1), (0, 9000), (1, 16000)]:
+        print(f"case 1M head={h} row-block={m}", flush=True)
+        rbo, rci = O.vs_index_row_py(vi_c[0, h].tolist(), si_c[0, h].tolist(), m, n)
+        rbc, rcc = len(rbo), len(rci)
+        assert int(bc[0, h, m]) == rbc and int(cc[0, h, m]) == rcc
+        assert bo[0, h, m, :rbc].cpu().tolist() == rbo and ci[0, h, m, :rcc].cpu().tolist() == rci
+        assert int(bo[0, h, m, rbc:].abs().max() if rbc < 6096 else 0) == 0          # zero tail
+        mask = O.vs_mask_rows(rbc, rbo, rcc, rci, m, n)
+        r0, r1 = m * 64, min(m * 64 + 64, n)
+        s = (q[0, h, r0:r1].float() @ kf.T) * (128 ** -0.5)
+        s = torch.where(torch.as_tensor(mask), s, torch.tensor(-torch.inf))
+        ref = torch.softmax(s, dim=-1) @ vf
+        err = (out[0, h, r0:r1].float().cpu() - ref).abs()
+        print(f"  max-abs {err.max().item():.3e} mean-abs {err.mean().item():.3e}", flush=True)
+        assert err.max() <= 2e-2 and err.mean() <= 1e-3
+
+
 def _rows_reference(q_rows, k, v, mask):
     s = (q_rows.float() @ k.float().T) * (q_rows.shape[-1] ** -0.5)
     s = torch.where(torch.as_tensor(mask), s, torch.tensor(-torch.inf))
