@@ -13,11 +13,12 @@ from .ops import (block_sparse_attention, block_sparse_attention_from_index, den
                   vertical_slash_sparse_attention)
 
 from .estimate import estimate_vertical_slash, topk_indices, vertical_slash_scores
-from .prefill import (load_best_pattern, minference_prefill_forward, minference_prefill_kernel,
+from .configs import get_support_models
+from .prefill import (a_shape_kernel, tri_shape_kernel, load_best_pattern, minference_prefill_forward, minference_prefill_kernel,
                       dilated_forward, static_vertical_slash_forward, tri_mix_forward,
                       tri_mix_minference_forward, vertical_slash_prefill)
 from .search import pattern_recall, search_pattern, search_patterns
-from .patch import MInference, MInferenceConfig
+from .patch import MInference, MInferenceConfig, minference_patch, patch_hf
 
 __all__ = [
     "estimate_vertical_slash", "vertical_slash_scores", "topk_indices", "vertical_slash_prefill",
@@ -27,5 +28,6 @@ __all__ = [
     "block_sparse_attention_from_index", "dense_causal_attention", "tri_shape_forward",
     "pattern_recall", "search_pattern", "search_patterns", "MInference", "MInferenceConfig",
     "tri_mix_forward", "tri_mix_minference_forward", "dilated_forward", "static_vertical_slash_forward",
+    "a_shape_kernel", "tri_shape_kernel", "minference_patch", "patch_hf", "get_support_models",
 ]
 __version__ = "0.1.0"

@@ -20,6 +20,8 @@ from __future__ import annotations
 
 import json
 
+from .configs import resolve_config_path
+
 SUPPORTED_ATTN_TYPES = ("minference", "tri_mix_minference", "tri_mix", "static", "dilated1", "dilated2", "dense",
                         "a_shape", "tri_shape", "hf")
 INTERFACE_NAME = "minference_amd"
@@ -42,6 +44,10 @@ class MInferenceConfig:
             raise TypeError(f"unknown arguments {sorted(kwargs)}")
         self.attn_type = attn_type
         self.model_name = model_name
+        # minference_configuration.py:85-93: only the types that read a best_pattern table look one
+        # up by model name; a search writes its table and therefore needs an explicit path
+        if attn_type in ("minference", "tri_mix_minference", "static") and not is_search:
+            config_path = resolve_config_path(config_path, model_name)
         self.config_path = config_path
         self.starting_layer = starting_layer
         self.is_search = is_search
@@ -171,3 +177,20 @@ class MInference:
         model.config.minference_amd = {"attn_type": c.attn_type, "attn_kwargs": kw}
         model.set_attn_implementation(INTERFACE_NAME)
         return model
+
+
+def minference_patch(model, config):
+    """``minference_patch(model, MInferenceConfig(...))`` (reference minference/patch.py:895-903)."""
+    patcher = MInference.__new__(MInference)
+    patcher.config = config
+    return patcher.patch_model(model)
+
+
+def patch_hf(model, attn_type="a_shape", attn_kwargs=None, **kwargs):
+    """``patch_hf(model, attn_type, attn_kwargs)`` (reference minference/patch.py:1313-1321, the call
+    the reference makes for its streaming types, models_patch.py:128-143): extra keyword arguments
+    are merged into ``attn_kwargs``.  The reference's default type of this function, InfLLM, is a
+    KV-cache method and not part of this package, hence the different default."""
+    kw = dict(attn_kwargs or {})
+    kw.update(kwargs)
+    return MInference(attn_type, attn_kwargs=kw)(model)

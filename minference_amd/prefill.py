@@ -129,12 +129,20 @@ def minference_prefill_forward(query_states, key_states, value_states, prefill_k
     return output
 
 
+def a_shape_kernel(query_states, key_states, value_states, prefill_kwargs):
+    """A-shape (sink + sliding window) attention with n_init (128) / n_local (3968) taken from
+    ``attn_forward_config`` (reference minference/ops/streaming_kernel.py:781-818)."""
+    cfg = prefill_kwargs["attn_forward_config"]
+    return streaming_forward(query_states, key_states, value_states, cfg.get("n_init", 128),
+                             cfg.get("n_local", 3968))
+
+
 def tri_shape_kernel(query_states, key_states, value_states, prefill_kwargs):
     """Tri-shape attention with n_init / n_local / n_last taken from ``attn_forward_config``
     (the dispatcher-level wrapper the reference's tri_mix module calls, modules/tri_mix.py:35-37)."""
     cfg = prefill_kwargs["attn_forward_config"]
-    return tri_shape_forward(query_states, key_states, value_states, cfg["n_init"], cfg["n_local"],
-                             cfg.get("n_last", 100))
+    return tri_shape_forward(query_states, key_states, value_states, cfg.get("n_init", 128),
+                             cfg.get("n_local", 3968), cfg.get("n_last", 100))
 
 
 def tri_mix_forward(query_states, key_states, value_states, prefill_kwargs):

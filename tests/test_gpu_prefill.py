@@ -46,6 +46,25 @@ def test_starting_layer_falls_back_to_dense(gpu):
     assert (out - ref).abs().max() <= 2e-2
 
 
+def test_a_shape_and_tri_shape_kernels_take_the_reference_config(gpu):
+    """``a_shape_kernel(q, k, v, config)`` / ``tri_shape_kernel(q, k, v, config)`` with the
+    reference's config dictionary and its defaults (streaming_kernel.py:781-833: n_init 128,
+    n_local 3968, n_last 100) against the masked-dense oracle."""
+    import minference_amd as M
+    n = 5000                                                        # longer than n_init + n_local
+    q, k, v = gen.qkv(1, 2, 2, n, 128, seed=21, scale=1.0)
+    q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
+    dq, dk, dv = q.to(gpu), k.to(gpu), v.to(gpu)
+    for cfg, (ni, nl, nlast) in (({}, (128, 3968, 100)), ({"n_init": 16, "n_local": 700, "n_last": 33}, (16, 700, 33))):
+        kwargs = {"attn_forward_config": cfg}
+        a = M.a_shape_kernel(dq, dk, dv, kwargs).float().cpu()
+        t = M.tri_shape_kernel(dq, dk, dv, kwargs).float().cpu()
+        for h in range(2):
+            for got, mask in ((a, O.ashape_mask(n, ni, nl)), (t, O.trishape_mask(n, ni, nl, nlast))):
+                err = (got[0, h] - O.masked_attention(q[0, h], k[0, h], v[0, h], mask)).abs()
+                assert err.max() <= 2e-2 and err.mean() <= 1e-3, (cfg, h, float(err.max()))
+
+
 def test_config1_shape_fp32_full(gpu):
     """BASELINE config 1 at full size (batch 1, 4 heads, seq 8192, head_dim 128, fp32, vertical 1000,
     slash 2048): op output vs fp32 masked-dense on identical indices, sampled row blocks."""

@@ -115,3 +115,35 @@ def test_patch_configuration_rejects_what_is_not_built():
     assert m.config.attn_type == "a_shape" and m.config.attn_kwargs == {"n_local": 100}
     sentinel = object()
     assert MInference("hf")(sentinel) is sentinel                     # "hf": model unchanged
+
+
+def test_model_name_resolves_to_a_pattern_file(tmp_path, monkeypatch):
+    """minference_configuration.py:85-93: explicit path wins, unknown model is an error; here the
+    files live in a user-filled directory, and a missing file is reported with its path."""
+    from minference_amd import MInference, get_support_models
+    from minference_amd.configs import PATTERN_FILES, resolve_config_path
+    names = get_support_models()
+    assert "meta-llama/Llama-3.1-8B-Instruct" in names and len(names) == len(set(names)) == 18
+    monkeypatch.setenv("MINFERENCE_CONFIG_DIR", str(tmp_path))
+    assert resolve_config_path("x.json", "no/such-model") == "x.json"
+    assert resolve_config_path(None, None) is None
+    with pytest.raises(ValueError):
+        MInference("minference", "no/such-model")
+    with pytest.raises(FileNotFoundError) as err:
+        MInference("minference", "Qwen/Qwen2-7B-Instruct")
+    assert str(tmp_path) in str(err.value)
+    path = tmp_path / PATTERN_FILES["Qwen/Qwen2-7B-Instruct"]
+    path.write_text("[]")
+    assert MInference("minference", "Qwen/Qwen2-7B-Instruct").config.config_path == str(path)
+    # types that read no table never look one up; a search needs its own output path
+    assert MInference("a_shape", "no/such-model").config.config_path is None
+    assert MInference("minference", "no/such-model", config_path="out.json", is_search=True).config.config_path == "out.json"
+
+
+def test_reference_patch_function_names():
+    from minference_amd import MInferenceConfig, minference_patch, patch_hf
+    sentinel = object()
+    assert minference_patch(sentinel, MInferenceConfig("hf")) is sentinel
+    assert patch_hf(sentinel, "hf", {"n_init": 1}, n_local=2) is sentinel
+    with pytest.raises(NotImplementedError):
+        patch_hf(sentinel, "inf_llm")
