@@ -21,8 +21,11 @@
 // LDS: one K and one V tile per workgroup, [64 tokens][128] 16-bit, 256-byte rows whose 16-byte
 // chunks are XOR-permuted (K: chunk ^ row%16, V: chunk ^ 4*(row%4)) so that the ds_read_b128 of 32
 // K rows and the 4-row transpose reads of V hit distinct banks.  Tiles are copied global -> LDS
-// directly (global_load_lds_dwordx4, no staging registers, no LDS store instructions); the
-// permutation is applied on the global-address side.  32 KB of LDS and <= 256 registers keep four
+// directly (no staging registers, no LDS store instructions); the permutation is applied on the
+// global-address side.  Contiguous tiles use buffer_load_dwordx4 ... lds with a scalar descriptor of
+// the 64 tile rows, a scalar row offset and one of five loop-invariant per-lane offsets: no vector
+// instruction per copy and 8 cycles less issue time per copy than the 64-bit-address form, which
+// remains for gathered and clamped rows (global_load_lds_dwordx4).  32 KB of LDS and <= 256 registers keep four
 // workgroups (two waves per SIMD) resident per CU.
 //
 // One iteration of a wave (two workgroup barriers per tile, single buffers):
@@ -377,6 +380,10 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
     const int cp_c = lane & 15;                  // LDS chunk
     // gathered tiles: lane l holds the token id of tile row l (one load per lane, issued an
     // iteration ahead); the copy fetches the ids of its own rows with wave shuffles
+    int k_lane[4], v_lane;
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) k_lane[jj] = cp_r * (int)k_row + ((cp_c ^ (4 * jj + cp_r)) << 4);
+    v_lane = cp_r * (int)v_row + ((cp_c ^ (cp_r << 2)) << 4);
     auto gather_ids = [&](const Tile &t) -> int {
         if (MODE == MODE_VS && t.gathered) return p.ci[ridx * p.nnz_v + t.start + min(lane, t.nvalid - 1)];
         return 0;
@@ -386,15 +393,16 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
         constexpr bool is_v = decltype(is_v_c)::value;
         const bool gathered = MODE == MODE_VS && t.gathered;
         if (!gathered && t.start >= 0 && t.start + BN <= seqlen) {
+            // buffer form: descriptor of the 64 tile rows (scalar), one of five per-lane offsets (the V
+            // swizzle does not depend on j, the K swizzle only on j % 4) and a scalar row offset
             const char *tb = base + (long long)t.start * rowstride;      // wave-uniform
+            const __amdgpu_buffer_rsrc_t srd = __builtin_amdgcn_make_buffer_rsrc((void *)tb, 0, BN * (int)rowstride, 0x00020000);
 #pragma unroll
             for (int j = 0; j < CROWS / 4; ++j) {
-                const int r = CROWS * wave_wg + 4 * j + cp_r;
-                const int c = is_v ? (cp_c ^ ((r & 3) << 2)) : (cp_c ^ (r & 15));
-                const char *gp = tb + (unsigned)(r * (int)rowstride + c * 16);
-                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
-                                                 (__attribute__((address_space(3))) void *)(ldsbuf + (CROWS * wave_wg + 4 * j) * ROW_BYTES),
-                                                 16, 0, 0);
+                const int voff = is_v ? v_lane : k_lane[j & 3];
+                const int soff = (CROWS * wave_wg + 4 * j) * (int)rowstride;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(srd, (__attribute__((address_space(3))) void *)(ldsbuf + (CROWS * wave_wg + 4 * j) * ROW_BYTES),
+                                                         16, voff, soff, 0, 0);
             }
             return;
         }
