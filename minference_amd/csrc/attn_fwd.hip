@@ -133,17 +133,15 @@ template <> __device__ __forceinline__ void cvt8<_Float16>(const float *x, Frag 
 
 typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
 typedef __attribute__((__vector_size__(2 * sizeof(_Float16)))) _Float16 f16x2_t;
-template <typename T> __device__ __forceinline__ float pair_sum(const Frag &f);
-template <> __device__ __forceinline__ float pair_sum<__bf16>(const Frag &f) {
+template <typename T> __device__ __forceinline__ float pair_sum(const Frag &f, float acc);
+template <> __device__ __forceinline__ float pair_sum<__bf16>(const Frag &f, float acc) {
     const bf16x2_t one = {(__bf16)1.0f, (__bf16)1.0f};
-    float acc = 0.f;
 #pragma unroll
     for (int j = 0; j < 4; ++j) { bf16x2_t pr = {f.b[2 * j], f.b[2 * j + 1]}; acc = __builtin_amdgcn_fdot2_f32_bf16(pr, one, acc, false); }
     return acc;
 }
-template <> __device__ __forceinline__ float pair_sum<_Float16>(const Frag &f) {
+template <> __device__ __forceinline__ float pair_sum<_Float16>(const Frag &f, float acc) {
     const f16x2_t one = {(_Float16)1.0f, (_Float16)1.0f};
-    float acc = 0.f;
 #pragma unroll
     for (int j = 0; j < 4; ++j) { f16x2_t pr = {f.h[2 * j], f.h[2 * j + 1]}; acc = __builtin_amdgcn_fdot2(pr, one, acc, false); }
     return acc;
@@ -568,14 +566,16 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
         // ---- online softmax (exp2 domain) -------------------------------------
         float mx;
         {
-            float m4[4];                 // four independent chains instead of one of 32 links
+            // four independent chains of three-operand maxima (8 scores each)
+            float m4[4];
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
-                m4[c] = fmaxf(s0[4 * c], s1[4 * c]);
-#pragma unroll
-                for (int e = 1; e < 4; ++e) m4[c] = fmaxf(m4[c], fmaxf(s0[4 * c + e], s1[4 * c + e]));
+                m4[c] = fmaxf(fmaxf(s0[4 * c], s1[4 * c]), s0[4 * c + 1]);
+                m4[c] = fmaxf(fmaxf(m4[c], s1[4 * c + 1]), s0[4 * c + 2]);
+                m4[c] = fmaxf(fmaxf(m4[c], s1[4 * c + 2]), s0[4 * c + 3]);
+                m4[c] = fmaxf(m4[c], s1[4 * c + 3]);
             }
-            mx = fmaxf(fmaxf(m4[0], m4[1]), fmaxf(m4[2], m4[3]));
+            mx = fmaxf(fmaxf(fmaxf(m4[0], m4[1]), m4[2]), m4[3]);
         }
         { const unsigned u = __float_as_uint(mx); auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false); mx = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1])); }
         const float cand = mx * p.scale_log2;
@@ -593,7 +593,7 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
 #pragma unroll
             for (int r = 0; r < 8; ++r) pv[r] = __builtin_amdgcn_exp2f(fmaf(sx[8 * (q & 1) + r], p.scale_log2, -m_use));
             cvt8<T>(&pv[0], pfr[q]);
-            psum += pair_sum<T>(pfr[q]);
+            psum = pair_sum<T>(pfr[q], psum);
         };
         probs(0);
         if (__any(alpha != 1.0f)) {
