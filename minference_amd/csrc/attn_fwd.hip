@@ -32,9 +32,9 @@
 //   wait own K(it) copies; barrier (all of K(it) visible, everyone done with V(it-1))
 //   issue V(it) copy; S^T = K.Q^T with the K fragments read two k-steps ahead of their MFMAs
 //   wait own V(it) copies; barrier (all of V(it) visible, everyone done with K(it))
-//   read the V^T fragments of keys 0..15; issue K(it+1) copy; row max; exponentials of keys 0..15
-//   O^T += V^T.P^T with the exponentials and the V^T fragment reads of key group s+1 (16 keys)
-//   placed behind the MFMAs of group s
+//   read all V^T fragments; issue K(it+1) copy; row max; exponentials of keys 0..15
+//   O^T += V^T.P^T with the exponentials of key group s+1 (16 keys) placed behind the MFMAs of
+//   group s
 // The compiler's own schedule read every fragment right before its MFMA (full LDS latency exposed
 // sixteen times per tile); the order above is pinned with sched_barrier / sched_group_barrier.
 //
@@ -513,16 +513,19 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
         }
         __builtin_amdgcn_s_waitcnt(0x0f70);      // vmcnt(0): this wave's part of V(it) is in LDS
         __syncthreads();
-        // V^T fragments of the first 16 keys: their LDS latency passes under the copy issue and the
-        // row max below
+        // all V^T fragments of the tile, read here: the PV block below is bound by its vector
+        // instructions, and every LDS read moved out of it shortens it (+3 % for the 24 reads that
+        // used to sit between its MFMAs); the latency passes under the copy issue and the row max
         Frag vf[4][4];
         if (active) {
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
 #pragma unroll
         for (int db = 0; db < 4; ++db)
 #pragma unroll
             for (int jj = 0; jj < 2; ++jj)
-                vf[0][db].s4[jj] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (__attribute__((address_space(3))) short4_t *)(lds_v + v_rd_off[db] + (8 * jj) * ROW_BYTES));
+                vf[s][db].s4[jj] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (__attribute__((address_space(3))) short4_t *)(lds_v + v_rd_off[db] + (16 * s + 8 * jj) * ROW_BYTES));
         __builtin_amdgcn_sched_barrier(0);
         }
         if (have_nxt) copy_tile(nxt, k_base, k_row, std::false_type{}, gt_nxt, lds_k);
@@ -607,17 +610,8 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
         }
 
         __builtin_amdgcn_s_setprio(2);
-        // ---- O^T += V^T . P^T; the exponentials of key group q+1 run under the MFMAs of group q,
-        // the V^T fragments of group q+1 are fetched under them as well ------------------------
+        // ---- O^T += V^T . P^T; the exponentials of key group q+1 run under the MFMAs of group q ----
         {
-#pragma unroll
-            for (int s = 1; s < 4; ++s)
-#pragma unroll
-                for (int db = 0; db < 4; ++db)
-#pragma unroll
-                    for (int jj = 0; jj < 2; ++jj)
-                        vf[s][db].s4[jj] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                            (__attribute__((address_space(3))) short4_t *)(lds_v + v_rd_off[db] + (16 * s + 8 * jj) * ROW_BYTES));
             probs(1);
             probs(2);
             probs(3);
@@ -631,7 +625,6 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
             for (int i = 0; i < 16; ++i) {
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
                 if (i < 12) __builtin_amdgcn_sched_group_barrier(VALU_MASK, VALU_PER_MFMA, 0);
-                if (i < 12) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
             }
         }
         __builtin_amdgcn_s_setprio(0);
