@@ -132,6 +132,15 @@ class MInference:
                                        starting_layer=starting_layer, kv_cache_cpu=kv_cache_cpu,
                                        kv_type=kv_type, is_search=is_search, attn_kwargs=attn_kwargs, **kwargs)
 
+    @classmethod
+    def from_config(cls, config):
+        """A patcher around an existing ``MInferenceConfig``."""
+        if not isinstance(config, MInferenceConfig):
+            raise TypeError("config must be a MInferenceConfig")
+        self = cls.__new__(cls)
+        self.config = config
+        return self
+
     def __call__(self, model):
         return self.patch_model(model)
 
@@ -181,9 +190,7 @@ class MInference:
 
 def minference_patch(model, config):
     """``minference_patch(model, MInferenceConfig(...))`` (reference minference/patch.py:895-903)."""
-    patcher = MInference.__new__(MInference)
-    patcher.config = config
-    return patcher.patch_model(model)
+    return MInference.from_config(config).patch_model(model)
 
 
 def patch_hf(model, attn_type="a_shape", attn_kwargs=None, **kwargs):
