@@ -27,8 +27,9 @@ PEAK_BF16_TFLOPS = 2500.0               # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the vertical-slash attention kernel on the default workload (seq 131072,
 # seed 100), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a 1 GiB copy kernel
-# (profiles/sparse_path_c2_128k_hbm_traffic.txt): 2.181 GB read + 1.074 GB written.
-ATTN_TRAFFIC_BYTES_C2 = 2_180_788_000 + 1_073_742_000
+# (profiles/sparse_path_c2_128k_hbm_traffic.txt): 2.262 GB read (2.09 - 2.26 GB over repeated runs) +
+# 1.074 GB written.
+ATTN_TRAFFIC_BYTES_C2 = 2_262_454_000 + 1_073_742_000
 
 
 def cpu_baseline(budget_s=25.0):
