@@ -31,8 +31,9 @@
 // One iteration of a wave (two workgroup barriers per tile, single buffers):
 //   wait own K(it) copies; barrier (all of K(it) visible, everyone done with V(it-1))
 //   issue V(it) copy; S^T = K.Q^T with the K fragments read two k-steps ahead of their MFMAs
-//   wait own V(it) copies; barrier (all of V(it) visible, everyone done with K(it))
-//   issue K(it+1) copy; read all V^T fragments; row max; exponentials of keys 0..15
+//   wait own V(it) copies; barrier (all of V(it) visible, everyone done with K(it)) -- in the 2-wave
+//   kernel already before the last four QK MFMAs, with all V^T fragment reads issued under them
+//   issue K(it+1) copy; (paired variant: read all V^T fragments;) row max; exponentials of keys 0..15
 //   O^T += V^T.P^T with the exponentials of key group s+1 (16 keys) placed behind the MFMAs of
 //   group s
 // The compiler's own schedule read every fragment right before its MFMA (full LDS latency exposed
@@ -73,6 +74,9 @@ constexpr int ROW_BYTES = HD * 2;
 // MFMAs; VALU_PER_MFMA softmax instructions are placed behind each of the first twelve PV MFMAs.
 constexpr int QK_AHEAD = 2;
 constexpr int VALU_PER_MFMA = 6;
+// 2-wave kernel: the second barrier of a tile comes after this k-step of the QK loop (all K
+// fragments have been read by then), and the V^T fragment reads follow it under the last MFMAs
+constexpr int EARLY_B2 = 5;
 constexpr int VALU_MASK = 0x402;             // sched_group_barrier classes: VALU | transcendental
 
 struct AttnParams {
@@ -484,6 +488,7 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
         if constexpr (PAIR && MODE == MODE_BS) active = have_rows && (half ? cur.on_b : cur.on_a);
         else if constexpr (PAIR) active = have_rows && tile_on_list<MODE>(p, m, cur.start);
         f32x16_t s0, s1;
+        Frag vf[4][4];
         if (active) {
         __builtin_amdgcn_s_setprio(2);
         // ---- S^T = K . Q^T --------------------------------------------------
@@ -507,13 +512,31 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
                 s0 = Mma<T>::mfma(frag_as<T>(a0[ks]), frag_as<T>(qf[ks]), s0);
                 s1 = Mma<T>::mfma(frag_as<T>(a1[ks]), frag_as<T>(qf[ks]), s1);
                 __builtin_amdgcn_sched_barrier(0);
+                if constexpr (!PAIR && EARLY_B2 >= 0) {
+                    if (ks == EARLY_B2) {
+                        // every K fragment has been read: the second barrier comes before the last
+                        // four MFMAs (2-wave kernel only: all its waves run this code) and the V^T
+                        // fragment reads are issued under them (+0.9 %)
+                        __builtin_amdgcn_s_waitcnt(0x0f70);
+                        __syncthreads();
+#pragma unroll
+                        for (int s = 0; s < 4; ++s)
+#pragma unroll
+                            for (int db = 0; db < 4; ++db)
+#pragma unroll
+                                for (int jj = 0; jj < 2; ++jj)
+                                    vf[s][db].s4[jj] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                                        (__attribute__((address_space(3))) short4_t *)(lds_v + v_rd_off[db] + (16 * s + 8 * jj) * ROW_BYTES));
+                    }
+                }
             }
         }
         __builtin_amdgcn_s_setprio(0);
         }
+        if constexpr (PAIR || EARLY_B2 < 0) {
         __builtin_amdgcn_s_waitcnt(0x0f70);      // vmcnt(0): this wave's part of V(it) is in LDS
         __syncthreads();
-        Frag vf[4][4];
+        }
         if (have_nxt) copy_tile(nxt, k_base, k_row, std::false_type{}, gt_nxt, lds_k);
         if (active) {
 
@@ -555,6 +578,7 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
             }
         }
 
+        if constexpr (PAIR || EARLY_B2 < 0) {
         // All V^T fragments of the tile are read here, in one scheduling region with the row-max
         // chain: the PV block below is bound by its vector instructions, so every LDS read moved out
         // of it shortens it (+3 % for the 24 reads that used to sit between its MFMAs), and the reads
@@ -567,6 +591,7 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
             for (int jj = 0; jj < 2; ++jj)
                 vf[s][db].s4[jj] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
                     (__attribute__((address_space(3))) short4_t *)(lds_v + v_rd_off[db] + (16 * s + 8 * jj) * ROW_BYTES));
+        }
         // ---- online softmax (exp2 domain) -------------------------------------
         float mx;
         {
