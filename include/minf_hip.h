@@ -11,7 +11,7 @@
  *     "last error";
  *   - no entry point allocates or frees device memory: the caller owns every
  *     buffer, including workspaces whose size the *_workspace_bytes() helpers
- *     report;
+ *     report (minf_vs_index_build_static brings its own fixed-size scratch);
  *   - `stream` is a hipStream_t passed as void* (NULL = the null stream);
  *     work is only enqueued, never synchronised;
  *   - tensors are described by a base pointer plus ELEMENT strides; the last
@@ -89,6 +89,27 @@ int minf_vs_index_build_ws(const int32_t *seqlens, const int32_t *vertical_idx,
                            int32_t *column_index, int batch, int heads, int rows,
                            int nnz_v, int nnz_s, int zero_fill, int32_t *error_flag,
                            void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * minf_vs_index_build_ws without a workspace argument and without any allocation: the tables and
+ * bitmaps live in a device array of MINF_VS_INDEX_STATIC_BYTES that is part of the library image
+ * (every GPU the library runs on holds its own copy until the process ends).  It has no
+ * counterpart in the reference; it is for callers that cannot allocate device memory: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  Same outputs, bit for
+ * bit, as minf_vs_index_build_ws.  Problems whose minf_vs_index_workspace_bytes() exceeds
+ * MINF_VS_INDEX_STATIC_BYTES return MINF_ERR_WORKSPACE before anything is enqueued (8 MiB holds
+ * 32 heads x 6096 slashes x 524288 tokens).  All calls on one GPU share the one array: calls that
+ * overlap in time on the same GPU (different streams or threads) race and must be serialised by
+ * the caller.  The device address of the array is looked up once per device, on the first call
+ * made with that device current.
+ */
+#define MINF_VS_INDEX_STATIC_BYTES (8u << 20)
+int minf_vs_index_build_static(const int32_t *seqlens, const int32_t *vertical_idx,
+                               const int32_t *slash_idx, int32_t *block_count,
+                               int32_t *block_offset, int32_t *column_count,
+                               int32_t *column_index, int batch, int heads, int rows,
+                               int nnz_v, int nnz_s, int zero_fill, int32_t *error_flag,
+                               void *stream);
 
 /*
  * Sparse flash-attention forward on one shared 64x64 bf16/f16 MFMA tile

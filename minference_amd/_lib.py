@@ -24,6 +24,7 @@ SIGNATURES = {
     "minf_vs_index_build": (c_int, [c_ptr] * 7 + [c_int] * 6 + [c_ptr, c_ptr]),
     "minf_vs_index_workspace_bytes": (ctypes.c_size_t, [c_int] * 4),
     "minf_vs_index_build_ws": (c_int, [c_ptr] * 7 + [c_int] * 6 + [c_ptr, c_ptr, ctypes.c_size_t, c_ptr]),
+    "minf_vs_index_build_static": (c_int, [c_ptr] * 7 + [c_int] * 6 + [c_ptr, c_ptr]),
     "minf_vs_attn_fwd": (c_int, [c_ptr] * 5 + [c_int] * 3 + [c_ptr]),
     "minf_bs_attn_fwd": (c_int, [c_ptr, c_ptr, c_int, c_int, c_ptr]),
     "minf_ashape_attn_fwd": (c_int, [c_ptr, c_int, c_int, c_ptr]),

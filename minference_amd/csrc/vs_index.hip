@@ -21,6 +21,7 @@
 // stores; all row offsets are 64-bit.
 #include "minf_common.h"
 #include <limits.h>
+#include <atomic>
 
 #define IDX_WAVES 4
 
@@ -594,6 +595,29 @@ extern "C" size_t minf_vs_index_workspace_bytes(int batch, int heads, int nnz_s,
     return (size_t)batch * heads * (size_t)idx_tab_ints(nnz_s, rows) * sizeof(int32_t);
 }
 
+// launches of the table-driven builder on a workspace that is known to be large enough
+static int index_build_tables(const int32_t *seqlens, const int32_t *vertical_idx, const int32_t *slash_idx,
+                              int32_t *block_count, int32_t *block_offset, int32_t *column_count,
+                              int32_t *column_index, int batch, int heads, int rows, int nnz_v, int nnz_s,
+                              int zero_fill, int32_t *error_flag, int32_t *workspace, long long total,
+                              hipStream_t stream) {
+    const long long nblk = (total + IDX_WAVES - 1) / IDX_WAVES;
+    if (nblk > 0x7fffffffLL || (long long)batch * heads > 65535) return MINF_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(vs_index_prep_kernel, dim3((unsigned)(batch * heads)), dim3(MINF_WAVE), 0,
+                       stream, slash_idx, workspace, nnz_s, rows);
+    int status = minf_launch_status();
+    if (status != MINF_OK) return status;
+    hipLaunchKernelGGL(vs_index_bitmap_kernel, dim3((unsigned)((idx_bm_words(rows) + 255) / 256), (unsigned)(batch * heads)),
+                       dim3(256), 0, stream, workspace, nnz_s, rows);
+    status = minf_launch_status();
+    if (status != MINF_OK) return status;
+    hipLaunchKernelGGL(vs_index_fast_kernel, dim3((unsigned)nblk), dim3(IDX_WAVES * MINF_WAVE), 0,
+                       stream, seqlens, vertical_idx, slash_idx, (const int32_t *)workspace,
+                       block_count, block_offset, column_count, column_index, heads, rows, nnz_v, nnz_s,
+                       zero_fill, error_flag, total);
+    return minf_launch_status();
+}
+
 extern "C" int minf_vs_index_build_ws(const int32_t *seqlens, const int32_t *vertical_idx,
                                       const int32_t *slash_idx, int32_t *block_count,
                                       int32_t *block_offset, int32_t *column_count,
@@ -609,20 +633,57 @@ extern "C" int minf_vs_index_build_ws(const int32_t *seqlens, const int32_t *ver
     if (!workspace || workspace_bytes < minf_vs_index_workspace_bytes(batch, heads, nnz_s, rows) ||
         ((uintptr_t)workspace & 3))
         return MINF_ERR_WORKSPACE;
-    const long long nblk = (total + IDX_WAVES - 1) / IDX_WAVES;
-    if (nblk > 0x7fffffffLL || (long long)batch * heads > 0x7fffffffLL) return MINF_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL(vs_index_prep_kernel, dim3((unsigned)(batch * heads)), dim3(MINF_WAVE), 0,
-                       (hipStream_t)stream, slash_idx, (int32_t *)workspace, nnz_s, rows);
-    int status = minf_launch_status();
-    if (status != MINF_OK) return status;
-    if ((long long)batch * heads > 65535) return MINF_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL(vs_index_bitmap_kernel, dim3((unsigned)((idx_bm_words(rows) + 255) / 256), (unsigned)(batch * heads)),
-                       dim3(256), 0, (hipStream_t)stream, (int32_t *)workspace, nnz_s, rows);
-    status = minf_launch_status();
-    if (status != MINF_OK) return status;
-    hipLaunchKernelGGL(vs_index_fast_kernel, dim3((unsigned)nblk), dim3(IDX_WAVES * MINF_WAVE), 0,
-                       (hipStream_t)stream, seqlens, vertical_idx, slash_idx, (const int32_t *)workspace,
-                       block_count, block_offset, column_count, column_index, heads, rows, nnz_v, nnz_s,
-                       zero_fill, error_flag, total);
-    return minf_launch_status();
+    return index_build_tables(seqlens, vertical_idx, slash_idx, block_count, block_offset, column_count,
+                              column_index, batch, heads, rows, nnz_v, nnz_s, zero_fill, error_flag,
+                              (int32_t *)workspace, total, (hipStream_t)stream);
+}
+
+// ---- the entry point that allocates nothing ---------------------------------------------------
+// The tables and bitmaps of minf_vs_index_build_ws live in this array instead of a caller-owned
+// workspace.  Every GPU holds its own copy at its own address; host code only ever uses the address
+// hipGetSymbolAddress returned for the current device, never the array's name.  Nothing in it has
+// to start at zero: the table pass and the bitmap pass write every word the row-block pass reads.
+static __device__ __align__(256) int32_t scratch[MINF_VS_INDEX_STATIC_BYTES / sizeof(int32_t)];
+
+#define IDX_MAX_DEVICES 64
+static std::atomic<int32_t *> scratch_ptr[IDX_MAX_DEVICES];
+
+static int scratch_for_current_device(int32_t **out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return minf_hip_status(e);
+    if (dev < 0 || dev >= IDX_MAX_DEVICES) return MINF_ERR_UNSUPPORTED;
+    int32_t *ptr = scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!ptr) {
+        // first call on this device; two threads racing here get the same address
+        e = hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return minf_hip_status(e);
+        if (!ptr) return MINF_ERR_HIP_BASE;
+        scratch_ptr[dev].store(ptr, std::memory_order_release);
+    }
+    *out = ptr;
+    return MINF_OK;
+}
+
+extern "C" int minf_vs_index_build_static(const int32_t *seqlens, const int32_t *vertical_idx,
+                                          const int32_t *slash_idx, int32_t *block_count,
+                                          int32_t *block_offset, int32_t *column_count,
+                                          int32_t *column_index, int batch, int heads, int rows,
+                                          int nnz_v, int nnz_s, int zero_fill, int32_t *error_flag,
+                                          void *stream) {
+    if (!seqlens || !vertical_idx || !slash_idx || !block_count || !block_offset ||
+        !column_count || !column_index)
+        return MINF_ERR_INVALID_ARG;
+    if (batch < 0 || heads < 0 || rows < 0 || nnz_v < 1 || nnz_s < 1) return MINF_ERR_INVALID_ARG;
+    const long long total = (long long)batch * heads * rows;
+    if (total == 0) return MINF_OK;
+    // sizes beyond the array are refused before any HIP call
+    if (minf_vs_index_workspace_bytes(batch, heads, nnz_s, rows) > (size_t)MINF_VS_INDEX_STATIC_BYTES)
+        return MINF_ERR_WORKSPACE;
+    int32_t *ws = nullptr;
+    const int st = scratch_for_current_device(&ws);
+    if (st != MINF_OK) return st;
+    return index_build_tables(seqlens, vertical_idx, slash_idx, block_count, block_offset, column_count,
+                              column_index, batch, heads, rows, nnz_v, nnz_s, zero_fill, error_flag,
+                              ws, total, (hipStream_t)stream);
 }

@@ -46,6 +46,11 @@ def test_argument_validation_needs_no_gpu(lib):
     # null pointers / bad sizes are rejected before any HIP call
     assert lib.minf_vs_index_build(None, None, None, None, None, None, None, 1, 1, 1, 1, 1, 1, None, None) == -1
     assert lib.minf_topk_indices(None, 1, 10, 10, 5, None, 5, -1, None) == -1
+    # the entry point without a workspace argument: null pointers, then a problem larger than its
+    # fixed array (refused by size alone, before any HIP call)
+    assert lib.minf_vs_index_build_static(None, None, None, None, None, None, None, 1, 1, 1, 1, 1, 1, None, None) == -1
+    assert lib.minf_vs_index_workspace_bytes(1, 64, 6096, 16384) > (8 << 20)
+    assert lib.minf_vs_index_build_static(16, 16, 16, 16, 16, 16, 16, 1, 64, 16384, 1000, 6096, 1, None, None) == -4
     t = _lib.QKVO()
     assert lib.minf_dense_attn_fwd(ctypes.byref(t), None) == -1          # null tensors
     t.q = t.k = t.v = t.o = 16
