@@ -12,7 +12,7 @@ from __future__ import annotations
 import torch
 
 from . import _lib
-from .ops import _check_qkv, _prep
+from .ops import _check_qkv, _narrow_fp32, _prep
 
 LAST_Q = 64            # minference_forward.py:41
 FORCE_VERTICAL = 30    # :606
@@ -21,7 +21,7 @@ FORCE_SLASH = 100      # :610
 
 def _prep16(q, k):
     if q.dtype == torch.float32:
-        q, k = q.bfloat16(), k.bfloat16()
+        q, k = _narrow_fp32(q, k)          # fp16 when the values fit, else bf16
     elif q.dtype not in (torch.bfloat16, torch.float16):
         raise ValueError(f"unsupported dtype {q.dtype}")
     if q.shape[-1] != 128:

@@ -33,6 +33,23 @@ def _prep(t: torch.Tensor) -> torch.Tensor:
     return t
 
 
+_F16_SAFE_ABS = 32768.0
+
+
+def _narrow_fp32(*tensors):
+    """16-bit operands for fp32 inputs.  The reference computes at the input element type
+    (pit_sparse_flash_attention_v2.py:96-99, :123 cast q and p to Q's dtype), which for fp32
+    means tl.dot's default TF32 products: 10 explicit mantissa bits.  fp16 operands have the same 10
+    bits, so fp32 tensors are narrowed to fp16 whenever every |value| is at most 32768 (one
+    max-abs reduction and a host read per call -- the fp32 path is the reference's CPU-checkable
+    case, not the serving path); otherwise to bf16 (8 bits, fp32's range).  Accumulation,
+    softmax statistics and the scale stay fp32 either way."""
+    amax = torch.stack([torch.linalg.vector_norm(t.reshape(-1).float(), float("inf")) if t.numel() else
+                        torch.zeros((), device=t.device) for t in tensors]).max().item()
+    dt = torch.float16 if amax <= _F16_SAFE_ABS else torch.bfloat16     # (NaN / inf -> bf16)
+    return tuple(t.to(dt) for t in tensors)
+
+
 def _check_qkv(q, k, v):
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
         raise ValueError("q, k, v must be [batch, heads, n, head_dim]")
@@ -56,7 +73,7 @@ class _Call:
         self.head_dim = q.shape[-1]
         if q.dtype == torch.float32:
             # the tile engine computes on 16-bit operands with fp32 accumulation
-            q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
+            q, k, v = _narrow_fp32(q, k, v)
         elif q.dtype not in (torch.bfloat16, torch.float16):
             raise ValueError(f"unsupported dtype {q.dtype}")
         D = q.shape[-1]

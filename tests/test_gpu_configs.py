@@ -1,0 +1,204 @@
+"""BASELINE configs at the shapes they name (head counts, GQA ratios, lengths), through the C ABI:
+config 3 at 524288 tokens (index builder, bit-exact), config 2 with 32 query / 8 kv heads, config 4
+with 4:1 GQA, and config 5 as a two-layer Llama-3-8B-shaped stack at 262144 tokens with the seeded
+70/20/10 pattern table.  Attention rows are compared with the fp32 masked-dense oracle on the index
+entries the GPU produced (max-abs 2e-2, mean-abs 1e-3); index rows with the reference algorithm."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+from tests import gen
+
+pytestmark = pytest.mark.gpu
+
+
+def _rows_reference(q_rows, k, v, mask):
+    s = (q_rows.float() @ k.float().T) * (q_rows.shape[-1] ** -0.5)
+    s = torch.where(torch.as_tensor(mask), s, torch.tensor(-torch.inf))
+    return torch.softmax(s, dim=-1) @ v.float()
+
+
+def _check_vs_row_block(tag, out_rows, q_rows, k, v, v_list, s_list, bc_m, bo_m, cc_m, ci_m, m, n):
+    """One row block of a vertical-slash head: the GPU's index row equals the reference algorithm's
+    row, and the attention rows agree with the fp32 masked-dense result on that row."""
+    rbo, rci = O.vs_index_row_py(v_list, s_list, m, n)
+    assert int(bc_m) == len(rbo) and int(cc_m) == len(rci), tag
+    assert bo_m[: len(rbo)].tolist() == rbo and ci_m[: len(rci)].tolist() == rci, tag
+    mask = O.vs_mask_rows(len(rbo), rbo, len(rci), rci, m, n)
+    err = (out_rows.float().cpu() - _rows_reference(q_rows, k, v, mask[: q_rows.shape[0]])).abs()
+    print(f"  {tag}: max-abs {err.max().item():.3e} mean-abs {err.mean().item():.3e}", flush=True)
+    assert err.max() <= 2e-2 and err.mean() <= 1e-3, tag
+
+
+def test_config3_index_at_524288_tokens(gpu):
+    """BASELINE config 3 at its longer length: 32 heads, 524288 tokens, 1000 verticals (0..3 forced),
+    6096 slashes (0..63 forced), seeded.  Both HIP builders on all 32 heads must produce identical
+    full tensors (7.4 GB each, zero tails included; compared on the GPU), and heads 0, 17 and 31 are
+    compared bit for bit, full tensors, with the C restatement of the reference kernel."""
+    from minference_amd import convert_vertical_slash_indexes
+    n, heads = 524288, 32
+    v, s = gen.vs_index_inputs(heads, n, 1000, 6096, seed=300)
+    seqlens = torch.tensor([n], dtype=torch.int32, device=gpu)
+    vg, sg = torch.from_numpy(v).to(gpu), torch.from_numpy(np.ascontiguousarray(s)).to(gpu)
+    print("case c3-524288 table-driven builder", flush=True)
+    fast = convert_vertical_slash_indexes(seqlens, vg, sg, n, 64, 64)
+    print("case c3-524288 plain builder", flush=True)
+    plain = convert_vertical_slash_indexes(seqlens, vg, sg, n, 64, 64, use_tables=False)
+    torch.cuda.synchronize()
+    names = ["block_count", "block_offset", "column_count", "column_index"]
+    for name, a, b in zip(names, fast, plain):
+        assert a.dtype == torch.int32 and torch.equal(a, b), f"builders differ in {name}"
+    del plain
+    torch.cuda.empty_cache()
+    for h in (0, 17, 31):
+        print(f"case c3-524288 oracle head {h}", flush=True)
+        ref = O.vs_index_build([n], v[:, h:h + 1], s[:, h:h + 1], n)
+        for name, a, r in zip(names, fast, ref):
+            got = a[:, h:h + 1].cpu().numpy()
+            assert got.shape == r.shape and np.array_equal(got, r), f"head {h}: {name} differs from the oracle"
+
+
+def test_config2_all_32_query_heads_8_kv_heads(gpu):
+    """BASELINE config 2 at its stated geometry (131072 tokens, 32 query / 8 kv heads, bf16,
+    vertical 1000, slash 6096): the launch shape the benchmark times.  Sampled (head, row block)
+    pairs from four kv groups, incl. the last head and the last row block."""
+    import minference_amd as M
+    n, hq, hk = 131072, 32, 8
+    q, k, v, _ = gen.planted_layer(n, hq, hk, seed=100, dtype=torch.bfloat16)
+    qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
+    v_idx, s_idx = M.estimate_vertical_slash(qg, kg, 1000, 6096)
+    seqlens = torch.full((1,), n, dtype=torch.int32, device=gpu)
+    bc, bo, cc, ci = M.convert_vertical_slash_indexes(seqlens, v_idx, s_idx, n, 64, 64, zero_fill=False)
+    out = M.vertical_slash_attention_from_index(qg, kg, vg, bc, bo, cc, ci, seqlens)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all()
+    rows = n // 64
+    vi_c, si_c = v_idx.cpu().numpy(), s_idx.cpu().numpy()
+    for h, m in [(0, 0), (3, 700), (13, 1), (13, 1999), (22, 1024), (31, rows - 1), (31, 64), (26, 333)]:
+        print(f"case c2-32x8 head={h} row-block={m}", flush=True)
+        kv = h // (hq // hk)
+        _check_vs_row_block(f"head {h} row block {m}", out[0, h, m * 64: m * 64 + 64], q[0, h, m * 64: m * 64 + 64],
+                            k[0, kv], v[0, kv], vi_c[0, h].tolist(), si_c[0, h].tolist(),
+                            bc[0, h, m], bo[0, h, m].cpu().numpy(), cc[0, h, m], ci[0, h, m].cpu().numpy(), m, n)
+
+
+def test_config4_gqa_4_to_1(gpu):
+    """BASELINE config 4 with the 4:1 GQA ratio of its 32 q / 8 kv heads (8 query heads on 2 kv
+    heads at 131072 tokens): top-100 block index with diagonal and block 0 forced, sampled query
+    blocks of heads from both kv groups against explicit per-block means and the masked-dense rows."""
+    from minference_amd.ops import _build_block_index, block_sparse_attention_from_index
+    n, hq, hk, top_k = 131072, 8, 2, 100
+    q, k, v, _ = gen.planted_layer(n, hq, hk, seed=100, dtype=torch.bfloat16)
+    qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
+    bi = _build_block_index(qg, kg, top_k, force_diag_first=True)
+    out = block_sparse_attention_from_index(qg, kg, vg, bi)
+    torch.cuda.synchronize()
+    R = n // 64 + 1
+    assert tuple(bi.shape) == (1, hq, R, top_k)
+    bic = bi[0].cpu().numpy()
+    for h, m in [(0, 0), (3, 150), (4, 99), (5, 1200), (7, 2047), (2, 100)]:
+        print(f"case c4-gqa head={h} query-block={m}", flush=True)
+        kv = h // (hq // hk)
+        # pooled scores by an explicit loop over the causal key blocks of this query block
+        qbar = q[0, h, m * 64: m * 64 + 64].float().mean(0)
+        p = np.full(R, -np.inf)
+        for j in range(m + 1):
+            p[j] = float(qbar @ k[0, kv, j * 64: j * 64 + 64].float().mean(0))
+        p[m] = p[0] = np.inf
+        row = bic[h, m]
+        assert (np.diff(row) > 0).all()
+        kth = np.sort(p)[::-1][top_k - 1]
+        sel = np.zeros(R, bool)
+        sel[row] = True
+        if np.isfinite(kth):
+            tol = 1e-5 * max(1.0, abs(kth))
+            assert sel[p > kth + tol].all() and (p[sel] >= kth - tol).all()
+        else:
+            assert sel[: m + 1].all()
+        mask = np.zeros((64, n), bool)
+        rr = np.arange(m * 64, m * 64 + 64)
+        for j in row[: min(m + 1, top_k)]:
+            cols = np.arange(j * 64, min(j * 64 + 64, n))
+            mask[:, cols] |= cols[None, :] <= rr[:, None]
+        err = (out[0, h, m * 64: m * 64 + 64].float().cpu()
+               - _rows_reference(q[0, h, m * 64: m * 64 + 64], k[0, kv], v[0, kv], mask)).abs()
+        print(f"  max-abs {err.max().item():.3e} mean-abs {err.mean().item():.3e}", flush=True)
+        assert err.max() <= 2e-2 and err.mean() <= 1e-3
+
+
+def test_config5_two_layer_llama3_8b_shape_at_262144_tokens(gpu, monkeypatch):
+    """BASELINE config 5 with two of its 32 layers: random-init Llama-3-8B shapes (hidden 4096, 32 q /
+    8 kv heads, RoPE theta 500000, SwiGLU 14336, vocab 128256), 262144 random tokens, the seeded
+    70 % vertical_slash / 20 % block_sparse / 10 % A-shape table through minference_prefill_forward.
+    The logits must be finite; for layer 0, one head of every pattern type is checked on sampled row
+    blocks against the oracle masks built from what the dispatcher's own stages produce on that
+    layer's q/k (the stages are deterministic, so re-running them gives the indices it used)."""
+    import minference_amd as M
+    from minference_amd import llama
+    from minference_amd.ops import _build_block_index
+    n = 262144
+    cfg = llama.LlamaConfig(num_layers=2)
+    model = llama.LlamaPrefill(cfg, device=gpu, seed=0)
+    ids = torch.randint(0, cfg.vocab_size, (n,), generator=torch.Generator().manual_seed(500))
+    table = llama.seeded_pattern_mix(cfg.num_layers, cfg.num_heads, seed=501)
+    types = {t: [h for h in range(cfg.num_heads) if table[0][str(h)][0] == t]
+             for t in ("vertical_and_slash", "block_sparse", "stream_llm")}
+    assert all(types.values()), types
+    picks = {t: hs[-1] for t, hs in types.items()}
+    blocks = [0, 70, 2500, n // 64 - 1]
+    captured = {}
+    real = llama.minference_prefill_forward
+
+    def recording(q, k, v, kwargs):
+        out = real(q, k, v, kwargs)
+        if kwargs["layer_idx"] == 0:
+            # q is overwritten by the next layer: keep the sampled rows, and K/V of the heads used
+            for t, h in picks.items():
+                kv = h // (cfg.num_heads // cfg.num_kv_heads)
+                captured[t] = {
+                    "h": h, "k": k[0, kv].float().cpu(), "v": v[0, kv].float().cpu(),
+                    "q": {m: q[0, h, m * 64: m * 64 + 64].clone() for m in blocks},
+                    "o": {m: out[0, h, m * 64: m * 64 + 64].clone() for m in blocks},
+                    "q_full": q[:, h:h + 1].clone(), "k_full": k[:, kv:kv + 1].clone()}
+        return out
+
+    monkeypatch.setattr(llama, "minference_prefill_forward", recording)
+    print("case c5 two-layer prefill", flush=True)
+    logits, _ = model.prefill(ids, {"best_pattern": table})
+    torch.cuda.synchronize()
+    assert logits.shape == (cfg.vocab_size,) and torch.isfinite(logits).all()
+
+    # vertical-slash head
+    c = captured["vertical_and_slash"]
+    v_idx, s_idx = M.estimate_vertical_slash(c["q_full"], c["k_full"], 1000, 6096)
+    seqlens = torch.full((1,), n, dtype=torch.int32, device=gpu)
+    bc, bo, cc, ci = M.convert_vertical_slash_indexes(seqlens, v_idx, s_idx, n, 64, 64, zero_fill=False)
+    vl, sl = v_idx[0, 0].cpu().tolist(), s_idx[0, 0].cpu().tolist()
+    for m in blocks:
+        print(f"case c5 vertical_slash head={c['h']} row-block={m}", flush=True)
+        _check_vs_row_block(f"vs head {c['h']} row block {m}", c["o"][m], c["q"][m].cpu(), c["k"], c["v"], vl, sl,
+                            bc[0, 0, m], bo[0, 0, m].cpu().numpy(), cc[0, 0, m], ci[0, 0, m].cpu().numpy(), m, n)
+    # block-sparse head (top-100, no forced blocks: the dispatcher's call, minference_forward.py:616-618)
+    c = captured["block_sparse"]
+    bi = _build_block_index(c["q_full"], c["k_full"], 100)[0, 0].cpu().numpy()
+    for m in blocks:
+        print(f"case c5 block_sparse head={c['h']} row-block={m}", flush=True)
+        mask = np.zeros((64, n), bool)
+        rr = np.arange(m * 64, m * 64 + 64)
+        for j in bi[m, : min(m + 1, 100)]:
+            cols = np.arange(j * 64, min(j * 64 + 64, n))
+            mask[:, cols] |= cols[None, :] <= rr[:, None]
+        err = (c["o"][m].float().cpu() - _rows_reference(c["q"][m].cpu(), c["k"], c["v"], mask)).abs()
+        print(f"  max-abs {err.max().item():.3e} mean-abs {err.mean().item():.3e}", flush=True)
+        assert err.max() <= 2e-2 and err.mean() <= 1e-3
+    # A-shape head: sink 128 + local 4096
+    c = captured["stream_llm"]
+    for m in blocks:
+        print(f"case c5 a-shape head={c['h']} row-block={m}", flush=True)
+        r = np.arange(m * 64, m * 64 + 64)[:, None]
+        col = np.arange(n)[None, :]
+        mask = ((col <= r) & (col > r - 4096)) | ((col < 128) & (col <= r - 4096))
+        err = (c["o"][m].float().cpu() - _rows_reference(c["q"][m].cpu(), c["k"], c["v"], mask)).abs()
+        print(f"  max-abs {err.max().item():.3e} mean-abs {err.mean().item():.3e}", flush=True)
+        assert err.max() <= 2e-2 and err.mean() <= 1e-3

@@ -77,6 +77,11 @@ def test_config1_shape_fp32_full(gpu):
     ref = O.vertical_slash_sparse_attention(q[:, :1], k[:, :1], v[:, :1], v_idx[:, :1].cpu(), s_idx[:, :1].cpu())
     err = (out[:, :1] - ref).abs()
     assert err.max() <= 2e-2 and err.mean() <= 1e-3
+    # the inputs are N(0,1)/sqrt(128): outputs are of order 1e-2, so the bound that means something
+    # is the one relative to the output magnitude
+    scale = ref.abs().max()
+    print(f"config 1: max-abs {err.max().item():.3e} mean-abs {err.mean().item():.3e} max|ref| {scale.item():.3e}", flush=True)
+    assert err.max() <= 2e-2 * scale and err.mean() <= 1e-3 * scale
 
 
 def test_config2_full_size_sampled_row_blocks(gpu):

@@ -1,6 +1,9 @@
 """Pins the attention side of the oracle (masks + fp32 masked-dense softmax) through special
 cases that reduce to torch's scaled_dot_product_attention and per-element brute force."""
+import math
+
 import numpy as np
+import pytest
 import torch
 
 from oracle import oracle as O
@@ -75,6 +78,55 @@ def test_block_sparse_index_properties_and_dense_limit():
     bf = O.bs_block_index(q, k, 3, force_diag_first=True)
     for m in range(10):
         assert 0 in bf[0, 0, m].tolist() and m in bf[0, 0, m].tolist()
+
+
+@pytest.mark.parametrize("n,d,top_k,force", [(128, 8, 2, False), (200, 16, 3, False), (192, 4, 2, True), (70, 8, 5, False)])
+def test_block_sparse_index_against_explicit_loops(n, d, top_k, force):
+    """bs_block_index restated without any vectorised pooling: per-block means by Python loops over
+    tokens (block_sparse_flash_attention.py:159-160), one dot product per (query block, key block)
+    pair (:163), block-causal -inf (:164), then the k best by an explicit scan.  The caller's padding
+    (:178: 64 - n % 64 zero rows, a WHOLE extra block when n % 64 == 0) is applied here with loops as
+    well, so a wrong pooling axis, a mean over the wrong count or a missing extra block would show."""
+    q, k, _ = gen.qkv(1, 2, 2, n, d, seed=40 + n, scale=1.0)
+    pad = 64 - (n & 63)
+    assert pad == 64 if n % 64 == 0 else pad == 64 - n % 64
+    qp = torch.nn.functional.pad(q, [0, 0, 0, pad])
+    kp = torch.nn.functional.pad(k, [0, 0, 0, pad])
+    got = O.bs_block_index(qp, kp, top_k, force_diag_first=force)
+    R = (n + pad) // 64
+    assert R == n // 64 + 1
+    kk = min(top_k, R)
+    assert tuple(got.shape) == (1, 2, R, kk)
+    for h in range(2):
+        qbar = [[0.0] * d for _ in range(R)]
+        kbar = [[0.0] * d for _ in range(R)]
+        for blk in range(R):
+            for t in range(64):                       # padded rows are zeros and still count in the mean
+                tok = blk * 64 + t
+                for e in range(d):
+                    if tok < n:
+                        qbar[blk][e] += float(q[0, h, tok, e])
+                        kbar[blk][e] += float(k[0, h, tok, e])
+            for e in range(d):
+                qbar[blk][e] /= 64.0
+                kbar[blk][e] /= 64.0
+        for m in range(R):
+            score = []
+            for j in range(R):
+                if j > m:
+                    score.append(-math.inf)
+                    continue
+                sc = sum(qbar[m][e] * kbar[j][e] for e in range(d))
+                if force and (j == m or j == 0):
+                    sc = math.inf
+                score.append(sc)
+            order = sorted(range(R), key=lambda j: (-score[j], j))[:kk]      # ties: lowest block id
+            want = sorted(order)
+            row = got[0, h, m].tolist()
+            if row != want:
+                # only a near-tie at the k-th score may differ (float32 einsum vs Python doubles)
+                kth = score[order[-1]]
+                assert all(abs(score[j] - kth) < 1e-5 for j in set(row) ^ set(want)), (h, m, row, want)
 
 
 def test_ashape_mask_closed_form():
