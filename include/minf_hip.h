@@ -40,6 +40,11 @@ extern "C" {
 /* Library version as major*10000 + minor*100 + patch. */
 int minf_version(void);
 
+/* sizeof(minf_qkvo) as this library was compiled.  A caller built against another revision of this
+ * header passes a struct of another size and must not call the attention entry points: compare with
+ * its own sizeof(minf_qkvo) once at start-up. */
+size_t minf_qkvo_size(void);
+
 /* Static text for a status code (pure function, thread-safe). */
 const char *minf_status_string(int status);
 
@@ -124,7 +129,8 @@ int minf_vs_index_build_static(const int32_t *seqlens, const int32_t *vertical_i
  *   seqlens [batch] int32 may be NULL (= n for every batch).  Rows >= seqlen
  *   are written as zeros (the reference leaves its zeros_like buffer untouched).
  *   sm_scale multiplies q.k before the softmax (reference: head_dim^-0.5).
- *   Every o element of every row < n is written; nothing else is.
+ *   Every o element of every row < n (of every selected head) is written; nothing else is.
+ *   Token strides must be at least head_dim (rows must not overlap).
  */
 typedef struct minf_qkvo {
     const void *q, *k, *v;
@@ -133,6 +139,16 @@ typedef struct minf_qkvo {
     int batch, heads_q, heads_kv, n, head_dim, dtype;
     const int32_t *seqlens;
     float sm_scale;
+    /* Optional head selection (per-head pattern tables: reference
+     * minference/modules/minference_forward.py:621, :657-667 loops over heads and calls one operator
+     * per head).  head_slot NULL: every query head is processed and index tensors have heads_q
+     * heads.  Otherwise head_slot is a device array [heads_q]: head h is skipped when
+     * head_slot[h] < 0 (its rows of o are not touched) and else reads its index rows at head
+     * position head_slot[h] of index tensors that have index_heads heads.  q, k, v, o are always
+     * addressed with the real head number, so a launch per pattern type writes its heads of one
+     * shared output in place. */
+    const int32_t *head_slot;
+    int index_heads;
 } minf_qkvo;
 
 /*
@@ -209,6 +225,21 @@ int minf_vs_estimate(const void *q, const void *k, const int64_t *q_stride,
                      size_t workspace_bytes, void *stream);
 
 /*
+ * minf_vs_estimate for a subset of the query heads (per-head pattern tables: the reference estimates
+ * inside its loop over heads, minference/modules/minference_forward.py:657-667, only for the heads
+ * whose pattern is vertical_and_slash).  head_slot [heads_q] int32 (device): head h is skipped when
+ * head_slot[h] < 0, otherwise its score rows are row head_slot[h] of vertical / slash
+ * [batch, index_heads, n]; q and k are addressed with the real head numbers.  Workspace:
+ * minf_vs_estimate_workspace_bytes(batch, index_heads, n).
+ */
+int minf_vs_estimate_heads(const void *q, const void *k, const int64_t *q_stride,
+                           const int64_t *k_stride, int batch, int heads_q, int heads_kv, int n,
+                           int head_dim, int dtype, float sm_scale, int last_q, int force_vertical,
+                           int force_slash, const int32_t *head_slot, int index_heads,
+                           float *vertical, float *slash, void *workspace,
+                           size_t workspace_bytes, void *stream);
+
+/*
  * Indices of the k largest entries of each fp32 row, written in ASCENDING
  * INDEX order (ties at the k-th value: lowest index first).  Replaces
  * torch.topk(...).indices followed by the sort in the op wrapper (reference
@@ -244,6 +275,24 @@ int minf_topk_indices_pair(const float *scores_a, int k_a, int32_t *out_a, int64
                            int64_t row_stride, void *stream);
 
 /*
+ * minf_topk_indices_pair with a different k for every row (the per-head vertical_size / slash_size
+ * of a pattern table, reference minference_forward.py:621-625): row i keeps k_rows[i] entries
+ * (device int32 [rows], clamped to 1..k_max) and the remaining k_max - k_rows[i] output slots are
+ * padding.  pad_mode 0: left unwritten; 1: the constant pad_value; 2: the last selected value
+ * repeated.  For the index builder both paddings are no-ops of the reference's merge loop
+ * (csrc/vertical_slash_index.cu:70-95): a vertical index at or beyond every range end is never
+ * emitted (pad verticals with a large constant), and a repeated slash offset neither starts nor
+ * extends a range (pad slashes with mode 2), so one index build and one attention launch with the
+ * list widths k_max serve heads with different sizes and produce, per head, the tensors of its own
+ * sizes (followed by zeros).
+ */
+int minf_topk_indices_pair_ragged(const float *scores_a, const int32_t *k_rows_a, int k_max_a, int32_t *out_a,
+                                  int64_t out_stride_a, int reverse_base_a, int pad_mode_a, int pad_value_a,
+                                  const float *scores_b, const int32_t *k_rows_b, int k_max_b, int32_t *out_b,
+                                  int64_t out_stride_b, int reverse_base_b, int pad_mode_b, int pad_value_b,
+                                  int rows, int n, int64_t row_stride, void *stream);
+
+/*
  * Block index of top-k block-sparse attention: replaces _build_block_index (reference
  * minference/ops/block_sparse_flash_attention.py:151-166) together with the zero padding its
  * caller applies first (:178-180).  Q and K are mean-pooled over 64-token blocks (the token axis
@@ -264,6 +313,18 @@ int minf_bs_block_index(const void *q, const void *k, const int64_t *q_stride,
                         int head_dim, int dtype, int top_k, int force_diag_first,
                         int32_t *block_index, void *workspace, size_t workspace_bytes,
                         void *stream);
+
+/*
+ * minf_bs_block_index for a subset of the query heads (head_slot as in minf_vs_estimate_heads):
+ * block_index [batch, index_heads, rows, min(top_k, rows)]; workspace
+ * minf_bs_block_index_workspace_bytes(batch, index_heads, heads_kv, n).
+ */
+int minf_bs_block_index_heads(const void *q, const void *k, const int64_t *q_stride,
+                              const int64_t *k_stride, int batch, int heads_q, int heads_kv, int n,
+                              int head_dim, int dtype, int top_k, int force_diag_first,
+                              const int32_t *head_slot, int index_heads,
+                              int32_t *block_index, void *workspace, size_t workspace_bytes,
+                              void *stream);
 
 /*
  * Offline pattern search: the share of the exact causal softmax mass that candidate sparse

@@ -21,6 +21,7 @@ c_ptr = ctypes.c_void_p
 SIGNATURES = {
     "minf_version": (c_int, []),
     "minf_status_string": (ctypes.c_char_p, [c_int]),
+    "minf_qkvo_size": (ctypes.c_size_t, []),
     "minf_vs_index_build": (c_int, [c_ptr] * 7 + [c_int] * 6 + [c_ptr, c_ptr]),
     "minf_vs_index_workspace_bytes": (ctypes.c_size_t, [c_int] * 4),
     "minf_vs_index_build_ws": (c_int, [c_ptr] * 7 + [c_int] * 6 + [c_ptr, c_ptr, ctypes.c_size_t, c_ptr]),
@@ -33,6 +34,12 @@ SIGNATURES = {
     "minf_vs_estimate_workspace_bytes": (ctypes.c_size_t, [c_int, c_int, c_int]),
     "minf_vs_estimate": (c_int, [c_ptr, c_ptr, c_ptr, c_ptr] + [c_int] * 6 + [c_f32] + [c_int] * 3
                          + [c_ptr, c_ptr, c_ptr, ctypes.c_size_t, c_ptr]),
+    "minf_vs_estimate_heads": (c_int, [c_ptr, c_ptr, c_ptr, c_ptr] + [c_int] * 6 + [c_f32] + [c_int] * 3 + [c_ptr, c_int]
+                               + [c_ptr, c_ptr, c_ptr, ctypes.c_size_t, c_ptr]),
+    "minf_topk_indices_pair_ragged": (c_int, [c_ptr, c_ptr, c_int, c_ptr, c_i64, c_int, c_int, c_int] * 2
+                                      + [c_int, c_int, c_i64, c_ptr]),
+    "minf_bs_block_index_heads": (c_int, [c_ptr, c_ptr, c_ptr, c_ptr] + [c_int] * 8 + [c_ptr, c_int]
+                                  + [c_ptr, c_ptr, ctypes.c_size_t, c_ptr]),
     "minf_topk_indices": (c_int, [c_ptr, c_int, c_int, c_i64, c_int, c_ptr, c_i64, c_int, c_ptr]),
     "minf_topk_indices_block_causal": (c_int, [c_ptr, c_int, c_int, c_i64, c_int, c_ptr, c_i64, c_int, c_ptr]),
     "minf_topk_indices_pair": (c_int, [c_ptr, c_int, c_ptr, c_i64, c_int] * 2 + [c_int, c_int, c_i64, c_ptr]),
@@ -58,6 +65,8 @@ class QKVO(ctypes.Structure):
         ("head_dim", c_int), ("dtype", c_int),
         ("seqlens", c_ptr),
         ("sm_scale", c_f32),
+        ("head_slot", c_ptr),
+        ("index_heads", c_int),
     ]
 
 
@@ -81,6 +90,9 @@ def load():
             fn = getattr(lib, name)
             fn.restype = res
             fn.argtypes = args
+        if lib.minf_qkvo_size() != ctypes.sizeof(QKVO):
+            raise MinfError(f"{LIB_PATH} was built from another revision of include/minf_hip.h "
+                            f"(struct minf_qkvo: {lib.minf_qkvo_size()} bytes there, {ctypes.sizeof(QKVO)} here); rebuild it")
         _lib = lib
     return _lib
 

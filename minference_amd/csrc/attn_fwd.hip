@@ -97,6 +97,10 @@ struct AttnParams {
     int n_init, n_local, dense_from;
     long long total_wg;
     int descending;          // row blocks are handed out from the last one down
+    // optional head selection: head_slot[h] < 0 skips query head h; otherwise it is the head's
+    // position in the index tensors, which then have index_heads heads (index_heads = hq without it)
+    const int *head_slot;
+    int index_heads;
 };
 
 typedef const __attribute__((address_space(4))) int *cint_ptr;
@@ -277,6 +281,11 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
     const int hkv = (int)(rest % p.hk);
     const int b = (int)(rest / p.hk);
     const int h = hkv * group + hin;
+    int hs = h;                                    // head position in the index tensors
+    if (p.head_slot) {
+        hs = as_const(p.head_slot)[h];
+        if (hs < 0) return;                        // not one of this launch's heads (workgroup-uniform)
+    }
 
     const int tid = (int)threadIdx.x;
     const int lane = tid & 63;
@@ -309,7 +318,7 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
     const char *k_base = p.k + ((long long)b * p.ks[0] + (long long)hkv * p.ks[1]) * 2;
     const char *v_base = p.v + ((long long)b * p.vs[0] + (long long)hkv * p.vs[1]) * 2;
     const long long k_row = p.ks[2] * 2, v_row = p.vs[2] * 2;
-    const long long ridx = ((long long)b * p.hq + h) * p.rows + min(m, p.rows - 1);
+    const long long ridx = ((long long)b * p.index_heads + hs) * p.rows + min(m, p.rows - 1);
 
     // ---- Q fragments (B operand of S^T): row qrow, d = 16*ks + 8*g + 0..7 ----
     Frag qf[8];
@@ -331,7 +340,7 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
     if constexpr (PAIR && MODE == MODE_BS) {
         bs_na = min(mA + 1, p.max_blocks);
         bs_nb = (2 * mslot + 1 < p.rows && (2 * mslot + 1) * BM < seqlen) ? min(mA + 2, p.max_blocks) : 0;
-        const long long rbase = ((long long)b * p.hq + h) * p.bidx_rows;
+        const long long rbase = ((long long)b * p.index_heads + hs) * p.bidx_rows;
         for (int i = tid; i < bs_na; i += NT) lds_list[i] = p.bidx[(rbase + mA) * p.max_blocks + i];
         for (int i = tid; i < bs_nb; i += NT) lds_list[BS_PAIR_MAX + i] = p.bidx[(rbase + mA + 1) * p.max_blocks + i];
         __syncthreads();
@@ -561,7 +570,9 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
                 wlo = qrow >= p.dense_from ? -(1 << 30) : qrow - cur.start - p.n_local - 4 * g;
                 slim = p.n_init - cur.start - 4 * g;
             } else {
-                need_mask = (cur.start + BN - 1 > wrow_lo) || (cur.start + BN > seqlen);
+                // (a list entry below zero is no key at all: the reference would read out of bounds)
+                need_mask = (cur.start + BN - 1 > wrow_lo) || (cur.start + BN > seqlen) || cur.start < 0;
+                wlo = -cur.start - 4 * g - 1;
             }
         }
         if (need_mask) {
@@ -572,6 +583,9 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
                 if constexpr (MODE == MODE_ASHAPE) {
                     k0 = k0 & ((tkc > wlo) | (tkc < slim));
                     k1 = k1 & (((tkc + 32) > wlo) | ((tkc + 32) < slim));
+                } else if constexpr (MODE == MODE_VS || MODE == MODE_BS) {
+                    k0 = k0 & (tkc > wlo);
+                    k1 = k1 & ((tkc + 32) > wlo);
                 }
                 s0[r] = k0 ? s0[r] : -INFINITY;
                 s1[r] = k1 ? s1[r] : -INFINITY;
@@ -695,6 +709,7 @@ int check_tensors(const minf_qkvo *t) {
     const bool empty = t->batch == 0 || t->n == 0;
     if (!empty && (!t->q || !t->k || !t->v || !t->o)) return MINF_ERR_INVALID_ARG;
     if (t->heads_q % t->heads_kv != 0) return MINF_ERR_INVALID_ARG;
+    if (t->head_slot && t->index_heads <= 0) return MINF_ERR_INVALID_ARG;
     if (t->head_dim != HD) return MINF_ERR_UNSUPPORTED;
     if (t->dtype != MINF_BF16 && t->dtype != MINF_F16) return MINF_ERR_UNSUPPORTED;
     const void *ptrs[4] = {t->q, t->k, t->v, t->o};
@@ -705,6 +720,9 @@ int check_tensors(const minf_qkvo *t) {
             if (strides[i][j] < 0 || (strides[i][j] & 7)) return MINF_ERR_ALIGNMENT;
         // 64 rows x token stride is formed in 32 bits inside the tile copies
         if (strides[i][2] > (1 << 23)) return MINF_ERR_UNSUPPORTED;
+        // rows must not overlap (expanded or interleaved views): the tile copies describe 64 rows of
+        // a tile by one buffer descriptor of 64 x token stride bytes
+        if (t->n > 1 && strides[i][2] < HD) return MINF_ERR_UNSUPPORTED;
     }
     return MINF_OK;
 }
@@ -724,6 +742,8 @@ void fill_params(AttnParams &p, const minf_qkvo *t) {
     p.n_init = p.n_local = 0; p.dense_from = 0x7fffffff;
     p.total_wg = (long long)t->batch * t->heads_q * p.rows;
     p.descending = 0;
+    p.head_slot = t->head_slot;
+    p.index_heads = t->head_slot ? t->index_heads : t->heads_q;
 }
 
 template <int MODE> int launch(AttnParams p, int dtype, void *stream) {

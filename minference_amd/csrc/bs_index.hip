@@ -38,6 +38,10 @@ struct PoolParams {
     float *out;               // [batch*heads, rows, 128] fp32
     int heads, n, rows;
     int blk;                  // tokens per block: 64 or 32
+    // optional head selection: head_slot[h] < 0 skips head h, otherwise it is the head's position in
+    // `out`, which then has out_heads heads (= heads without it)
+    const int *head_slot;
+    int out_heads;
 };
 
 template <typename T> __device__ __forceinline__ float to_f32(unsigned short bits);
@@ -55,6 +59,11 @@ template <typename T> __global__ __launch_bounds__(256) void bs_pool_kernel(cons
     const int blk = blockIdx.x;
     const int bh = blockIdx.y;
     const int b = bh / p.heads, h = bh % p.heads;
+    int slot = h;
+    if (p.head_slot) {
+        slot = p.head_slot[h];
+        if (slot < 0) return;
+    }
     const int tid = (int)threadIdx.x;
     const int c = tid & 15, r4 = tid >> 4;
     const char *base = p.x + ((long long)b * p.xs[0] + (long long)h * p.xs[1]) * 2;
@@ -80,7 +89,7 @@ template <typename T> __global__ __launch_bounds__(256) void bs_pool_kernel(cons
         float s = 0.f;
 #pragma unroll
         for (int r = 0; r < 16; ++r) s += red[r][tid];
-        p.out[((long long)bh * p.rows + blk) * HD + tid] = s / (float)p.blk;
+        p.out[(((long long)b * p.out_heads + slot) * p.rows + blk) * HD + tid] = s / (float)p.blk;
     }
 }
 
@@ -90,6 +99,8 @@ struct ScoreParams {
     int heads_q, heads_kv, rows, pitch, force;
     int mtiles, ntiles;
     int skip_masked;
+    const int *head_slot;     // as in PoolParams; qp and scores have index_heads heads
+    int index_heads;
 };
 
 // lane l supplies row l%32 and, for MFMA step (s, j), contraction index 8*s + 4*(l/32) + j:
@@ -107,9 +118,15 @@ __global__ __launch_bounds__(256) void bs_scores_kernel(const ScoreParams p) {
     const int bh = blockIdx.y;
     const int b = bh / p.heads_q, h = bh % p.heads_q;
     const int hkv = h / (p.heads_q / p.heads_kv);
-    const float *qbase = p.qp + (long long)bh * p.rows * HD;
+    int slot = h;
+    if (p.head_slot) {
+        slot = p.head_slot[h];
+        if (slot < 0) return;
+    }
+    const long long bs = (long long)b * p.index_heads + slot;
+    const float *qbase = p.qp + bs * p.rows * HD;
     const float *kbase = p.kp + ((long long)b * p.heads_kv + hkv) * p.rows * HD;
-    float *out = p.scores + (long long)bh * p.rows * p.pitch;
+    float *out = p.scores + bs * p.rows * p.pitch;
     const int m0 = mt * 32;
 
     f32x4_t aq[16], bk[16];
@@ -162,8 +179,10 @@ namespace {
 int block_index_impl(const void *q, const void *k, const int64_t *q_stride, const int64_t *k_stride, int batch,
                      int heads_q, int heads_kv, int n, int head_dim, int dtype, int blk, int rows, int top_k,
                      int force_diag_first, int32_t *block_index, void *workspace, size_t workspace_bytes,
-                     void *stream) {
+                     void *stream, const int32_t *head_slot = nullptr, int index_heads = 0) {
     if (!q || !k || !q_stride || !k_stride || !block_index) return MINF_ERR_INVALID_ARG;
+    if (head_slot && index_heads <= 0) return MINF_ERR_INVALID_ARG;
+    if (!head_slot) index_heads = heads_q;
     if (batch < 0 || heads_q <= 0 || heads_kv <= 0 || n <= 0 || top_k <= 0) return MINF_ERR_INVALID_ARG;
     if (heads_q % heads_kv != 0) return MINF_ERR_INVALID_ARG;
     if (head_dim != HD) return MINF_ERR_UNSUPPORTED;
@@ -172,21 +191,21 @@ int block_index_impl(const void *q, const void *k, const int64_t *q_stride, cons
     for (int i = 0; i < 3; ++i)
         if ((q_stride[i] | k_stride[i]) & 7) return MINF_ERR_ALIGNMENT;
     if (batch == 0) return MINF_OK;
-    const size_t need = workspace_for(batch, heads_q, heads_kv, rows);
+    const size_t need = workspace_for(batch, index_heads, heads_kv, rows);
     if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 15)) return MINF_ERR_WORKSPACE;
     const int pitch = score_pitch(rows);
-    if ((long long)batch * heads_q * rows > 0x7fffffffLL || (long long)batch * heads_q > 65535) return MINF_ERR_UNSUPPORTED;
+    if ((long long)batch * index_heads * rows > 0x7fffffffLL || (long long)batch * heads_q > 65535) return MINF_ERR_UNSUPPORTED;
 
     char *ws = (char *)workspace;
     float *qp = (float *)ws;
-    ws += align256((size_t)batch * heads_q * rows * HD * 4);
+    ws += align256((size_t)batch * index_heads * rows * HD * 4);
     float *kp = (float *)ws;
     ws += align256((size_t)batch * heads_kv * rows * HD * 4);
     float *scores = (float *)ws;
     hipStream_t st = (hipStream_t)stream;
 
-    PoolParams pq{(const char *)q, {q_stride[0], q_stride[1], q_stride[2]}, qp, heads_q, n, rows, blk};
-    PoolParams pk{(const char *)k, {k_stride[0], k_stride[1], k_stride[2]}, kp, heads_kv, n, rows, blk};
+    PoolParams pq{(const char *)q, {q_stride[0], q_stride[1], q_stride[2]}, qp, heads_q, n, rows, blk, head_slot, index_heads};
+    PoolParams pk{(const char *)k, {k_stride[0], k_stride[1], k_stride[2]}, kp, heads_kv, n, rows, blk, nullptr, heads_kv};
     if (dtype == MINF_BF16) {
         hipLaunchKernelGGL(bs_pool_kernel<__bf16>, dim3(rows, batch * heads_q), dim3(256), 0, st, pq);
         hipLaunchKernelGGL(bs_pool_kernel<__bf16>, dim3(rows, batch * heads_kv), dim3(256), 0, st, pk);
@@ -199,15 +218,15 @@ int block_index_impl(const void *q, const void *k, const int64_t *q_stride, cons
 
     const bool causal_topk = rows <= 64 * 64;      // one wave per row: reads only the stored prefix of a row
     ScoreParams sp{qp, kp, scores, heads_q, heads_kv, rows, pitch, force_diag_first ? 1 : 0,
-                   (rows + 31) / 32, (pitch + 31) / 32, causal_topk ? 1 : 0};
+                   (rows + 31) / 32, (pitch + 31) / 32, causal_topk ? 1 : 0, head_slot, index_heads};
     hipLaunchKernelGGL(bs_scores_kernel, dim3(sp.mtiles, batch * heads_q), dim3(256), 0, st, sp);
     status = minf_launch_status();
     if (status != MINF_OK) return status;
 
     const int kk = top_k < rows ? top_k : rows;
     if (causal_topk)
-        return minf_topk_indices_block_causal(scores, batch * heads_q * rows, rows, pitch, kk, block_index, kk, rows, stream);
-    return minf_topk_indices(scores, batch * heads_q * rows, rows, pitch, kk, block_index, kk, -1, stream);
+        return minf_topk_indices_block_causal(scores, batch * index_heads * rows, rows, pitch, kk, block_index, kk, rows, stream);
+    return minf_topk_indices(scores, batch * index_heads * rows, rows, pitch, kk, block_index, kk, -1, stream);
 }
 
 }  // namespace
@@ -227,6 +246,17 @@ extern "C" int minf_bs_block_index(const void *q, const void *k, const int64_t *
                             workspace_bytes, stream);
 }
 
+extern "C" int minf_bs_block_index_heads(const void *q, const void *k, const int64_t *q_stride,
+                                         const int64_t *k_stride, int batch, int heads_q, int heads_kv,
+                                         int n, int head_dim, int dtype, int top_k, int force_diag_first,
+                                         const int32_t *head_slot, int index_heads,
+                                         int32_t *block_index, void *workspace, size_t workspace_bytes,
+                                         void *stream) {
+    if (!head_slot) return MINF_ERR_INVALID_ARG;
+    return block_index_impl(q, k, q_stride, k_stride, batch, heads_q, heads_kv, n, head_dim, dtype, BLK,
+                            n > 0 ? padded_rows(n) : 0, top_k, force_diag_first, block_index, workspace,
+                            workspace_bytes, stream, head_slot, index_heads);
+}
 extern "C" size_t minf_search_block_index_workspace_bytes(int batch, int heads_q, int heads_kv, int n) {
     if (batch <= 0 || heads_q <= 0 || heads_kv <= 0 || n <= 0) return 0;
     return workspace_for(batch, heads_q, heads_kv, (n + 31) / 32);

@@ -1,7 +1,9 @@
 // Version and status text of libminf_hip.so.
 #include "minf_common.h"
 
-extern "C" int minf_version(void) { return 100; }   // 0.1.0
+extern "C" int minf_version(void) { return 200; }   // 0.2.0
+
+extern "C" size_t minf_qkvo_size(void) { return sizeof(minf_qkvo); }
 
 extern "C" const char *minf_status_string(int status) {
     switch (status) {

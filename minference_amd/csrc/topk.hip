@@ -36,6 +36,11 @@ struct TopkProblem {
     // block-causal score rows (wave kernel only): row r belongs to query block m = r % causal_rows and
     // only its first 32 * (m / 32 + 1) entries are stored; the rest counts as -inf.  0 = plain rows
     int causal_rows;
+    // ragged selection: row i keeps k_rows[i] entries (clamped to 1..k) and the rest of its k output
+    // slots is padding -- pad_mode 1: the constant pad_value, 2: the last selected value repeated.
+    // k_rows == nullptr: every row keeps k entries.
+    const int *k_rows;
+    int pad_mode, pad_value;
 };
 
 // blockIdx.y selects one of two problems over rows of the same length n (vertical and slash
@@ -44,7 +49,8 @@ __global__ __launch_bounds__(TK_THREADS) void topk_kernel(const TopkProblem p0, 
     const TopkProblem &pr = blockIdx.y == 0 ? p0 : p1;
     const float *__restrict__ scores = pr.scores;
     const long long row_stride = pr.row_stride;
-    const int k = pr.k;
+    const int kmax = pr.k;
+    const int k = pr.k_rows ? max(1, min(pr.k_rows[blockIdx.x], kmax)) : kmax;
     int32_t *__restrict__ out = pr.out;
     const long long out_stride = pr.out_stride;
     const int reverse_base = pr.reverse_base;
@@ -54,6 +60,7 @@ __global__ __launch_bounds__(TK_THREADS) void topk_kernel(const TopkProblem p0, 
     __shared__ unsigned hist[256 * 32];
     __shared__ unsigned bins[256];
     __shared__ unsigned sh_prefix, sh_need;
+    __shared__ int sh_last;
     __shared__ int wave_gt[TK_WAVES], wave_eq[TK_WAVES];
 
     const float *x = scores + (long long)blockIdx.x * row_stride;
@@ -169,7 +176,9 @@ __global__ __launch_bounds__(TK_THREADS) void topk_kernel(const TopkProblem p0, 
         for (int c = 0; c < 4; ++c) {
             if (gt[c] || (eq[c] && e_here < r)) {
                 const int i = i0 + c;
-                o[g_here + min(e_here, r)] = reverse_base >= 0 ? reverse_base - i : i;
+                const int pos = g_here + min(e_here, r), val = reverse_base >= 0 ? reverse_base - i : i;
+                o[pos] = val;
+                if (pos == k - 1) sh_last = val;
             }
             g_here += gt[c];
             e_here += eq[c];
@@ -187,11 +196,17 @@ __global__ __launch_bounds__(TK_THREADS) void topk_kernel(const TopkProblem p0, 
         const int e_here = eq_before + __builtin_popcountll(me & lt);
         const bool take = gt || (eq && e_here < r);
         if (take) {
-            const int pos = g_here + min(e_here, r);
-            o[pos] = reverse_base >= 0 ? reverse_base - i : i;
+            const int pos = g_here + min(e_here, r), val = reverse_base >= 0 ? reverse_base - i : i;
+            o[pos] = val;
+            if (pos == k - 1) sh_last = val;
         }
         gt_before += __builtin_popcountll(mg);
         eq_before += __builtin_popcountll(me);
+    }
+    if (k < kmax && pr.pad_mode) {                 // (workgroup-uniform)
+        __syncthreads();
+        const int pad = pr.pad_mode == 2 ? sh_last : pr.pad_value;
+        for (int i = k + tid; i < kmax; i += TK_THREADS) o[i] = pad;
     }
 }
 
@@ -213,7 +228,8 @@ __global__ __launch_bounds__(TKW_WAVES * 64, ITEMS >= 64 ? 3 : (ITEMS >= 40 ? 5 
     if (row >= rows) return;
     const float *__restrict__ x = pr.scores + (long long)row * pr.row_stride;
     int32_t *__restrict__ o = pr.out + (long long)row * pr.out_stride;
-    const int k = pr.k, reverse_base = pr.reverse_base;
+    const int kcap = pr.k, reverse_base = pr.reverse_base;
+    const int k = pr.k_rows ? max(1, min(pr.k_rows[row], kcap)) : kcap;
     if (k >= n) {
         for (int i = lane; i < n; i += 64) o[i] = reverse_base >= 0 ? reverse_base - i : i;
         return;
@@ -291,6 +307,8 @@ __global__ __launch_bounds__(TKW_WAVES * 64, ITEMS >= 64 ? 3 : (ITEMS >= 40 ? 5 
     }
     const int r = k - cgt;                           // entries equal to T that are taken, lowest index first
     int gt_before = 0, eq_before = 0;
+    int lastv = 0;
+    bool has_last = false;
     const uint64_t lt = minf_lanemask_lt();
 #pragma unroll
     for (int jb = 0; jb < ITEMS; jb += GROUP) {
@@ -303,12 +321,22 @@ __global__ __launch_bounds__(TKW_WAVES * 64, ITEMS >= 64 ? 3 : (ITEMS >= 40 ? 5 
                 const int e_here = eq_before + __builtin_popcountll(me & lt);
                 if (gt || (eq && e_here < r)) {
                     const int pos = gt_before + __builtin_popcountll(mg & lt) + min(e_here, r);
-                    o[pos] = reverse_base >= 0 ? reverse_base - i : i;
+                    const int val = reverse_base >= 0 ? reverse_base - i : i;
+                    o[pos] = val;
+                    if (pos == k - 1) { lastv = val; has_last = true; }
                 }
                 gt_before += __builtin_popcountll(mg);
                 eq_before += __builtin_popcountll(me);
             }
         }
+    }
+    if (k < kcap && pr.pad_mode) {                 // (wave-uniform)
+        int pad = pr.pad_value;
+        if (pr.pad_mode == 2) {
+            const uint64_t who = __ballot(has_last);
+            pad = who ? minf_readlane(lastv, __builtin_ctzll(who)) : 0;
+        }
+        for (int i = k + lane; i < kcap; i += 64) o[i] = pad;
     }
 }
 
@@ -333,7 +361,7 @@ extern "C" int minf_topk_indices(const float *scores, int rows, int n, int64_t r
     if (!scores || !out || rows < 0 || n <= 0 || k <= 0) return MINF_ERR_INVALID_ARG;
     if (row_stride < n || out_stride < (k < n ? k : n)) return MINF_ERR_INVALID_ARG;
     if (rows == 0) return MINF_OK;
-    TopkProblem p{scores, (long long)row_stride, k, out, (long long)out_stride, reverse_base, 0};
+    TopkProblem p{scores, (long long)row_stride, k, out, (long long)out_stride, reverse_base, 0, nullptr, 0, 0};
     launch_topk(p, p, 1, rows, n, (hipStream_t)stream);
     return minf_launch_status();
 }
@@ -344,7 +372,7 @@ extern "C" int minf_topk_indices_block_causal(const float *scores, int rows, int
     if (row_stride < n || out_stride < (k < n ? k : n)) return MINF_ERR_INVALID_ARG;
     if (n > 64 * 64) return MINF_ERR_UNSUPPORTED;      // only the one-wave-per-row kernel knows about stored prefixes
     if (rows == 0) return MINF_OK;
-    TopkProblem p{scores, (long long)row_stride, k, out, (long long)out_stride, -1, rows_per_head};
+    TopkProblem p{scores, (long long)row_stride, k, out, (long long)out_stride, -1, rows_per_head, nullptr, 0, 0};
     launch_topk(p, p, 1, rows, n, (hipStream_t)stream);
     return minf_launch_status();
 }
@@ -358,8 +386,26 @@ extern "C" int minf_topk_indices_pair(const float *scores_a, int k_a, int32_t *o
     if (row_stride < n || out_stride_a < (k_a < n ? k_a : n) || out_stride_b < (k_b < n ? k_b : n))
         return MINF_ERR_INVALID_ARG;
     if (rows == 0) return MINF_OK;
-    TopkProblem pa{scores_a, (long long)row_stride, k_a, out_a, (long long)out_stride_a, reverse_base_a, 0};
-    TopkProblem pb{scores_b, (long long)row_stride, k_b, out_b, (long long)out_stride_b, reverse_base_b, 0};
+    TopkProblem pa{scores_a, (long long)row_stride, k_a, out_a, (long long)out_stride_a, reverse_base_a, 0, nullptr, 0, 0};
+    TopkProblem pb{scores_b, (long long)row_stride, k_b, out_b, (long long)out_stride_b, reverse_base_b, 0, nullptr, 0, 0};
+    launch_topk(pa, pb, 2, rows, n, (hipStream_t)stream);
+    return minf_launch_status();
+}
+
+extern "C" int minf_topk_indices_pair_ragged(const float *scores_a, const int32_t *k_rows_a, int k_max_a, int32_t *out_a,
+                                             int64_t out_stride_a, int reverse_base_a, int pad_mode_a, int pad_value_a,
+                                             const float *scores_b, const int32_t *k_rows_b, int k_max_b, int32_t *out_b,
+                                             int64_t out_stride_b, int reverse_base_b, int pad_mode_b, int pad_value_b,
+                                             int rows, int n, int64_t row_stride, void *stream) {
+    if (!scores_a || !out_a || !scores_b || !out_b || !k_rows_a || !k_rows_b || rows < 0 || n <= 0 || k_max_a <= 0 || k_max_b <= 0)
+        return MINF_ERR_INVALID_ARG;
+    if (pad_mode_a < 0 || pad_mode_a > 2 || pad_mode_b < 0 || pad_mode_b > 2) return MINF_ERR_INVALID_ARG;
+    if (k_max_a > n) k_max_a = n;
+    if (k_max_b > n) k_max_b = n;
+    if (row_stride < n || out_stride_a < k_max_a || out_stride_b < k_max_b) return MINF_ERR_INVALID_ARG;
+    if (rows == 0) return MINF_OK;
+    TopkProblem pa{scores_a, (long long)row_stride, k_max_a, out_a, (long long)out_stride_a, reverse_base_a, 0, k_rows_a, pad_mode_a, pad_value_a};
+    TopkProblem pb{scores_b, (long long)row_stride, k_max_b, out_b, (long long)out_stride_b, reverse_base_b, 0, k_rows_b, pad_mode_b, pad_value_b};
     launch_topk(pa, pb, 2, rows, n, (hipStream_t)stream);
     return minf_launch_status();
 }

@@ -49,6 +49,10 @@ struct EstParams {
     float *vertical, *slash;    // [B, Hq, N]
     int force_v, force_s;
     long long total_wg;
+    // optional head selection: head_slot[h] < 0 skips query head h, otherwise it is the head's
+    // position in the outputs and the workspace, which have index_heads heads (= hq without it)
+    const int *head_slot;
+    int index_heads;
 };
 
 union Frag {
@@ -65,7 +69,7 @@ template <> __device__ __forceinline__ f32x16_t mma<_Float16>(const Frag &a, con
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a.h, b.h, c, 0, 0, 0);
 }
 
-struct WgId { int b, h, hkv, chunk; bool valid; };
+struct WgId { int b, h, hkv, chunk, slot; bool valid; };
 
 // XCD-aware order: (batch, kv head, chunk, query head in group) contiguous per XCD
 __device__ __forceinline__ WgId decode_wg(const EstParams &p) {
@@ -80,6 +84,11 @@ __device__ __forceinline__ WgId decode_wg(const EstParams &p) {
     w.hkv = (int)(rest % p.hk);
     w.b = (int)(rest / p.hk);
     w.h = w.hkv * group + hin;
+    w.slot = w.h;
+    if (w.valid && p.head_slot) {
+        w.slot = p.head_slot[w.h];
+        w.valid = w.slot >= 0;
+    }
     return w;
 }
 
@@ -187,7 +196,7 @@ __global__ __launch_bounds__(EST_THREADS, 3) void est_stats_kernel(const EstPara
             l = l * __builtin_amdgcn_exp2f(m - m_use) + lo * __builtin_amdgcn_exp2f(mo - m_use);
             m = m_new;
         }
-        float *dst = p.stats + ((((long long)w.b * p.hq + w.h) * p.nchunks + w.chunk) * LQ + tid) * 2;
+        float *dst = p.stats + ((((long long)w.b * p.index_heads + w.slot) * p.nchunks + w.chunk) * LQ + tid) * 2;
         dst[0] = m;
         dst[1] = l;
     }
@@ -232,7 +241,7 @@ __global__ __launch_bounds__(EST_THREADS, 2) void est_scores_kernel(const EstPar
     const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, g = lane >> 5;
     const char *kb = p.k + ((long long)w.b * p.ks[0] + (long long)w.hkv * p.ks[1]) * 2;
-    const long long bh = (long long)w.b * p.hq + w.h;
+    const long long bh = (long long)w.b * p.index_heads + w.slot;
     float *tile = lds_tile + wave * 63 * TP;
     float *wwin = lds_wwin[wave];
 
@@ -331,8 +340,11 @@ __global__ __launch_bounds__(256) void est_finalize_kernel(const EstParams p) {
 
 int fill(EstParams &p, const void *q, const void *k, const int64_t *q_stride, const int64_t *k_stride,
          int batch, int heads_q, int heads_kv, int n, int head_dim, int dtype, float sm_scale,
-         int last_q, int force_v, int force_s, float *vertical, float *slash, void *ws, size_t ws_bytes) {
+         int last_q, int force_v, int force_s, float *vertical, float *slash, void *ws, size_t ws_bytes,
+         const int32_t *head_slot, int index_heads) {
     if (!q || !k || !vertical || !slash || !ws) return MINF_ERR_INVALID_ARG;
+    if (head_slot && index_heads <= 0) return MINF_ERR_INVALID_ARG;
+    if (!head_slot) index_heads = heads_q;
     if (batch < 0 || heads_q <= 0 || heads_kv <= 0 || n <= 0 || heads_q % heads_kv) return MINF_ERR_INVALID_ARG;
     if (head_dim != HD || (dtype != MINF_BF16 && dtype != MINF_F16)) return MINF_ERR_UNSUPPORTED;
     if (last_q < 1 || last_q > LQ || force_v < 0 || force_s < 0) return MINF_ERR_INVALID_ARG;
@@ -345,7 +357,7 @@ int fill(EstParams &p, const void *q, const void *k, const int64_t *q_stride, co
     p.last_q = last_q < n ? last_q : n;
     p.scale_log2 = sm_scale * 1.4426950408889634f;
     p.nchunks = (n + KC - 1) / KC;
-    const long long bh = (long long)batch * heads_q;
+    const long long bh = (long long)batch * index_heads;
     const size_t stats_b = (size_t)bh * p.nchunks * LQ * 2 * sizeof(float);
     const size_t row_b = (size_t)bh * LQ * sizeof(float);
     const size_t win_b = (size_t)bh * p.nchunks * WIN * sizeof(float);
@@ -356,7 +368,9 @@ int fill(EstParams &p, const void *q, const void *k, const int64_t *q_stride, co
     p.win = (float *)((char *)ws + stats_b + row_b);
     p.vertical = vertical; p.slash = slash;
     p.force_v = force_v; p.force_s = force_s;
-    p.total_wg = bh * p.nchunks;
+    p.total_wg = (long long)batch * heads_q * p.nchunks;
+    p.head_slot = head_slot;
+    p.index_heads = index_heads;
     return MINF_OK;
 }
 
@@ -369,20 +383,21 @@ extern "C" size_t minf_vs_estimate_workspace_bytes(int batch, int heads_q, int n
     return bh * nchunks * LQ * 2 * sizeof(float) + bh * LQ * sizeof(float) + bh * nchunks * WIN * sizeof(float);
 }
 
-extern "C" int minf_vs_estimate(const void *q, const void *k, const int64_t *q_stride,
-                                const int64_t *k_stride, int batch, int heads_q, int heads_kv, int n,
-                                int head_dim, int dtype, float sm_scale, int last_q, int force_vertical,
-                                int force_slash, float *vertical, float *slash, void *workspace,
-                                size_t workspace_bytes, void *stream) {
+static int estimate_launch(const void *q, const void *k, const int64_t *q_stride, const int64_t *k_stride,
+                           int batch, int heads_q, int heads_kv, int n, int head_dim, int dtype, float sm_scale,
+                           int last_q, int force_vertical, int force_slash, float *vertical, float *slash,
+                           void *workspace, size_t workspace_bytes, const int32_t *head_slot, int index_heads,
+                           void *stream) {
     EstParams p;
     if (batch == 0) return MINF_OK;
     int st = fill(p, q, k, q_stride, k_stride, batch, heads_q, heads_kv, n, head_dim, dtype, sm_scale,
-                  last_q, force_vertical, force_slash, vertical, slash, workspace, workspace_bytes);
+                  last_q, force_vertical, force_slash, vertical, slash, workspace, workspace_bytes,
+                  head_slot, index_heads);
     if (st) return st;
     const long long grid = ((p.total_wg + 7) >> 3) * 8;
     if (grid > 0x7fffffffLL) return MINF_ERR_UNSUPPORTED;
     hipStream_t s = (hipStream_t)stream;
-    const long long bh = (long long)batch * heads_q;
+    const long long bh = (long long)batch * p.index_heads;       // heads of the outputs
     if (dtype == MINF_BF16) hipLaunchKernelGGL(est_stats_kernel<__bf16>, dim3((unsigned)grid), dim3(EST_THREADS), 0, s, p);
     else hipLaunchKernelGGL(est_stats_kernel<_Float16>, dim3((unsigned)grid), dim3(EST_THREADS), 0, s, p);
     hipLaunchKernelGGL(est_reduce_kernel, dim3((unsigned)bh), dim3(LQ), 0, s, p);
@@ -390,4 +405,25 @@ extern "C" int minf_vs_estimate(const void *q, const void *k, const int64_t *q_s
     else hipLaunchKernelGGL(est_scores_kernel<_Float16>, dim3((unsigned)grid), dim3(EST_THREADS), 0, s, p);
     hipLaunchKernelGGL(est_finalize_kernel, dim3((unsigned)((n + 255) / 256), (unsigned)bh), dim3(256), 0, s, p);
     return minf_launch_status();
+}
+
+extern "C" int minf_vs_estimate(const void *q, const void *k, const int64_t *q_stride,
+                                const int64_t *k_stride, int batch, int heads_q, int heads_kv, int n,
+                                int head_dim, int dtype, float sm_scale, int last_q, int force_vertical,
+                                int force_slash, float *vertical, float *slash, void *workspace,
+                                size_t workspace_bytes, void *stream) {
+    return estimate_launch(q, k, q_stride, k_stride, batch, heads_q, heads_kv, n, head_dim, dtype, sm_scale, last_q,
+                           force_vertical, force_slash, vertical, slash, workspace, workspace_bytes, nullptr, 0, stream);
+}
+
+extern "C" int minf_vs_estimate_heads(const void *q, const void *k, const int64_t *q_stride,
+                                      const int64_t *k_stride, int batch, int heads_q, int heads_kv, int n,
+                                      int head_dim, int dtype, float sm_scale, int last_q, int force_vertical,
+                                      int force_slash, const int32_t *head_slot, int index_heads,
+                                      float *vertical, float *slash, void *workspace,
+                                      size_t workspace_bytes, void *stream) {
+    if (!head_slot) return MINF_ERR_INVALID_ARG;
+    return estimate_launch(q, k, q_stride, k_stride, batch, heads_q, heads_kv, n, head_dim, dtype, sm_scale, last_q,
+                           force_vertical, force_slash, vertical, slash, workspace, workspace_bytes, head_slot,
+                           index_heads, stream);
 }

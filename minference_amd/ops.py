@@ -106,6 +106,15 @@ class _Call:
     def ref(self):
         return ctypes.byref(self.struct)
 
+    def select_heads(self, head_slot=None, index_heads=0):
+        """Restrict the following launches to the query heads h with head_slot[h] >= 0 (int32
+        [heads_q] on the device; that value is the head's position in index tensors that have
+        index_heads heads).  None = all heads again.  The output buffer is shared, so one launch
+        per pattern type fills its heads in place."""
+        self._head_slot = head_slot                       # keeps the tensor alive
+        self.struct.head_slot = head_slot.data_ptr() if head_slot is not None else None
+        self.struct.index_heads = int(index_heads) if head_slot is not None else 0
+
     def result(self):
         o = self.o
         if self.head_dim != _SUPPORTED_D:

@@ -6,9 +6,9 @@ Counterpart of ``minference_prefill_kernel`` / ``minference_prefill_forward``
 ``best_pattern`` (list over layers of ``{"<head>": [type, vertical_size,
 slash_size, score]}``), ``starting_layer``, ``minference_ratio`` and the search mode
 (``is_search``, ``config_path``, with ``num_hidden_layers`` in ``prefill_kwargs``).  Heads are
-grouped by (pattern, sizes) and every group is one batched launch sequence
-instead of the reference's Python loop over heads.  K/V may have fewer heads
-than Q (no repeat_kv needed).
+grouped by pattern TYPE and every type is one batched launch chain over the original tensors
+(per-head sizes are ragged inside the chain; nothing is gathered or scattered) instead of the
+reference's Python loop over heads.  K/V may have fewer heads than Q (no repeat_kv needed).
 """
 from __future__ import annotations
 
@@ -55,17 +55,116 @@ def _head_plan(config, layer_idx, num_heads):
     return plan
 
 
-def _kv_for_heads(k, heads, group):
-    """K/V heads feeding the query heads ``heads`` -> (tensor, heads_kv) so that the query
-    subset [len(heads)] maps onto it with the usual h // (Hq/Hk) rule."""
-    if group == 1:
-        return k[:, heads]
-    kv = sorted({h // group for h in heads})
-    full = all(h // group in kv for h in heads) and len(heads) == len(kv) * group and \
-        heads == [g * group + i for g in kv for i in range(group)]
-    if full:
-        return k[:, kv]
-    return k[:, [h // group for h in heads]]          # one kv head per query head
+VERTICAL_PAD = 0x3FFFFFFF      # a vertical index no range ever reaches: never emitted by the index builder
+
+
+def _slot_tensor(heads, num_heads, device):
+    """int32 [num_heads]: position of head h in ``heads`` or -1."""
+    slot = torch.full((num_heads,), -1, dtype=torch.int32)
+    slot[torch.as_tensor(heads, dtype=torch.long)] = torch.arange(len(heads), dtype=torch.int32)
+    return slot.to(device)
+
+
+def _mixed_layer(query_states, key_states, value_states, plan):
+    """All heads of a layer whose pattern table mixes types and sizes: q/k/v are prepared once, the
+    output is one shared buffer, and every pattern type is ONE launch chain over the original
+    tensors with a head selection -- no gathered copies of Q, no scattered writes of O:
+
+    * vertical_and_slash heads with any mix of (vertical_size, slash_size): one estimation over those
+      heads, one ragged top-k (every head keeps its own sizes; shorter lists are padded with entries
+      that are no-ops of the index builder's merge), one index build, one attention launch;
+    * block_sparse heads: one block index + one attention launch;
+    * stream_llm heads: one launch per distinct (n_init, n_local).
+
+    The reference runs one operator call per head here (minference_forward.py:657-667)."""
+    from . import _lib
+    from .estimate import FORCE_SLASH, FORCE_VERTICAL, LAST_Q
+    from .ops import _Call, _SUPPORTED_D
+    import ctypes
+    B, H, N, D = query_states.shape
+    dev = query_states.device
+    c = _Call(query_states, key_states, value_states)
+    lib = _lib.load()
+    stream = _lib.stream_ptr(dev)
+    i64x3 = _lib.c_i64 * 3
+    qs, ks = i64x3(*c.q.stride()[:3]), i64x3(*c.k.stride()[:3])
+    rows = (N + 63) // 64
+    keep = []                                             # tensors the enqueued kernels still read
+
+    vs = [(h, v, s) for (ty, v, s), hs in plan.items() if ty == "vertical_and_slash" for h in hs]
+    bs = sorted(h for (ty, _, _), hs in plan.items() if ty == "block_sparse" for h in hs)
+    st_groups = {}
+    for (ty, v, s), hs in plan.items():
+        if ty == "stream_llm":
+            st_groups.setdefault((v, s), []).extend(hs)
+        elif ty not in ("vertical_and_slash", "block_sparse"):
+            raise KeyError(ty)
+
+    with torch.cuda.device(dev):
+        if vs:
+            vs.sort()
+            heads = [h for h, _, _ in vs]
+            nh = len(heads)
+            # sizes clamped like the reference (:600)
+            kv = [min(N, max(int(v), 30)) for _, v, _ in vs]
+            ksl = [min(N, max(int(s), 50)) for _, _, s in vs]
+            vmax, smax = max(kv), max(ksl)
+            slot = _slot_tensor(heads, H, dev)
+            vertical = torch.empty((B, nh, N), dtype=torch.float32, device=dev)
+            slash = torch.empty((B, nh, N), dtype=torch.float32, device=dev)
+            ws_bytes = lib.minf_vs_estimate_workspace_bytes(B, nh, N)
+            ws = torch.empty((ws_bytes + 15) // 16 * 16, dtype=torch.uint8, device=dev)
+            st = lib.minf_vs_estimate_heads(c.q.data_ptr(), c.k.data_ptr(), qs, ks, B, H, c.Hk, N, _SUPPORTED_D,
+                                            c.struct.dtype, float(D) ** -0.5, LAST_Q, FORCE_VERTICAL, FORCE_SLASH,
+                                            slot.data_ptr(), nh, vertical.data_ptr(), slash.data_ptr(),
+                                            ws.data_ptr(), ws_bytes, stream)
+            _lib.check(st, "minf_vs_estimate_heads")
+            kv_t = torch.tensor(kv * B, dtype=torch.int32).to(dev)
+            ks_t = torch.tensor(ksl * B, dtype=torch.int32).to(dev)
+            v_idx = torch.empty((B, nh, vmax), dtype=torch.int32, device=dev)
+            s_idx = torch.empty((B, nh, smax), dtype=torch.int32, device=dev)
+            st = lib.minf_topk_indices_pair_ragged(vertical.data_ptr(), kv_t.data_ptr(), vmax, v_idx.data_ptr(), vmax, -1, 1, VERTICAL_PAD,
+                                                   slash.data_ptr(), ks_t.data_ptr(), smax, s_idx.data_ptr(), smax, N - 1, 2, 0,
+                                                   B * nh, N, N, stream)
+            _lib.check(st, "minf_topk_indices_pair_ragged")
+            seqlens = torch.full((B,), N, dtype=torch.int32, device=dev)
+            bc, bo, cc, ci = convert_vertical_slash_indexes(seqlens, v_idx, s_idx, N, 64, 64, zero_fill=False)
+            c.struct.seqlens = seqlens.data_ptr()
+            c.select_heads(slot, nh)
+            st = lib.minf_vs_attn_fwd(c.ref, bc.data_ptr(), bo.data_ptr(), cc.data_ptr(), ci.data_ptr(), rows,
+                                      smax, vmax, stream)
+            _lib.check(st, "minf_vs_attn_fwd")
+            c.struct.seqlens = None
+            keep += [slot, vertical, slash, ws, kv_t, ks_t, v_idx, s_idx, seqlens, bc, bo, cc, ci]
+        if bs:
+            nh = len(bs)
+            slot = _slot_tensor(bs, H, dev)
+            brows = lib.minf_bs_block_index_rows(N)
+            kk = min(100, brows)                          # top_k fixed at 100 (:616-618)
+            ws_bytes = lib.minf_bs_block_index_workspace_bytes(B, nh, c.Hk, N)
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+            bi = torch.empty((B, nh, brows, kk), dtype=torch.int32, device=dev)
+            st = lib.minf_bs_block_index_heads(c.q.data_ptr(), c.k.data_ptr(), qs, ks, B, H, c.Hk, N, _SUPPORTED_D,
+                                               c.struct.dtype, 100, 0, slot.data_ptr(), nh, bi.data_ptr(),
+                                               ws.data_ptr(), ws_bytes, stream)
+            _lib.check(st, "minf_bs_block_index_heads")
+            c.select_heads(slot, nh)
+            st = lib.minf_bs_attn_fwd(c.ref, bi.data_ptr(), brows, kk, stream)
+            _lib.check(st, "minf_bs_attn_fwd")
+            keep += [slot, ws, bi]
+        for (n_init, n_local), hs in st_groups.items():
+            slot = _slot_tensor(sorted(hs), H, dev)
+            c.select_heads(slot, len(hs))
+            if N > 0:
+                st = lib.minf_ashape_attn_fwd(c.ref, int(n_init), int(n_local), stream)
+                _lib.check(st, "minf_ashape_attn_fwd")
+            keep.append(slot)
+    c.select_heads(None)
+    out = c.result()
+    # torch's caching allocator hands a freed block only to work enqueued later on the same stream, so
+    # dropping `keep` here is safe for kernels that are still running
+    del keep
+    return out
 
 
 def minference_prefill_kernel(q, k, v, pattern, vertical_size, slash_size):
@@ -120,13 +219,7 @@ def minference_prefill_forward(query_states, key_states, value_states, prefill_k
     if len(plan) == 1:
         (ty, vs, ss), _ = next(iter(plan.items()))
         return minference_prefill_kernel(query_states, key_states, value_states, ty, vs, ss)
-    output = torch.empty_like(query_states)
-    for (ty, vs, ss), heads in plan.items():
-        qh = query_states[:, heads]
-        kh = _kv_for_heads(key_states, heads, group)
-        vh = _kv_for_heads(value_states, heads, group)
-        output[:, heads] = minference_prefill_kernel(qh, kh, vh, ty, vs, ss)
-    return output
+    return _mixed_layer(query_states, key_states, value_states, plan)
 
 
 def a_shape_kernel(query_states, key_states, value_states, prefill_kwargs):

@@ -100,6 +100,11 @@ int main() {
     for (auto &x : k) x = to_bf16(lcg_normalish());
     for (auto &x : v) x = to_bf16(lcg_normalish());
     printf("libminf_hip version %d\n", minf_version());
+    if (minf_qkvo_size() != sizeof(minf_qkvo)) {
+        fprintf(stderr, "this program and libminf_hip.so were built from different revisions of include/minf_hip.h "
+                        "(minf_qkvo: %zu bytes here, %zu in the library): rebuild both\n", sizeof(minf_qkvo), minf_qkvo_size());
+        return 3;
+    }
 
     void *dq, *dk, *dv, *dout;
     CHECK_HIP(hipMalloc(&dq, qn * 2));

@@ -16,6 +16,11 @@ EXE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cabi", "c_caller
 def test_c_program_calls_the_library_directly(gpu):
     if not os.path.exists(EXE):
         pytest.fail("tests/cabi/c_caller has not been built (run __graft_entry__.build())")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    for dep in (os.path.join(root, "include", "minf_hip.h"), os.path.join(root, "tests", "cabi", "c_caller.cpp")):
+        # a program compiled against an older header would hand the library a struct of the wrong size
+        if os.path.getmtime(dep) > os.path.getmtime(EXE):
+            pytest.fail(f"tests/cabi/c_caller is older than {os.path.relpath(dep, root)}: run __graft_entry__.build()")
     r = subprocess.run([EXE], capture_output=True, text=True, timeout=120)
     print(r.stdout)
     print(r.stderr)

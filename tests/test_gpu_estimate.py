@@ -74,3 +74,37 @@ def test_estimate_sets_vs_oracle(gpu):
         assert len(a & b) >= 0.99 * 200 and len(c & d) >= 0.99 * 600
         assert set(range(30)) <= a and set(range(100)) <= c
         assert (np.diff(v_idx[0, h].numpy()) > 0).all() and (np.diff(s_idx[0, h].numpy()) < 0).all()
+
+
+@pytest.mark.parametrize("n", [3000, 20000])
+def test_ragged_topk_pads_with_noop_entries(gpu, n):
+    """minf_topk_indices_pair_ragged: every row keeps its own k; the first k entries equal the plain
+    selection with that k, the rest of the row is the padding (a constant for the first problem, the
+    last selected value repeated for the second).  n = 3000 runs the one-wave-per-row kernel,
+    n = 20000 the wide one."""
+    from minference_amd import _lib
+    from minference_amd.estimate import topk_indices
+    lib = _lib.load()
+    rows = 5
+    g = torch.Generator().manual_seed(n)
+    a = torch.randn(rows, n, generator=g).to(gpu)
+    b = torch.randn(rows, n, generator=g).to(gpu)
+    ka = [30, 1000, 1, 577, 1000]
+    kb = [2048, 50, 2048, 1, 999]
+    kam, kbm = max(ka), max(kb)
+    out_a = torch.full((rows, kam), -5, dtype=torch.int32, device=gpu)
+    out_b = torch.full((rows, kbm), -5, dtype=torch.int32, device=gpu)
+    ka_t = torch.tensor(ka, dtype=torch.int32, device=gpu)
+    kb_t = torch.tensor(kb, dtype=torch.int32, device=gpu)
+    st = lib.minf_topk_indices_pair_ragged(a.data_ptr(), ka_t.data_ptr(), kam, out_a.data_ptr(), kam, -1, 1, 0x3FFFFFFF,
+                                           b.data_ptr(), kb_t.data_ptr(), kbm, out_b.data_ptr(), kbm, n - 1, 2, 0,
+                                           rows, n, n, _lib.stream_ptr(gpu))
+    torch.cuda.synchronize()
+    assert st == 0
+    for r in range(rows):
+        want_a = topk_indices(a[r:r + 1].contiguous(), ka[r])[0]
+        assert torch.equal(out_a[r, :ka[r]], want_a)
+        assert (out_a[r, ka[r]:] == 0x3FFFFFFF).all()
+        want_b = topk_indices(b[r:r + 1].contiguous(), kb[r], reverse_base=n - 1)[0]
+        assert torch.equal(out_b[r, :kb[r]], want_b)
+        assert (out_b[r, kb[r]:] == want_b[-1]).all()

@@ -36,6 +36,111 @@ def test_mixed_patterns_route_to_the_right_kernels(gpu):
     assert (out[:, 3:5] - ref_def).abs().max() <= 2e-2
 
 
+def _ragged_table(hq):
+    """Per-head patterns in the shape of the shipped Llama-3-8B table: vertical_and_slash heads with
+    five distinct (vertical, slash) sizes, block_sparse heads, stream_llm heads with two settings."""
+    sizes = [(1000, 6096), (500, 3000), (30, 800), (100, 750), (3500, 100)]
+    layer = {}
+    for h in range(hq):
+        if h % 8 == 3:
+            layer[str(h)] = ["block_sparse", 100, 0, 1.0]
+        elif h % 8 == 6:
+            layer[str(h)] = ["stream_llm", 100, 800, 1.0] if h < hq // 2 else ["stream_llm", 64, 1500, 1.0]
+        else:
+            v, s = sizes[(h * 7) % 5]
+            layer[str(h)] = ["vertical_and_slash", v, s, 1.0]
+    return layer
+
+
+def test_ragged_per_head_sizes_one_launch_chain_per_type(gpu, monkeypatch):
+    """A 32-head layer (8 kv heads) whose table mixes five (vertical, slash) sizes, block_sparse and
+    two stream_llm settings: the dispatcher must issue ONE estimation, ONE top-k, ONE index build and
+    ONE attention launch for all vertical_and_slash heads (ragged sizes), one block index + one
+    attention launch for the block_sparse heads, one launch per stream_llm setting -- and the result
+    must be bit-identical to running every head on its own through the public operators (what the
+    reference's per-head loop does, minference_forward.py:657-667)."""
+    import minference_amd as M
+    from minference_amd import _lib
+    n, hq, hk = 8192 + 40, 32, 8
+    q, k, v, _ = gen.planted_layer(n, hq, hk, seed=7, dtype=torch.bfloat16)
+    qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
+    layer = _ragged_table(hq)
+    kwargs = {"layer_idx": 0, "attn_forward_config": {"best_pattern": [layer]}}
+    lib = _lib.load()
+    counts = {}
+    for name in ("minf_vs_estimate_heads", "minf_topk_indices_pair_ragged", "minf_vs_index_build_ws", "minf_vs_attn_fwd",
+                 "minf_bs_block_index_heads", "minf_bs_attn_fwd", "minf_ashape_attn_fwd", "minf_vs_estimate"):
+        real = getattr(lib, name)
+
+        def counting(*a, _real=real, _name=name):
+            counts[_name] = counts.get(_name, 0) + 1
+            return _real(*a)
+        monkeypatch.setattr(lib, name, counting)
+    print("case ragged dispatcher, one chain per type", flush=True)
+    out = M.minference_prefill_forward(qg, kg, vg, kwargs)
+    torch.cuda.synchronize()
+    assert counts == {"minf_vs_estimate_heads": 1, "minf_topk_indices_pair_ragged": 1, "minf_vs_index_build_ws": 1,
+                      "minf_vs_attn_fwd": 1, "minf_bs_block_index_heads": 1, "minf_bs_attn_fwd": 1,
+                      "minf_ashape_attn_fwd": 2}, counts
+    monkeypatch.undo()
+    assert out.shape == q.shape and out.dtype == torch.bfloat16 and torch.isfinite(out.float()).all()
+    group = hq // hk
+    for h in range(hq):
+        ty, a, b, _ = layer[str(h)]
+        qh, kh, vh = qg[:, h:h + 1], kg[:, h // group:h // group + 1], vg[:, h // group:h // group + 1]
+        if ty == "vertical_and_slash":
+            ref = M.vertical_slash_prefill(qh, kh, vh, a, b)
+        elif ty == "block_sparse":
+            ref = M.block_sparse_attention(qh, kh, vh, 100)
+        else:
+            ref = M.streaming_forward(qh, kh, vh, a, b)
+        assert torch.equal(out[:, h:h + 1], ref), f"head {h} ({ty} {a} {b}) differs from its own per-head run"
+    # and against the oracle for one head of each kind (same indices as the GPU produced)
+    for h in (0, 3, 6):
+        ty, a, b, _ = layer[str(h)]
+        kv = h // group
+        if ty == "vertical_and_slash":
+            v_idx, s_idx = M.estimate_vertical_slash(qg[:, h:h + 1], kg[:, kv:kv + 1], a, b)
+            ref = O.vertical_slash_sparse_attention(q[:, h:h + 1], k[:, kv:kv + 1], v[:, kv:kv + 1], v_idx.cpu(), s_idx.cpu())
+        elif ty == "block_sparse":
+            from minference_amd.ops import _build_block_index
+            bi = _build_block_index(qg[:, h:h + 1], kg[:, kv:kv + 1], 100)[0, 0].cpu().numpy()
+            ref = O.masked_attention(q[0, h], k[0, kv], v[0, kv], O.bs_mask(bi, n))[None, None]
+        else:
+            ref = O.streaming_forward(q[:, h:h + 1], k[:, kv:kv + 1], v[:, kv:kv + 1], a, b)
+        err = (out[:, h:h + 1].float().cpu() - ref).abs()
+        print(f"  head {h} {ty}: max-abs {err.max().item():.3e} mean-abs {err.mean().item():.3e}", flush=True)
+        assert err.max() <= 2e-2 and err.mean() <= 1e-3
+
+
+def test_head_selection_leaves_other_heads_untouched(gpu):
+    """minf_qkvo.head_slot through the C ABI: a dense launch restricted to heads {1, 4, 5} of 6 writes
+    exactly those heads of the output buffer and reproduces the unrestricted launch on them."""
+    import ctypes
+    from minference_amd import _lib
+    from minference_amd.ops import _Call
+    n, hq, hk = 700, 6, 2
+    q, k, v = gen.qkv(1, hq, hk, n, 128, seed=12, scale=1.0)
+    q, k, v = q.bfloat16().to(gpu), k.bfloat16().to(gpu), v.bfloat16().to(gpu)
+    lib = _lib.load()
+    full = _Call(q, k, v)
+    assert lib.minf_dense_attn_fwd(full.ref, _lib.stream_ptr(gpu)) == 0
+    part = _Call(q, k, v)
+    part.o.fill_(-3.0)
+    slot = torch.tensor([-1, 0, -1, -1, 1, 2], dtype=torch.int32, device=gpu)
+    part.select_heads(slot, 3)
+    assert lib.minf_dense_attn_fwd(part.ref, _lib.stream_ptr(gpu)) == 0
+    torch.cuda.synchronize()
+    for h in range(hq):
+        if h in (1, 4, 5):
+            assert torch.equal(part.o[:, h], full.o[:, h])
+        else:
+            assert (part.o[:, h] == -3.0).all()
+    # a selection without a slot count is refused
+    part.struct.index_heads = 0
+    assert lib.minf_dense_attn_fwd(part.ref, _lib.stream_ptr(gpu)) == -1
+
+
 def test_starting_layer_falls_back_to_dense(gpu):
     import minference_amd as M
     q, k, v = gen.qkv(1, 4, 4, 512, 128, seed=4, scale=1.0)

@@ -31,15 +31,11 @@ def test_minference_ratio_truncates_like_the_reference():
     assert list(plan) == [("vertical_and_slash", int(1000 * 0.33), int(6096 * 0.33))]
 
 
-def test_kv_head_selection_for_gqa_groups():
-    k = torch.arange(8).float().reshape(1, 8, 1, 1)
-    # whole groups -> the kv heads themselves (shared, not expanded)
-    sel = prefill._kv_for_heads(k, [4, 5, 6, 7, 12, 13, 14, 15], 4)
-    assert sel.flatten().tolist() == [1, 3]
-    # partial groups -> one kv head per query head
-    sel = prefill._kv_for_heads(k, [0, 5, 6], 4)
-    assert sel.flatten().tolist() == [0, 1, 1]
-    assert prefill._kv_for_heads(k, [2, 7], 1).flatten().tolist() == [2, 7]
+def test_head_slot_tensor_of_a_pattern_group():
+    # position of every selected head in the group's index tensors, -1 for all other heads
+    slot = prefill._slot_tensor([1, 4, 5], 8, "cpu")
+    assert slot.dtype == torch.int32 and slot.tolist() == [-1, 0, -1, -1, 1, 2, -1, -1]
+    assert prefill._slot_tensor([], 3, "cpu").tolist() == [-1, -1, -1]
 
 
 def test_search_mode_has_no_cpu_path_and_respects_a_finished_file(tmp_path):

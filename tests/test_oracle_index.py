@@ -124,3 +124,24 @@ def test_properties_config3_generator():
                 cols = r - s[0, h][s[0, h] <= r]
                 assert cover[cols].all()
                 assert cover[v[0, h][v[0, h] <= 64 * m - 1]].all() or True
+
+
+@pytest.mark.parametrize("n,nv,ns,seed", [(1024, 7, 5, 0), (4096, 100, 300, 1), (8192, 1000, 2048, 2), (5000, 33, 65, 3)])
+def test_list_padding_is_a_noop_of_the_merge_loop(n, nv, ns, seed):
+    """One index build serves heads with different (vertical_size, slash_size) when the shorter lists
+    are padded to the longest: verticals with a constant no range ever reaches (never emitted:
+    csrc/vertical_slash_index.cu:71-74 only emits v < range_start), slashes with their last offset
+    repeated (the same column end again neither starts a range, :87-90, nor extends one, :91-92).
+    The reference algorithm must give, for the padded lists, exactly the tensors of the unpadded
+    ones followed by zeros."""
+    v, s = gen.vs_index_inputs(2, n, nv, ns, seed=seed, force_v=min(4, nv), force_s=min(64, ns))
+    bc, bo, cc, ci = O.vs_index_build([n], v, s, n)
+    vp = np.concatenate([v, np.full((1, 2, 37), 0x3FFFFFFF, np.int32)], axis=2)
+    sp = np.concatenate([s, np.repeat(s[:, :, -1:], 100, axis=2)], axis=2)
+    pbc, pbo, pcc, pci = O.vs_index_build([n], vp, sp, n)
+    assert np.array_equal(pbc, bc) and np.array_equal(pcc, cc)
+    assert np.array_equal(pbo[..., :ns], bo) and not pbo[..., ns:].any()
+    assert np.array_equal(pci[..., :nv], ci) and not pci[..., nv:].any()
+    # and row by row with the pure-Python twin
+    for m in (0, 1, (n + 63) // 64 - 1):
+        assert O.vs_index_row_py(vp[0, 1].tolist(), sp[0, 1].tolist(), m, n) == O.vs_index_row_py(v[0, 1].tolist(), s[0, 1].tolist(), m, n)
