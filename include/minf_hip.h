@@ -141,13 +141,14 @@ typedef struct minf_qkvo {
     float sm_scale;
     /* Optional head selection (per-head pattern tables: reference
      * minference/modules/minference_forward.py:621, :657-667 loops over heads and calls one operator
-     * per head).  head_slot NULL: every query head is processed and index tensors have heads_q
-     * heads.  Otherwise head_slot is a device array [heads_q]: head h is skipped when
-     * head_slot[h] < 0 (its rows of o are not touched) and else reads its index rows at head
-     * position head_slot[h] of index tensors that have index_heads heads.  q, k, v, o are always
-     * addressed with the real head number, so a launch per pattern type writes its heads of one
-     * shared output in place. */
-    const int32_t *head_slot;
+     * per head).  head_list NULL: every query head is processed and index tensors have heads_q
+     * heads.  Otherwise head_list is a device array of index_heads distinct query head numbers
+     * (ascending order keeps heads that share a kv head together): only these heads are processed
+     * (the o rows of all other heads are not touched) and head_list[i] reads its index rows at head
+     * position i of index tensors that have index_heads heads.  q, k, v, o are always addressed
+     * with the real head number, so a launch per pattern type writes its heads of one shared
+     * output in place. */
+    const int32_t *head_list;
     int index_heads;
 } minf_qkvo;
 
@@ -227,15 +228,15 @@ int minf_vs_estimate(const void *q, const void *k, const int64_t *q_stride,
 /*
  * minf_vs_estimate for a subset of the query heads (per-head pattern tables: the reference estimates
  * inside its loop over heads, minference/modules/minference_forward.py:657-667, only for the heads
- * whose pattern is vertical_and_slash).  head_slot [heads_q] int32 (device): head h is skipped when
- * head_slot[h] < 0, otherwise its score rows are row head_slot[h] of vertical / slash
- * [batch, index_heads, n]; q and k are addressed with the real head numbers.  Workspace:
+ * whose pattern is vertical_and_slash).  head_list [index_heads] int32 (device): the query heads to
+ * score; the scores of head_list[i] are row i of vertical / slash [batch, index_heads, n]; q and k
+ * are addressed with the real head numbers.  Workspace:
  * minf_vs_estimate_workspace_bytes(batch, index_heads, n).
  */
 int minf_vs_estimate_heads(const void *q, const void *k, const int64_t *q_stride,
                            const int64_t *k_stride, int batch, int heads_q, int heads_kv, int n,
                            int head_dim, int dtype, float sm_scale, int last_q, int force_vertical,
-                           int force_slash, const int32_t *head_slot, int index_heads,
+                           int force_slash, const int32_t *head_list, int index_heads,
                            float *vertical, float *slash, void *workspace,
                            size_t workspace_bytes, void *stream);
 
@@ -315,14 +316,14 @@ int minf_bs_block_index(const void *q, const void *k, const int64_t *q_stride,
                         void *stream);
 
 /*
- * minf_bs_block_index for a subset of the query heads (head_slot as in minf_vs_estimate_heads):
+ * minf_bs_block_index for a subset of the query heads (head_list as in minf_vs_estimate_heads):
  * block_index [batch, index_heads, rows, min(top_k, rows)]; workspace
  * minf_bs_block_index_workspace_bytes(batch, index_heads, heads_kv, n).
  */
 int minf_bs_block_index_heads(const void *q, const void *k, const int64_t *q_stride,
                               const int64_t *k_stride, int batch, int heads_q, int heads_kv, int n,
                               int head_dim, int dtype, int top_k, int force_diag_first,
-                              const int32_t *head_slot, int index_heads,
+                              const int32_t *head_list, int index_heads,
                               int32_t *block_index, void *workspace, size_t workspace_bytes,
                               void *stream);
 

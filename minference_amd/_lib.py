@@ -65,7 +65,7 @@ class QKVO(ctypes.Structure):
         ("head_dim", c_int), ("dtype", c_int),
         ("seqlens", c_ptr),
         ("sm_scale", c_f32),
-        ("head_slot", c_ptr),
+        ("head_list", c_ptr),
         ("index_heads", c_int),
     ]
 

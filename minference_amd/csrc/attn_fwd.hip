@@ -2,10 +2,19 @@
 // sources (vertical-slash block+column lists, block-sparse lists, analytic
 // A-shape ranges, dense causal).
 //
-// Work split: one workgroup (2 wavefronts) per (batch, query head, 64-row
-// block); each wavefront owns 32 query rows.  Dense, A-shape / tri-shape and block-sparse launches
-// use the paired variant: 4 wavefronts over two neighbouring row blocks that walk the union of
-// their tile lists and share every K/V tile copy.
+// Work split: one workgroup of 4 wavefronts per (batch, query head, PAIR of neighbouring 64-row
+// blocks); each wavefront owns 32 query rows.  The two row blocks walk their tile lists in lockstep:
+// a tile that is on both lists is copied into LDS once for 128 query rows, a tile that only one of
+// them visits is copied by that half into buffers of its own while the other half does the same
+// with a tile of its list.  For dense causal and A-shape / tri-shape the lists are analytic and
+// differ by at most their ends; block-sparse lists are merged on the fly; vertical-slash lists are
+// split into common and leftover entries once, in LDS, before the tile loop.  Besides halving the
+// copies of shared tiles, the lockstep is what keeps long scattered lists fast: row block m+1's
+// list is row block m's shifted by 64 keys, so what one half fetches now the other fetched a step
+// ago and finds in L2 (measured +23..38 % on lists of several hundred blocks, +1 % on the
+// cache-friendly benchmark layer, against one 2-wave workgroup per row block).  The 2-wave form
+// (one workgroup per 64-row block) remains for block-sparse lists longer than the paired walk
+// keeps in LDS.
 // Everything is computed in the TRANSPOSED orientation so that softmax statistics are per lane:
 //
 //   S^T[token][qrow] = K_tile . Q^T      v_mfma_f32_32x32x16 (A = K from LDS, B = Q in VGPRs)
@@ -18,15 +27,16 @@
 // the probabilities of a lane are exactly the B operand of the second MFMA once
 // the contraction (token) index is permuted the same way on the V side.
 //
-// LDS: one K and one V tile per workgroup, [64 tokens][128] 16-bit, 256-byte rows whose 16-byte
+// LDS: one K and one V tile per workgroup (two of each for vertical-slash lists: the second pair
+// serves row block B in split steps), [64 tokens][128] 16-bit, 256-byte rows whose 16-byte
 // chunks are XOR-permuted (K: chunk ^ row%16, V: chunk ^ 4*(row%4)) so that the ds_read_b128 of 32
 // K rows and the 4-row transpose reads of V hit distinct banks.  Tiles are copied global -> LDS
 // directly (no staging registers, no LDS store instructions); the permutation is applied on the
 // global-address side.  Contiguous tiles use buffer_load_dwordx4 ... lds with a scalar descriptor of
 // the 64 tile rows, a scalar row offset and one of five loop-invariant per-lane offsets: no vector
 // instruction per copy and 8 cycles less issue time per copy than the 64-bit-address form, which
-// remains for gathered and clamped rows (global_load_lds_dwordx4).  32 KB of LDS and <= 256 registers keep four
-// workgroups (two waves per SIMD) resident per CU.
+// remains for gathered and clamped rows (global_load_lds_dwordx4).  32-68 KB of LDS and <= 256 registers
+// keep two waves per SIMD resident (two 4-wave or four 2-wave workgroups per CU).
 //
 // One iteration of a wave (two workgroup barriers per tile, single buffers):
 //   wait own K(it) copies; barrier (all of K(it) visible, everyone done with V(it-1))
@@ -97,9 +107,10 @@ struct AttnParams {
     int n_init, n_local, dense_from;
     long long total_wg;
     int descending;          // row blocks are handed out from the last one down
-    // optional head selection: head_slot[h] < 0 skips query head h; otherwise it is the head's
-    // position in the index tensors, which then have index_heads heads (index_heads = hq without it)
-    const int *head_slot;
+    // optional head selection: head_list[i], i < index_heads, are the query heads to process and i is
+    // the head's position in the index tensors (which then have index_heads heads); without a list
+    // every head is processed and index_heads = hq
+    const int *head_list;
     int index_heads;
 };
 
@@ -161,9 +172,12 @@ struct Tile {
     int start;          // first token (contiguous) / first list position (gathered)
     int gathered;       // 0/1
     int nvalid;         // gathered: number of valid list entries in this tile
-    int on_a, on_b;     // paired block-sparse walk: is the tile on the list of row block A / B
+    int on_a, on_b;     // paired walks: is the tile on the list of row block A / B
+    int split;          // paired vertical-slash: each row block has a tile of its own in this step
 };
 constexpr int BS_PAIR_MAX = 512;   // longest block list the paired block-sparse walk keeps in LDS
+constexpr int VS_PAIR_MAX = 2048;  // longest vertical-slash block list the paired kernel merges in LDS
+constexpr int VS_ONLY_MAX = 512;   // ... and the most entries of one list that the other one lacks
 
 template <int MODE>
 __device__ __forceinline__ int tile_count(const AttnParams &p, long long ridx, int m, int &nblk) {
@@ -253,12 +267,18 @@ __device__ __forceinline__ bool tile_on_list(const AttnParams &p, int m, int sta
 
 template <typename T, int MODE, bool PAIR>
 __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_kernel(const AttnParams p) {
-    static_assert(!PAIR || MODE != MODE_VS, "paired variant: no vertical-slash lists");
     constexpr int NT = PAIR ? 2 * NTHREADS : NTHREADS;      // threads per workgroup
-    constexpr int CROWS = PAIR ? 16 : 32;                   // tile rows copied by one wave
-    // two separate LDS objects: the compiler then lets reads of one overtake copies into the other
-    __shared__ __attribute__((aligned(16))) char lds_k[BN * ROW_BYTES];
-    __shared__ __attribute__((aligned(16))) char lds_v[BN * ROW_BYTES];
+    constexpr int CROWS = PAIR ? 16 : 32;                   // tile rows copied by one wave (shared tile)
+    constexpr bool VSP = PAIR && MODE == MODE_VS;
+    constexpr int TILE_BYTES = BN * ROW_BYTES;
+    // separate LDS objects: the compiler then lets reads of one overtake copies into the other
+    // paired vertical-slash: a second K and V tile (row block B's buffers in the steps in which each
+    // row block has a tile of its own); before that, the second K tile stages the two block lists and
+    // the second V tile holds their merge
+    __shared__ __attribute__((aligned(16))) char lds_k[(VSP ? 2 : 1) * TILE_BYTES];
+    __shared__ __attribute__((aligned(16))) char lds_v[(VSP ? 2 : 1) * TILE_BYTES];
+    char *const lds_k1 = lds_k + (VSP ? TILE_BYTES : 0);
+    char *const lds_v1 = lds_v + (VSP ? TILE_BYTES : 0);
 
     // ---- which (batch, head, row block): XCD-aware remap --------------------
     // Consecutive workgroup ids are dealt round-robin to the 8 XCDs; give each
@@ -278,13 +298,22 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
     const int rows_wg = PAIR ? (p.rows + 1) >> 1 : p.rows;           // row-block slots per (batch, head)
     const int mi = (int)(rest % rows_wg); rest /= rows_wg;
     const int mslot = p.descending ? rows_wg - 1 - mi : mi;
-    const int hkv = (int)(rest % p.hk);
-    const int b = (int)(rest / p.hk);
-    const int h = hkv * group + hin;
-    int hs = h;                                    // head position in the index tensors
-    if (p.head_slot) {
-        hs = as_const(p.head_slot)[h];
-        if (hs < 0) return;                        // not one of this launch's heads (workgroup-uniform)
+    int hkv, b, h, hs;                               // hs: head position in the index tensors
+    if (p.head_list) {
+        // the selected heads in chunks of `group` consecutive list entries take the place of the kv
+        // groups: neighbours in the (ascending) list mostly share a kv head
+        const int nch = (p.index_heads + group - 1) / group;
+        const int ch = (int)(rest % nch);
+        b = (int)(rest / nch);
+        hs = ch * group + hin;
+        if (hs >= p.index_heads) return;             // padding of the last chunk (workgroup-uniform)
+        h = as_const(p.head_list)[hs];
+        hkv = h / group;
+    } else {
+        hkv = (int)(rest % p.hk);
+        b = (int)(rest / p.hk);
+        h = hkv * group + hin;
+        hs = h;
     }
 
     const int tid = (int)threadIdx.x;
@@ -345,6 +374,91 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
         for (int i = tid; i < bs_nb; i += NT) lds_list[BS_PAIR_MAX + i] = p.bidx[(rbase + mA + 1) * p.max_blocks + i];
         __syncthreads();
     }
+    // Paired vertical-slash: the block lists of the two row blocks (ascending key starts; those of
+    // neighbouring row blocks are each other's translate by 64 keys wherever no entry is clipped, so
+    // runs of blocks share all but their ends) are split ONCE, by all 256 threads, before the tile
+    // loop: both lists are staged in LDS, every entry looks itself up in the other list by binary
+    // search, and a workgroup prefix sum over the hits places it either in the list of COMMON
+    // entries (tiles that both row blocks visit: copied once by four waves, one LDS word per step)
+    // or in its row block's list of entries the other one lacks (run ends).  The walk is then
+    //   common tiles, both halves computing;
+    //   split steps: every half visits its own leftover tiles -- the entries the other list lacks,
+    //   then its gathered column tiles -- with the K/V buffers of its own half,
+    // i.e. exactly max(tiles of A, tiles of B) steps, never more than the longer list alone.
+    // Lists that are too long for LDS or not strictly ascending are not split: each half then walks
+    // its whole list in split steps (still in lockstep with its neighbour, which is what keeps the
+    // neighbour's tiles in L2 when the lists are long and scattered).
+    [[maybe_unused]] int vs_na = 0, vs_nb = 0, vs_cca = 0, vs_ccb = 0, vs_nc = 0;
+    [[maybe_unused]] bool vs_merged = false;
+    [[maybe_unused]] long long vs_ra = 0, vs_rb = 0;
+    __shared__ int vs_only[VSP ? 2 * VS_ONLY_MAX : 1];        // [row block][entries the other list lacks]
+    if constexpr (VSP) {
+        __shared__ int vs_wsum[4];
+        __shared__ int vs_bad;
+        const bool b_exists = 2 * mslot + 1 < p.rows && (2 * mslot + 1) * BM < seqlen;
+        vs_ra = ((long long)b * p.index_heads + hs) * p.rows + mA;
+        vs_rb = b_exists ? vs_ra + 1 : vs_ra;
+        vs_na = max(0, min(as_const(p.bc)[vs_ra], p.nnz_s));
+        vs_cca = max(0, min(as_const(p.cc)[vs_ra], p.nnz_v));
+        vs_nb = b_exists ? max(0, min(as_const(p.bc)[vs_rb], p.nnz_s)) : 0;
+        vs_ccb = b_exists ? max(0, min(as_const(p.cc)[vs_rb], p.nnz_v)) : 0;
+        if (vs_na <= VS_PAIR_MAX && vs_nb <= VS_PAIR_MAX && vs_na > 0 && vs_nb > 0) {
+            int *rawA = reinterpret_cast<int *>(lds_k1), *rawB = rawA + VS_PAIR_MAX;
+            int *common = reinterpret_cast<int *>(lds_v1);
+            const int *ga = p.bo + vs_ra * p.nnz_s, *gb = p.bo + vs_rb * p.nnz_s;
+            if (tid == 0) vs_bad = 0;
+            for (int i = tid; i < vs_na; i += NT) rawA[i] = ga[i];
+            for (int i = tid; i < vs_nb; i += NT) rawB[i] = gb[i];
+            __syncthreads();
+            bool bad = false;                              // the look-ups need strictly ascending lists
+            for (int i = tid; i + 1 < vs_na; i += NT) bad |= rawA[i + 1] <= rawA[i];
+            for (int i = tid; i + 1 < vs_nb; i += NT) bad |= rawB[i + 1] <= rawB[i];
+            if (__any(bad) && lane == 0) vs_bad = 1;
+            __syncthreads();
+            if (!vs_bad) {                                 // (workgroup-uniform)
+                const unsigned long long lt = (1ull << lane) - 1ull;
+                // entry i of `mine` goes to common[#hits before i] when `other` holds it too (first
+                // pass only), else to only[i - #hits before i]; -> number of hits
+                auto pass = [&](const int *mine, int nmine, const int *other, int nother, int *only, bool write_common) {
+                    int carry = 0;
+                    for (int base = 0; base < nmine; base += NT) {        // uniform trip count
+                        const int i = base + tid;
+                        const bool valid = i < nmine;
+                        const int x = valid ? mine[i] : 0;
+                        int lo = 0, hi = nother;                           // first entry of `other` >= x
+                        while (lo < hi) {
+                            const int mid = (lo + hi) >> 1;
+                            if (other[mid] < x) lo = mid + 1; else hi = mid;
+                        }
+                        const bool eq = valid && lo < nother && other[lo] == x;
+                        const unsigned long long bal = __ballot(eq);
+                        if (lane == 0) vs_wsum[wave_wg] = __builtin_popcountll(bal);
+                        __syncthreads();
+                        int pre = carry, tot = 0;
+#pragma unroll
+                        for (int w = 0; w < 4; ++w) {
+                            const int c = vs_wsum[w];
+                            pre += w < wave_wg ? c : 0;
+                            tot += c;
+                        }
+                        pre += __builtin_popcountll(bal & lt);
+                        if (valid) {
+                            if (eq) { if (write_common) common[pre] = x; }
+                            else if (i - pre < VS_ONLY_MAX) only[i - pre] = x;
+                        }
+                        carry += tot;
+                        __syncthreads();
+                    }
+                    return carry;
+                };
+                vs_nc = pass(rawA, vs_na, rawB, vs_nb, vs_only, true);
+                pass(rawB, vs_nb, rawA, vs_na, vs_only + VS_ONLY_MAX, false);
+                // (the last barrier of the passes also orders these LDS lists before their readers)
+                vs_merged = vs_nc > 0 && vs_na - vs_nc <= VS_ONLY_MAX && vs_nb - vs_nc <= VS_ONLY_MAX;
+                if (!vs_merged) vs_nc = 0;
+            }
+        }
+    }
     auto bs_merge_next = [&]() -> Tile {      // one step of the merged walk (wave-uniform)
         Tile t;
         t.gathered = 0;
@@ -361,15 +475,57 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
     };
     // the merged walk ends when both lists are used up (its length is not known in advance)
     int ntiles = 0;
-    if constexpr (!(PAIR && MODE == MODE_BS))
+    // paired vertical-slash: vs_nc common steps, then the split steps: per half its leftover block
+    // entries (from LDS when the lists were split, else its whole list from global memory) and its
+    // gathered column tiles.  The barriers are the workgroup's: both halves make max(A, B) split
+    // steps and a half without a tile only keeps the barriers.
+    [[maybe_unused]] int vs_nb_mine = 0, vs_cc_mine = 0, vs_nt_mine = 0;
+    if constexpr (VSP) {
+        const int nb_a = vs_na - vs_nc, nb_b = vs_nb - vs_nc;
+        const int nt_a = nb_a + ((vs_cca + BN - 1) >> 6), nt_b = nb_b + ((vs_ccb + BN - 1) >> 6);
+        vs_nb_mine = half ? nb_b : nb_a;
+        vs_cc_mine = half ? vs_ccb : vs_cca;
+        vs_nt_mine = have_rows ? (half ? nt_b : nt_a) : 0;
+        ntiles = vs_nc + max(nt_a, nt_b);
+    }
+    else if constexpr (!(PAIR && MODE == MODE_BS))
         ntiles = PAIR ? pair_tile_count<MODE>(p, mA, mB, nblk) : tile_count<MODE>(p, ridx, m, nblk);
     auto more_tiles = [&](int it) -> bool {   // is there a tile number `it` ?
         if constexpr (PAIR && MODE == MODE_BS) return bs_ia < bs_na || bs_ib < bs_nb;
         else return it < ntiles;
     };
+    // paired vertical-slash: entry it+1 of the common list sits in a scalar when step `it` starts; the
+    // LDS read of entry it+2 is issued at the top of step `it` (no tile copy is in flight there: the
+    // list shares an LDS object with the V tiles and must not wait for one) and turns into the next
+    // scalar at the end of the step, its latency hidden behind the tile's work
+    [[maybe_unused]] int vs_entry = 0, vs_pref = 0;
+    auto vs_list = [&](int i) -> int { return reinterpret_cast<const int *>(lds_v1)[min(i, 2 * VS_PAIR_MAX - 1)]; };
     auto tile_of = [&](int it) -> Tile {      // called with it = 0, 1, 2, ... in order
         if constexpr (PAIR && MODE == MODE_BS) {
             return bs_merge_next();
+        } else if constexpr (VSP) {
+            Tile t;
+            t.gathered = 0;
+            t.nvalid = BN;
+            if (it < vs_nc) {
+                t.split = 0;
+                t.on_a = t.on_b = 1;
+                t.start = vs_entry;                        // common entry `it`, fetched a step ahead
+            } else {
+                const int j = it - vs_nc;
+                t.split = 1;
+                t.on_a = t.on_b = j < vs_nt_mine;          // (this half's own flag)
+                t.start = 0;
+                if (j < vs_nb_mine) {
+                    if (vs_merged) t.start = __builtin_amdgcn_readfirstlane(vs_only[half * VS_ONLY_MAX + j]);
+                    else t.start = as_const(p.bo)[ridx * p.nnz_s + j];
+                } else if (j < vs_nt_mine) {
+                    t.gathered = 1;
+                    t.start = (j - vs_nb_mine) * BN;
+                    t.nvalid = min(BN, vs_cc_mine - t.start);
+                }
+            }
+            return t;
         } else if constexpr (PAIR) {
             Tile t;
             t.gathered = 0;
@@ -399,51 +555,72 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
     for (int jj = 0; jj < 4; ++jj) k_lane[jj] = cp_r * (int)k_row + ((cp_c ^ (4 * jj + cp_r)) << 4);
     v_lane = cp_r * (int)v_row + ((cp_c ^ (cp_r << 2)) << 4);
     auto gather_ids = [&](const Tile &t) -> int {
-        if (MODE == MODE_VS && t.gathered) return p.ci[ridx * p.nnz_v + t.start + min(lane, t.nvalid - 1)];
+        if (MODE == MODE_VS && t.gathered) return p.ci[ridx * p.nnz_v + t.start + min(lane, max(t.nvalid, 1) - 1)];
         return 0;
     };
-    auto copy_tile = [&](const Tile &t, const char *base, long long rowstride, auto is_v_c, int idv,
-                         char *ldsbuf) {
+    // rows_c: tile rows copied by one wave (16: the four waves of a pair share the tile, 32: the
+    // two waves of a row block copy it); wsel: which part of the tile this wave copies
+    auto copy_rows = [&](const Tile &t, const char *base, long long rowstride, auto is_v_c, int idv,
+                         char *ldsbuf, auto rows_c, const int wsel) {
         constexpr bool is_v = decltype(is_v_c)::value;
+        constexpr int CROWS = decltype(rows_c)::value;
         const bool gathered = MODE == MODE_VS && t.gathered;
         if (!gathered && t.start >= 0 && t.start + BN <= seqlen) {
             // buffer form: descriptor of the 64 tile rows (scalar), one of five per-lane offsets (the V
             // swizzle does not depend on j, the K swizzle only on j % 4) and a scalar row offset
             const char *tb = base + (long long)t.start * rowstride;      // wave-uniform
             const __amdgpu_buffer_rsrc_t srd = __builtin_amdgcn_make_buffer_rsrc((void *)tb, 0, BN * (int)rowstride, 0x00020000);
+            // first row offset and step of this wave's part; in the paired vertical-slash kernel (two
+            // copy shapes, K and V strides) they are made opaque so that the per-copy offsets are formed
+            // with one scalar add each instead of living in two dozen loop-invariant scalar registers
+            int soff0 = CROWS * wsel * (int)rowstride, sstep = 4 * (int)rowstride;
+            int lds0 = (int)(unsigned)(unsigned long long)(__attribute__((address_space(3))) char *)ldsbuf + CROWS * wsel * ROW_BYTES;
+            if constexpr (VSP) asm volatile("" : "+s"(soff0), "+s"(sstep), "+s"(lds0));
 #pragma unroll
             for (int j = 0; j < CROWS / 4; ++j) {
                 const int voff = is_v ? v_lane : k_lane[j & 3];
-                const int soff = (CROWS * wave_wg + 4 * j) * (int)rowstride;
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(srd, (__attribute__((address_space(3))) void *)(ldsbuf + (CROWS * wave_wg + 4 * j) * ROW_BYTES),
-                                                         16, voff, soff, 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(srd, (__attribute__((address_space(3))) void *)(unsigned long long)(unsigned)(lds0 + 4 * j * ROW_BYTES),
+                                                         16, voff, soff0 + j * sstep, 0, 0);
             }
             return;
         }
-        // three straight-line variants (a per-row select would turn into sixteen tiny branches)
+        // three straight-line variants (a per-row select would turn into sixteen tiny branches).
+        // The two rare ones recompute their per-lane rows and chunks on the spot (the empty asm
+        // keeps the compiler from hoisting a dozen loop-invariant registers out of the tile loop).
+        int cp_r = lane >> 4, cp_c = lane & 15;
+        asm volatile("" : "+v"(cp_r), "+v"(cp_c));
         if (gathered) {
 #pragma unroll
             for (int j = 0; j < CROWS / 4; ++j) {
-                const int r = CROWS * wave_wg + 4 * j + cp_r;          // tile row
+                const int r = CROWS * wsel + 4 * j + cp_r;          // tile row
                 const int tk = max(0, min(__shfl(idv, r), seqlen - 1));
                 const int c = is_v ? (cp_c ^ ((r & 3) << 2)) : (cp_c ^ (r & 15));
                 const char *gp = base + tk * rowstride + c * 16;
                 __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
-                                                 (__attribute__((address_space(3))) void *)(ldsbuf + (CROWS * wave_wg + 4 * j) * ROW_BYTES),
+                                                 (__attribute__((address_space(3))) void *)(ldsbuf + (CROWS * wsel + 4 * j) * ROW_BYTES),
                                                  16, 0, 0);
             }
             return;
         }
 #pragma unroll
         for (int j = 0; j < CROWS / 4; ++j) {
-            const int r = CROWS * wave_wg + 4 * j + cp_r;
+            const int r = CROWS * wsel + 4 * j + cp_r;
             const int tk = max(0, min(t.start + r, seqlen - 1));
             const int c = is_v ? (cp_c ^ ((r & 3) << 2)) : (cp_c ^ (r & 15));
             const char *gp = base + tk * rowstride + c * 16;
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
-                                             (__attribute__((address_space(3))) void *)(ldsbuf + (CROWS * wave_wg + 4 * j) * ROW_BYTES),
+                                             (__attribute__((address_space(3))) void *)(ldsbuf + (CROWS * wsel + 4 * j) * ROW_BYTES),
                                              16, 0, 0);
         }
+    };
+    auto copy_tile = [&](const Tile &t, const char *base, long long rowstride, auto is_v_c, int idv, char *ldsbuf) {
+        if constexpr (VSP) {
+            if (t.split) {
+                if (t.on_a) copy_rows(t, base, rowstride, is_v_c, idv, ldsbuf + half * TILE_BYTES, std::integral_constant<int, 32>{}, wave);
+                return;
+            }
+        }
+        copy_rows(t, base, rowstride, is_v_c, idv, ldsbuf, std::integral_constant<int, CROWS>{}, wave_wg);
     };
 
     // ---- accumulators -------------------------------------------------------
@@ -469,87 +646,54 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
     for (int db = 0; db < 4; ++db)
         v_rd_off[db] = (4 * g + v_rd_rsub) * ROW_BYTES + ((((db ^ v_rd_rsub) << 2) + v_rd_vc) << 4) + ((lane & 1) << 3);
 
-    // Single K and V buffers, two barriers per tile:
-    //   [own K(it) copies landed] barrier B1 (also: every wave is done with V(it-1))
-    //   issue V(it) copy; fetch gathered ids of tile it+1; S^T = K.Q^T
-    //   [own V(it) copies landed] barrier B2 (also: every wave is done with K(it))
-    //   issue K(it+1) copy; softmax; O^T += V^T.P^T
-    Tile cur, nxt;
-    int gt_cur = 0, gt_nxt = 0;
-    bool have_cur = more_tiles(0);
-    if (have_cur) {
-        cur = tile_of(0);
-        gt_cur = gather_ids(cur);
-        copy_tile(cur, k_base, k_row, std::false_type{}, gt_cur, lds_k);
-    }
-
-    for (int it = 0; have_cur; ++it) {
-        __builtin_amdgcn_s_waitcnt(0x0f70);      // vmcnt(0): this wave's part of K(it) is in LDS
-        __syncthreads();
+    // ---- S^T = K . Q^T for this wave's 32 query rows; K tile in kbuf.  EARLY (2-wave kernel, whose
+    // waves all run this code): the tile's second barrier comes after k-step EARLY_B2, when every K
+    // fragment has been read, and all V^T fragment reads are issued under the last four MFMAs.
+    auto qk_block = [&](const char *kbuf, const char *vbuf, f32x16_t &s0, f32x16_t &s1, Frag (&vf)[4][4], auto early_c) {
+        constexpr bool EARLY = decltype(early_c)::value;
         Frag a0[8], a1[8];
-        copy_tile(cur, v_base, v_row, std::true_type{}, gt_cur, lds_v);
-        const bool have_nxt = more_tiles(it + 1);
-        nxt = have_nxt ? tile_of(it + 1) : cur;
-        gt_nxt = gather_ids(nxt);
-
-        // paired variant: is this tile on the list of this wave's row block ?
-        bool active = true;
-        if constexpr (PAIR && MODE == MODE_BS) active = have_rows && (half ? cur.on_b : cur.on_a);
-        else if constexpr (PAIR) active = have_rows && tile_on_list<MODE>(p, m, cur.start);
-        f32x16_t s0, s1;
-        Frag vf[4][4];
-        if (active) {
         __builtin_amdgcn_s_setprio(2);
-        // ---- S^T = K . Q^T --------------------------------------------------
 #pragma unroll
         for (int r = 0; r < 16; ++r) { s0[r] = 0.f; s1[r] = 0.f; }
-        {
-            // K fragments are fetched QK_AHEAD k-steps before the MFMAs that consume them; the
-            // scheduling fences keep the compiler from sinking the reads back to their use
+        // K fragments are fetched QK_AHEAD k-steps before the MFMAs that consume them; the
+        // scheduling fences keep the compiler from sinking the reads back to their use
 #pragma unroll
-            for (int ks = 0; ks < QK_AHEAD; ++ks) {
-                a0[ks].u = *reinterpret_cast<const u32x4_t *>(lds_k + k_rd_off[ks]);
-                a1[ks].u = *reinterpret_cast<const u32x4_t *>(lds_k + k_rd_off[ks] + 32 * ROW_BYTES);
+        for (int ks = 0; ks < QK_AHEAD; ++ks) {
+            a0[ks].u = *reinterpret_cast<const u32x4_t *>(kbuf + k_rd_off[ks]);
+            a1[ks].u = *reinterpret_cast<const u32x4_t *>(kbuf + k_rd_off[ks] + 32 * ROW_BYTES);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) {
+            if (ks + QK_AHEAD < 8) {
+                a0[ks + QK_AHEAD].u = *reinterpret_cast<const u32x4_t *>(kbuf + k_rd_off[ks + QK_AHEAD]);
+                a1[ks + QK_AHEAD].u = *reinterpret_cast<const u32x4_t *>(kbuf + k_rd_off[ks + QK_AHEAD] + 32 * ROW_BYTES);
             }
+            s0 = Mma<T>::mfma(frag_as<T>(a0[ks]), frag_as<T>(qf[ks]), s0);
+            s1 = Mma<T>::mfma(frag_as<T>(a1[ks]), frag_as<T>(qf[ks]), s1);
             __builtin_amdgcn_sched_barrier(0);
+            if constexpr (EARLY) {
+                if (ks == EARLY_B2) {
+                    __builtin_amdgcn_s_waitcnt(0x0f70);
+                    __syncthreads();
 #pragma unroll
-            for (int ks = 0; ks < 8; ++ks) {
-                if (ks + QK_AHEAD < 8) {
-                    a0[ks + QK_AHEAD].u = *reinterpret_cast<const u32x4_t *>(lds_k + k_rd_off[ks + QK_AHEAD]);
-                    a1[ks + QK_AHEAD].u = *reinterpret_cast<const u32x4_t *>(lds_k + k_rd_off[ks + QK_AHEAD] + 32 * ROW_BYTES);
-                }
-                s0 = Mma<T>::mfma(frag_as<T>(a0[ks]), frag_as<T>(qf[ks]), s0);
-                s1 = Mma<T>::mfma(frag_as<T>(a1[ks]), frag_as<T>(qf[ks]), s1);
-                __builtin_amdgcn_sched_barrier(0);
-                if constexpr (!PAIR && EARLY_B2 >= 0) {
-                    if (ks == EARLY_B2) {
-                        // every K fragment has been read: the second barrier comes before the last
-                        // four MFMAs (2-wave kernel only: all its waves run this code) and the V^T
-                        // fragment reads are issued under them (+0.9 %)
-                        __builtin_amdgcn_s_waitcnt(0x0f70);
-                        __syncthreads();
+                    for (int s = 0; s < 4; ++s)
 #pragma unroll
-                        for (int s = 0; s < 4; ++s)
+                        for (int db = 0; db < 4; ++db)
 #pragma unroll
-                            for (int db = 0; db < 4; ++db)
-#pragma unroll
-                                for (int jj = 0; jj < 2; ++jj)
-                                    vf[s][db].s4[jj] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                                        (__attribute__((address_space(3))) short4_t *)(lds_v + v_rd_off[db] + (16 * s + 8 * jj) * ROW_BYTES));
-                    }
+                            for (int jj = 0; jj < 2; ++jj)
+                                vf[s][db].s4[jj] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                                    (__attribute__((address_space(3))) short4_t *)(vbuf + v_rd_off[db] + (16 * s + 8 * jj) * ROW_BYTES));
                 }
             }
         }
         __builtin_amdgcn_s_setprio(0);
-        }
-        if constexpr (PAIR || EARLY_B2 < 0) {
-        __builtin_amdgcn_s_waitcnt(0x0f70);      // vmcnt(0): this wave's part of V(it) is in LDS
-        __syncthreads();
-        }
-        if (have_nxt) copy_tile(nxt, k_base, k_row, std::false_type{}, gt_nxt, lds_k);
-        if (active) {
+    };
 
-        // ---- mask -----------------------------------------------------------
+    // ---- mask, online softmax, O^T += V^T . P^T.  READ_V: the V^T fragments have not been read yet
+    // (4-wave variants, whose second barrier sits between the two blocks).
+    auto sm_pv_block = [&](const Tile &cur, const char *vbuf, f32x16_t &s0, f32x16_t &s1, Frag (&vf)[4][4], auto read_v_c) {
+        constexpr bool READ_V = decltype(read_v_c)::value;
         // element (blk, r) of this lane is tile-local key tk = tkc + 4*g with the compile-time
         // part tkc = 32*blk + 8*(r/4) + r%4.  keep <=> tk <= hi && (tk > wlo || tk < slim).
         bool need_mask;
@@ -592,7 +736,7 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
             }
         }
 
-        if constexpr (PAIR || EARLY_B2 < 0) {
+        if constexpr (READ_V) {
         // All V^T fragments of the tile are read here, in one scheduling region with the row-max
         // chain: the PV block below is bound by its vector instructions, so every LDS read moved out
         // of it shortens it (+3 % for the 24 reads that used to sit between its MFMAs), and the reads
@@ -604,7 +748,7 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
 #pragma unroll
             for (int jj = 0; jj < 2; ++jj)
                 vf[s][db].s4[jj] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (__attribute__((address_space(3))) short4_t *)(lds_v + v_rd_off[db] + (16 * s + 8 * jj) * ROW_BYTES));
+                    (__attribute__((address_space(3))) short4_t *)(vbuf + v_rd_off[db] + (16 * s + 8 * jj) * ROW_BYTES));
         }
         // ---- online softmax (exp2 domain) -------------------------------------
         float mx;
@@ -665,7 +809,67 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
             }
         }
         __builtin_amdgcn_s_setprio(0);
+    };
+
+    // Single K and V buffers, two barriers per tile:
+    //   [own K(it) copies landed] barrier B1 (also: every wave is done with V(it-1))
+    //   issue V(it) copy; fetch gathered ids of tile it+1; S^T = K.Q^T
+    //   [own V(it) copies landed] barrier B2 (also: every wave is done with K(it))
+    //   issue K(it+1) copy; softmax; O^T += V^T.P^T
+    Tile cur, nxt;
+    int gt_cur = 0, gt_nxt = 0;
+    [[maybe_unused]] bool vs_shifted = false;
+    bool have_cur = more_tiles(0);
+    if (have_cur) {
+        if constexpr (VSP) vs_entry = __builtin_amdgcn_readfirstlane(vs_list(0));
+        cur = tile_of(0);
+        if constexpr (VSP) vs_entry = __builtin_amdgcn_readfirstlane(vs_list(1));
+        gt_cur = gather_ids(cur);
+        copy_tile(cur, k_base, k_row, std::false_type{}, gt_cur, lds_k);
+    }
+
+    for (int it = 0; have_cur; ++it) {
+        __builtin_amdgcn_s_waitcnt(0x0f70);      // vmcnt(0): this wave's part of K(it) is in LDS
+        __syncthreads();
+        bool have_nxt;
+        if constexpr (VSP) {
+            // the merged list shares an LDS object with the V tiles: its entry is read while no copy
+            // is in flight, so that the read never waits for one
+            vs_pref = vs_list(it + 2);
+            have_nxt = more_tiles(it + 1);
+            nxt = have_nxt ? tile_of(it + 1) : cur;
+            gt_nxt = gather_ids(nxt);
+            copy_tile(cur, v_base, v_row, std::true_type{}, gt_cur, lds_v);
+            if (cur.split && !vs_shifted) {
+                // first split step: row block B reads the second tiles from here on (the LDS read
+                // offsets move in place, once)
+                vs_shifted = true;
+#pragma unroll
+                for (int ks = 0; ks < 8; ++ks) k_rd_off[ks] += half * TILE_BYTES;
+#pragma unroll
+                for (int db = 0; db < 4; ++db) v_rd_off[db] += half * TILE_BYTES;
+            }
+        } else {
+            copy_tile(cur, v_base, v_row, std::true_type{}, gt_cur, lds_v);
+            have_nxt = more_tiles(it + 1);
+            nxt = have_nxt ? tile_of(it + 1) : cur;
+            gt_nxt = gather_ids(nxt);
         }
+
+        // paired variant: is this tile on the list of this wave's row block ?
+        bool active = true;
+        if constexpr (PAIR && (MODE == MODE_BS || MODE == MODE_VS)) active = have_rows && (half ? cur.on_b : cur.on_a);   // (split steps: on_a == on_b == own flag)
+        else if constexpr (PAIR) active = have_rows && tile_on_list<MODE>(p, m, cur.start);
+        f32x16_t s0, s1;
+        Frag vf[4][4];
+        if (active) qk_block(lds_k, lds_v, s0, s1, vf, std::integral_constant<bool, !PAIR>{});
+        if constexpr (PAIR) {
+            __builtin_amdgcn_s_waitcnt(0x0f70);      // vmcnt(0): this wave's part of V(it) is in LDS
+            __syncthreads();
+        }
+        if (have_nxt) copy_tile(nxt, k_base, k_row, std::false_type{}, gt_nxt, lds_k);
+        if (active) sm_pv_block(cur, lds_v, s0, s1, vf, std::integral_constant<bool, PAIR>{});
+        if constexpr (VSP) vs_entry = __builtin_amdgcn_readfirstlane(vs_pref);
         cur = nxt;
         gt_cur = gt_nxt;
         have_cur = have_nxt;
@@ -709,7 +913,7 @@ int check_tensors(const minf_qkvo *t) {
     const bool empty = t->batch == 0 || t->n == 0;
     if (!empty && (!t->q || !t->k || !t->v || !t->o)) return MINF_ERR_INVALID_ARG;
     if (t->heads_q % t->heads_kv != 0) return MINF_ERR_INVALID_ARG;
-    if (t->head_slot && t->index_heads <= 0) return MINF_ERR_INVALID_ARG;
+    if (t->head_list && t->index_heads <= 0) return MINF_ERR_INVALID_ARG;
     if (t->head_dim != HD) return MINF_ERR_UNSUPPORTED;
     if (t->dtype != MINF_BF16 && t->dtype != MINF_F16) return MINF_ERR_UNSUPPORTED;
     const void *ptrs[4] = {t->q, t->k, t->v, t->o};
@@ -740,20 +944,23 @@ void fill_params(AttnParams &p, const minf_qkvo *t) {
     p.bc = p.bo = p.cc = p.ci = nullptr; p.nnz_s = p.nnz_v = 0;
     p.bidx = nullptr; p.max_blocks = 0; p.bidx_rows = 0;
     p.n_init = p.n_local = 0; p.dense_from = 0x7fffffff;
-    p.total_wg = (long long)t->batch * t->heads_q * p.rows;
+    p.head_list = t->head_list;
+    p.index_heads = t->head_list ? t->index_heads : t->heads_q;
+    p.total_wg = 0;          // set by the launcher
     p.descending = 0;
-    p.head_slot = t->head_slot;
-    p.index_heads = t->head_slot ? t->index_heads : t->heads_q;
 }
 
 template <int MODE> int launch(AttnParams p, int dtype, void *stream) {
-    if (p.total_wg == 0) return MINF_OK;
-    // vertical-slash lists (blocks + gathered columns per row block) run on the 2-wave kernel,
-    // everything else on the paired one -- except block lists too long for the paired walk's LDS copy
-    constexpr bool CAN_PAIR = MODE != MODE_VS;
-    constexpr bool CAN_SINGLE = MODE == MODE_VS || MODE == MODE_BS;
+    if (p.batch == 0 || p.rows == 0) return MINF_OK;
+    // every mode runs on the paired (4-wave) kernel, except block-sparse lists that are too long for
+    // the paired walk's LDS copy: those run on the 2-wave kernel
+    constexpr bool CAN_PAIR = true;
+    constexpr bool CAN_SINGLE = MODE == MODE_BS;
     const bool pair = CAN_PAIR && (MODE != MODE_BS || p.max_blocks <= BS_PAIR_MAX);
-    if (pair) p.total_wg = (long long)p.batch * p.hq * ((p.rows + 1) / 2);
+    // heads of the grid: all of them, or the selected ones rounded up to whole chunks of hq / hk
+    const int group = p.hq / p.hk;
+    const long long grid_heads = p.head_list ? (long long)((p.index_heads + group - 1) / group) * group : p.hq;
+    p.total_wg = (long long)p.batch * grid_heads * (pair ? (p.rows + 1) / 2 : p.rows);
     p.descending = MODE == MODE_DENSE || (MODE == MODE_VS && p.rows <= 1024);
     const long long per_xcd = (p.total_wg + 7) >> 3;
     const long long grid = per_xcd * 8;

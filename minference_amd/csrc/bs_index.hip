@@ -38,9 +38,9 @@ struct PoolParams {
     float *out;               // [batch*heads, rows, 128] fp32
     int heads, n, rows;
     int blk;                  // tokens per block: 64 or 32
-    // optional head selection: head_slot[h] < 0 skips head h, otherwise it is the head's position in
-    // `out`, which then has out_heads heads (= heads without it)
-    const int *head_slot;
+    // optional head selection: `out` has out_heads heads and head i of it is head head_list[i] of x
+    // (without a list: out_heads = heads, same numbering)
+    const int *head_list;
     int out_heads;
 };
 
@@ -58,12 +58,8 @@ template <typename T> __global__ __launch_bounds__(256) void bs_pool_kernel(cons
     __shared__ float red[16][HD + 4];
     const int blk = blockIdx.x;
     const int bh = blockIdx.y;
-    const int b = bh / p.heads, h = bh % p.heads;
-    int slot = h;
-    if (p.head_slot) {
-        slot = p.head_slot[h];
-        if (slot < 0) return;
-    }
+    const int b = bh / p.out_heads, slot = bh % p.out_heads;      // (grid: batch x out_heads)
+    const int h = p.head_list ? p.head_list[slot] : slot;
     const int tid = (int)threadIdx.x;
     const int c = tid & 15, r4 = tid >> 4;
     const char *base = p.x + ((long long)b * p.xs[0] + (long long)h * p.xs[1]) * 2;
@@ -99,7 +95,7 @@ struct ScoreParams {
     int heads_q, heads_kv, rows, pitch, force;
     int mtiles, ntiles;
     int skip_masked;
-    const int *head_slot;     // as in PoolParams; qp and scores have index_heads heads
+    const int *head_list;     // as in PoolParams; qp and scores have index_heads heads
     int index_heads;
 };
 
@@ -116,14 +112,10 @@ __global__ __launch_bounds__(256) void bs_scores_kernel(const ScoreParams p) {
     const int l32 = lane & 31, g = lane >> 5;
     const int mt = p.mtiles - 1 - (int)blockIdx.x;            // heavy (late) query tiles first
     const int bh = blockIdx.y;
-    const int b = bh / p.heads_q, h = bh % p.heads_q;
+    const int b = bh / p.index_heads, slot = bh % p.index_heads;   // (grid: batch x index_heads)
+    const int h = p.head_list ? p.head_list[slot] : slot;
     const int hkv = h / (p.heads_q / p.heads_kv);
-    int slot = h;
-    if (p.head_slot) {
-        slot = p.head_slot[h];
-        if (slot < 0) return;
-    }
-    const long long bs = (long long)b * p.index_heads + slot;
+    const long long bs = bh;
     const float *qbase = p.qp + bs * p.rows * HD;
     const float *kbase = p.kp + ((long long)b * p.heads_kv + hkv) * p.rows * HD;
     float *out = p.scores + bs * p.rows * p.pitch;
@@ -179,10 +171,10 @@ namespace {
 int block_index_impl(const void *q, const void *k, const int64_t *q_stride, const int64_t *k_stride, int batch,
                      int heads_q, int heads_kv, int n, int head_dim, int dtype, int blk, int rows, int top_k,
                      int force_diag_first, int32_t *block_index, void *workspace, size_t workspace_bytes,
-                     void *stream, const int32_t *head_slot = nullptr, int index_heads = 0) {
+                     void *stream, const int32_t *head_list = nullptr, int index_heads = 0) {
     if (!q || !k || !q_stride || !k_stride || !block_index) return MINF_ERR_INVALID_ARG;
-    if (head_slot && index_heads <= 0) return MINF_ERR_INVALID_ARG;
-    if (!head_slot) index_heads = heads_q;
+    if (head_list && index_heads <= 0) return MINF_ERR_INVALID_ARG;
+    if (!head_list) index_heads = heads_q;
     if (batch < 0 || heads_q <= 0 || heads_kv <= 0 || n <= 0 || top_k <= 0) return MINF_ERR_INVALID_ARG;
     if (heads_q % heads_kv != 0) return MINF_ERR_INVALID_ARG;
     if (head_dim != HD) return MINF_ERR_UNSUPPORTED;
@@ -194,7 +186,7 @@ int block_index_impl(const void *q, const void *k, const int64_t *q_stride, cons
     const size_t need = workspace_for(batch, index_heads, heads_kv, rows);
     if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 15)) return MINF_ERR_WORKSPACE;
     const int pitch = score_pitch(rows);
-    if ((long long)batch * index_heads * rows > 0x7fffffffLL || (long long)batch * heads_q > 65535) return MINF_ERR_UNSUPPORTED;
+    if ((long long)batch * index_heads * rows > 0x7fffffffLL || (long long)batch * index_heads > 65535) return MINF_ERR_UNSUPPORTED;
 
     char *ws = (char *)workspace;
     float *qp = (float *)ws;
@@ -204,13 +196,13 @@ int block_index_impl(const void *q, const void *k, const int64_t *q_stride, cons
     float *scores = (float *)ws;
     hipStream_t st = (hipStream_t)stream;
 
-    PoolParams pq{(const char *)q, {q_stride[0], q_stride[1], q_stride[2]}, qp, heads_q, n, rows, blk, head_slot, index_heads};
+    PoolParams pq{(const char *)q, {q_stride[0], q_stride[1], q_stride[2]}, qp, heads_q, n, rows, blk, head_list, index_heads};
     PoolParams pk{(const char *)k, {k_stride[0], k_stride[1], k_stride[2]}, kp, heads_kv, n, rows, blk, nullptr, heads_kv};
     if (dtype == MINF_BF16) {
-        hipLaunchKernelGGL(bs_pool_kernel<__bf16>, dim3(rows, batch * heads_q), dim3(256), 0, st, pq);
+        hipLaunchKernelGGL(bs_pool_kernel<__bf16>, dim3(rows, batch * index_heads), dim3(256), 0, st, pq);
         hipLaunchKernelGGL(bs_pool_kernel<__bf16>, dim3(rows, batch * heads_kv), dim3(256), 0, st, pk);
     } else {
-        hipLaunchKernelGGL(bs_pool_kernel<_Float16>, dim3(rows, batch * heads_q), dim3(256), 0, st, pq);
+        hipLaunchKernelGGL(bs_pool_kernel<_Float16>, dim3(rows, batch * index_heads), dim3(256), 0, st, pq);
         hipLaunchKernelGGL(bs_pool_kernel<_Float16>, dim3(rows, batch * heads_kv), dim3(256), 0, st, pk);
     }
     int status = minf_launch_status();
@@ -218,8 +210,8 @@ int block_index_impl(const void *q, const void *k, const int64_t *q_stride, cons
 
     const bool causal_topk = rows <= 64 * 64;      // one wave per row: reads only the stored prefix of a row
     ScoreParams sp{qp, kp, scores, heads_q, heads_kv, rows, pitch, force_diag_first ? 1 : 0,
-                   (rows + 31) / 32, (pitch + 31) / 32, causal_topk ? 1 : 0, head_slot, index_heads};
-    hipLaunchKernelGGL(bs_scores_kernel, dim3(sp.mtiles, batch * heads_q), dim3(256), 0, st, sp);
+                   (rows + 31) / 32, (pitch + 31) / 32, causal_topk ? 1 : 0, head_list, index_heads};
+    hipLaunchKernelGGL(bs_scores_kernel, dim3(sp.mtiles, batch * index_heads), dim3(256), 0, st, sp);
     status = minf_launch_status();
     if (status != MINF_OK) return status;
 
@@ -249,13 +241,13 @@ extern "C" int minf_bs_block_index(const void *q, const void *k, const int64_t *
 extern "C" int minf_bs_block_index_heads(const void *q, const void *k, const int64_t *q_stride,
                                          const int64_t *k_stride, int batch, int heads_q, int heads_kv,
                                          int n, int head_dim, int dtype, int top_k, int force_diag_first,
-                                         const int32_t *head_slot, int index_heads,
+                                         const int32_t *head_list, int index_heads,
                                          int32_t *block_index, void *workspace, size_t workspace_bytes,
                                          void *stream) {
-    if (!head_slot) return MINF_ERR_INVALID_ARG;
+    if (!head_list) return MINF_ERR_INVALID_ARG;
     return block_index_impl(q, k, q_stride, k_stride, batch, heads_q, heads_kv, n, head_dim, dtype, BLK,
                             n > 0 ? padded_rows(n) : 0, top_k, force_diag_first, block_index, workspace,
-                            workspace_bytes, stream, head_slot, index_heads);
+                            workspace_bytes, stream, head_list, index_heads);
 }
 extern "C" size_t minf_search_block_index_workspace_bytes(int batch, int heads_q, int heads_kv, int n) {
     if (batch <= 0 || heads_q <= 0 || heads_kv <= 0 || n <= 0) return 0;

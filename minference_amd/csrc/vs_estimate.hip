@@ -49,9 +49,9 @@ struct EstParams {
     float *vertical, *slash;    // [B, Hq, N]
     int force_v, force_s;
     long long total_wg;
-    // optional head selection: head_slot[h] < 0 skips query head h, otherwise it is the head's
-    // position in the outputs and the workspace, which have index_heads heads (= hq without it)
-    const int *head_slot;
+    // optional head selection: head_list[i], i < index_heads, are the query heads to score and i is
+    // the head's position in the outputs and the workspace (index_heads = hq without a list)
+    const int *head_list;
     int index_heads;
 };
 
@@ -81,13 +81,19 @@ __device__ __forceinline__ WgId decode_wg(const EstParams &p) {
     long long rest = logical;
     const int hin = (int)(rest % group); rest /= group;
     w.chunk = (int)(rest % p.nchunks); rest /= p.nchunks;
-    w.hkv = (int)(rest % p.hk);
-    w.b = (int)(rest / p.hk);
-    w.h = w.hkv * group + hin;
-    w.slot = w.h;
-    if (w.valid && p.head_slot) {
-        w.slot = p.head_slot[w.h];
-        w.valid = w.slot >= 0;
+    if (p.head_list) {
+        // chunks of `group` consecutive list entries take the place of the kv groups
+        const int nch = (p.index_heads + group - 1) / group;
+        w.slot = (int)(rest % nch) * group + hin;
+        w.b = (int)(rest / nch);
+        w.valid = w.valid && w.slot < p.index_heads;
+        w.h = w.valid ? p.head_list[w.slot] : 0;
+        w.hkv = w.h / group;
+    } else {
+        w.hkv = (int)(rest % p.hk);
+        w.b = (int)(rest / p.hk);
+        w.h = w.hkv * group + hin;
+        w.slot = w.h;
     }
     return w;
 }
@@ -341,10 +347,10 @@ __global__ __launch_bounds__(256) void est_finalize_kernel(const EstParams p) {
 int fill(EstParams &p, const void *q, const void *k, const int64_t *q_stride, const int64_t *k_stride,
          int batch, int heads_q, int heads_kv, int n, int head_dim, int dtype, float sm_scale,
          int last_q, int force_v, int force_s, float *vertical, float *slash, void *ws, size_t ws_bytes,
-         const int32_t *head_slot, int index_heads) {
+         const int32_t *head_list, int index_heads) {
     if (!q || !k || !vertical || !slash || !ws) return MINF_ERR_INVALID_ARG;
-    if (head_slot && index_heads <= 0) return MINF_ERR_INVALID_ARG;
-    if (!head_slot) index_heads = heads_q;
+    if (head_list && index_heads <= 0) return MINF_ERR_INVALID_ARG;
+    if (!head_list) index_heads = heads_q;
     if (batch < 0 || heads_q <= 0 || heads_kv <= 0 || n <= 0 || heads_q % heads_kv) return MINF_ERR_INVALID_ARG;
     if (head_dim != HD || (dtype != MINF_BF16 && dtype != MINF_F16)) return MINF_ERR_UNSUPPORTED;
     if (last_q < 1 || last_q > LQ || force_v < 0 || force_s < 0) return MINF_ERR_INVALID_ARG;
@@ -368,8 +374,10 @@ int fill(EstParams &p, const void *q, const void *k, const int64_t *q_stride, co
     p.win = (float *)((char *)ws + stats_b + row_b);
     p.vertical = vertical; p.slash = slash;
     p.force_v = force_v; p.force_s = force_s;
-    p.total_wg = (long long)batch * heads_q * p.nchunks;
-    p.head_slot = head_slot;
+    const int group = heads_q / heads_kv;
+    const long long grid_heads = head_list ? (long long)((index_heads + group - 1) / group) * group : heads_q;
+    p.total_wg = (long long)batch * grid_heads * p.nchunks;
+    p.head_list = head_list;
     p.index_heads = index_heads;
     return MINF_OK;
 }
@@ -386,13 +394,13 @@ extern "C" size_t minf_vs_estimate_workspace_bytes(int batch, int heads_q, int n
 static int estimate_launch(const void *q, const void *k, const int64_t *q_stride, const int64_t *k_stride,
                            int batch, int heads_q, int heads_kv, int n, int head_dim, int dtype, float sm_scale,
                            int last_q, int force_vertical, int force_slash, float *vertical, float *slash,
-                           void *workspace, size_t workspace_bytes, const int32_t *head_slot, int index_heads,
+                           void *workspace, size_t workspace_bytes, const int32_t *head_list, int index_heads,
                            void *stream) {
     EstParams p;
     if (batch == 0) return MINF_OK;
     int st = fill(p, q, k, q_stride, k_stride, batch, heads_q, heads_kv, n, head_dim, dtype, sm_scale,
                   last_q, force_vertical, force_slash, vertical, slash, workspace, workspace_bytes,
-                  head_slot, index_heads);
+                  head_list, index_heads);
     if (st) return st;
     const long long grid = ((p.total_wg + 7) >> 3) * 8;
     if (grid > 0x7fffffffLL) return MINF_ERR_UNSUPPORTED;
@@ -419,11 +427,11 @@ extern "C" int minf_vs_estimate(const void *q, const void *k, const int64_t *q_s
 extern "C" int minf_vs_estimate_heads(const void *q, const void *k, const int64_t *q_stride,
                                       const int64_t *k_stride, int batch, int heads_q, int heads_kv, int n,
                                       int head_dim, int dtype, float sm_scale, int last_q, int force_vertical,
-                                      int force_slash, const int32_t *head_slot, int index_heads,
+                                      int force_slash, const int32_t *head_list, int index_heads,
                                       float *vertical, float *slash, void *workspace,
                                       size_t workspace_bytes, void *stream) {
-    if (!head_slot) return MINF_ERR_INVALID_ARG;
+    if (!head_list) return MINF_ERR_INVALID_ARG;
     return estimate_launch(q, k, q_stride, k_stride, batch, heads_q, heads_kv, n, head_dim, dtype, sm_scale, last_q,
-                           force_vertical, force_slash, vertical, slash, workspace, workspace_bytes, head_slot,
+                           force_vertical, force_slash, vertical, slash, workspace, workspace_bytes, head_list,
                            index_heads, stream);
 }

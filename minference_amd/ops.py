@@ -106,14 +106,14 @@ class _Call:
     def ref(self):
         return ctypes.byref(self.struct)
 
-    def select_heads(self, head_slot=None, index_heads=0):
-        """Restrict the following launches to the query heads h with head_slot[h] >= 0 (int32
-        [heads_q] on the device; that value is the head's position in index tensors that have
-        index_heads heads).  None = all heads again.  The output buffer is shared, so one launch
-        per pattern type fills its heads in place."""
-        self._head_slot = head_slot                       # keeps the tensor alive
-        self.struct.head_slot = head_slot.data_ptr() if head_slot is not None else None
-        self.struct.index_heads = int(index_heads) if head_slot is not None else 0
+    def select_heads(self, head_list=None):
+        """Restrict the following launches to the query heads in head_list (int32 device tensor of
+        distinct head numbers; head_list[i] reads head position i of the index tensors).  None = all
+        heads again.  The output buffer is shared, so one launch per pattern type fills its heads in
+        place."""
+        self._head_list = head_list                       # keeps the tensor alive
+        self.struct.head_list = head_list.data_ptr() if head_list is not None else None
+        self.struct.index_heads = int(head_list.numel()) if head_list is not None else 0
 
     def result(self):
         o = self.o

@@ -58,11 +58,9 @@ def _head_plan(config, layer_idx, num_heads):
 VERTICAL_PAD = 0x3FFFFFFF      # a vertical index no range ever reaches: never emitted by the index builder
 
 
-def _slot_tensor(heads, num_heads, device):
-    """int32 [num_heads]: position of head h in ``heads`` or -1."""
-    slot = torch.full((num_heads,), -1, dtype=torch.int32)
-    slot[torch.as_tensor(heads, dtype=torch.long)] = torch.arange(len(heads), dtype=torch.int32)
-    return slot.to(device)
+def _head_list(heads, device):
+    """int32 device tensor of the (ascending) query head numbers of one pattern group."""
+    return torch.tensor(sorted(heads), dtype=torch.int32).to(device)
 
 
 def _mixed_layer(query_states, key_states, value_states, plan):
@@ -109,7 +107,7 @@ def _mixed_layer(query_states, key_states, value_states, plan):
             kv = [min(N, max(int(v), 30)) for _, v, _ in vs]
             ksl = [min(N, max(int(s), 50)) for _, _, s in vs]
             vmax, smax = max(kv), max(ksl)
-            slot = _slot_tensor(heads, H, dev)
+            slot = _head_list(heads, dev)
             vertical = torch.empty((B, nh, N), dtype=torch.float32, device=dev)
             slash = torch.empty((B, nh, N), dtype=torch.float32, device=dev)
             ws_bytes = lib.minf_vs_estimate_workspace_bytes(B, nh, N)
@@ -130,7 +128,7 @@ def _mixed_layer(query_states, key_states, value_states, plan):
             seqlens = torch.full((B,), N, dtype=torch.int32, device=dev)
             bc, bo, cc, ci = convert_vertical_slash_indexes(seqlens, v_idx, s_idx, N, 64, 64, zero_fill=False)
             c.struct.seqlens = seqlens.data_ptr()
-            c.select_heads(slot, nh)
+            c.select_heads(slot)
             st = lib.minf_vs_attn_fwd(c.ref, bc.data_ptr(), bo.data_ptr(), cc.data_ptr(), ci.data_ptr(), rows,
                                       smax, vmax, stream)
             _lib.check(st, "minf_vs_attn_fwd")
@@ -138,7 +136,7 @@ def _mixed_layer(query_states, key_states, value_states, plan):
             keep += [slot, vertical, slash, ws, kv_t, ks_t, v_idx, s_idx, seqlens, bc, bo, cc, ci]
         if bs:
             nh = len(bs)
-            slot = _slot_tensor(bs, H, dev)
+            slot = _head_list(bs, dev)
             brows = lib.minf_bs_block_index_rows(N)
             kk = min(100, brows)                          # top_k fixed at 100 (:616-618)
             ws_bytes = lib.minf_bs_block_index_workspace_bytes(B, nh, c.Hk, N)
@@ -148,13 +146,13 @@ def _mixed_layer(query_states, key_states, value_states, plan):
                                                c.struct.dtype, 100, 0, slot.data_ptr(), nh, bi.data_ptr(),
                                                ws.data_ptr(), ws_bytes, stream)
             _lib.check(st, "minf_bs_block_index_heads")
-            c.select_heads(slot, nh)
+            c.select_heads(slot)
             st = lib.minf_bs_attn_fwd(c.ref, bi.data_ptr(), brows, kk, stream)
             _lib.check(st, "minf_bs_attn_fwd")
             keep += [slot, ws, bi]
         for (n_init, n_local), hs in st_groups.items():
-            slot = _slot_tensor(sorted(hs), H, dev)
-            c.select_heads(slot, len(hs))
+            slot = _head_list(hs, dev)
+            c.select_heads(slot)
             if N > 0:
                 st = lib.minf_ashape_attn_fwd(c.ref, int(n_init), int(n_local), stream)
                 _lib.check(st, "minf_ashape_attn_fwd")

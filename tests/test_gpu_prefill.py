@@ -114,7 +114,7 @@ def test_ragged_per_head_sizes_one_launch_chain_per_type(gpu, monkeypatch):
 
 
 def test_head_selection_leaves_other_heads_untouched(gpu):
-    """minf_qkvo.head_slot through the C ABI: a dense launch restricted to heads {1, 4, 5} of 6 writes
+    """minf_qkvo.head_list through the C ABI: a dense launch restricted to heads {1, 4, 5} of 6 writes
     exactly those heads of the output buffer and reproduces the unrestricted launch on them."""
     import ctypes
     from minference_amd import _lib
@@ -127,8 +127,7 @@ def test_head_selection_leaves_other_heads_untouched(gpu):
     assert lib.minf_dense_attn_fwd(full.ref, _lib.stream_ptr(gpu)) == 0
     part = _Call(q, k, v)
     part.o.fill_(-3.0)
-    slot = torch.tensor([-1, 0, -1, -1, 1, 2], dtype=torch.int32, device=gpu)
-    part.select_heads(slot, 3)
+    part.select_heads(torch.tensor([1, 4, 5], dtype=torch.int32, device=gpu))
     assert lib.minf_dense_attn_fwd(part.ref, _lib.stream_ptr(gpu)) == 0
     torch.cuda.synchronize()
     for h in range(hq):
@@ -136,7 +135,7 @@ def test_head_selection_leaves_other_heads_untouched(gpu):
             assert torch.equal(part.o[:, h], full.o[:, h])
         else:
             assert (part.o[:, h] == -3.0).all()
-    # a selection without a slot count is refused
+    # a list without a length is refused
     part.struct.index_heads = 0
     assert lib.minf_dense_attn_fwd(part.ref, _lib.stream_ptr(gpu)) == -1
 

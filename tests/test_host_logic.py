@@ -31,11 +31,11 @@ def test_minference_ratio_truncates_like_the_reference():
     assert list(plan) == [("vertical_and_slash", int(1000 * 0.33), int(6096 * 0.33))]
 
 
-def test_head_slot_tensor_of_a_pattern_group():
-    # position of every selected head in the group's index tensors, -1 for all other heads
-    slot = prefill._slot_tensor([1, 4, 5], 8, "cpu")
-    assert slot.dtype == torch.int32 and slot.tolist() == [-1, 0, -1, -1, 1, 2, -1, -1]
-    assert prefill._slot_tensor([], 3, "cpu").tolist() == [-1, -1, -1]
+def test_head_list_of_a_pattern_group():
+    # the ascending head numbers of a group: entry i is the head that owns index position i
+    hl = prefill._head_list([5, 1, 4], "cpu")
+    assert hl.dtype == torch.int32 and hl.tolist() == [1, 4, 5]
+    assert prefill._head_list([], "cpu").numel() == 0
 
 
 def test_search_mode_has_no_cpu_path_and_respects_a_finished_file(tmp_path):
