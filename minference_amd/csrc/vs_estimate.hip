@@ -19,6 +19,13 @@
 //            conflict-free strided reads (no atomics); the per-chunk window is written out whole;
 //   finalize: stitch the chunk windows together (each diagonal gets at most two
 //            pieces, added in a fixed order) and apply the forced +inf entries.
+// Work split: a workgroup owns one 2048-key chunk of one group of up to four query heads that are
+// neighbours in head order (with grouped-query attention: heads that read the same K): wave w
+// scores head w % gw over key sub-range w / gw of the chunk (gw = heads per workgroup: 4, 2 or 1),
+// so the K fragments that the four waves fetch are the same cache lines at the same time -- one
+// trip to L2/HBM per kv head instead of one per query head.  The second sweep hands out its
+// workgroups in the reverse order of the first, so that it starts on the K chunks that the first
+// sweep touched last and finds part of K still cached.
 // All arithmetic is fp32 on 16-bit inputs (the reference rounds q.k to bf16
 // before its fp32 softmax).
 #include "minf_common.h"
@@ -53,6 +60,8 @@ struct EstParams {
     // the head's position in the outputs and the workspace (index_heads = hq without a list)
     const int *head_list;
     int index_heads;
+    int gw;                     // query heads per workgroup (waves w % gw), 4 / gw key sub-ranges each
+    int nhc;                    // head groups: ceil(index_heads / gw)
 };
 
 union Frag {
@@ -69,32 +78,27 @@ template <> __device__ __forceinline__ f32x16_t mma<_Float16>(const Frag &a, con
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a.h, b.h, c, 0, 0, 0);
 }
 
-struct WgId { int b, h, hkv, chunk, slot; bool valid; };
+struct WgId { int b, h, hkv, chunk, slot, kq; bool valid, wave_valid; };
 
-// XCD-aware order: (batch, kv head, chunk, query head in group) contiguous per XCD
-__device__ __forceinline__ WgId decode_wg(const EstParams &p) {
+// Workgroup order: (batch, head group, chunk), contiguous per XCD: the chunks of one head group --
+// i.e. of (mostly) one kv head -- are swept by consecutive workgroups of one XCD.  `reverse` flips
+// the order (second sweep).  Wave `wave` of the workgroup gets head hc * gw + wave % gw.
+__device__ __forceinline__ WgId decode_wg(const EstParams &p, int wave, bool reverse) {
     WgId w;
     const long long per_xcd = (p.total_wg + 7) >> 3;
-    const long long logical = (long long)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    long long logical = (long long)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
     w.valid = logical < p.total_wg;
+    if (reverse) logical = p.total_wg - 1 - logical;
     const int group = p.hq / p.hk;
     long long rest = logical;
-    const int hin = (int)(rest % group); rest /= group;
     w.chunk = (int)(rest % p.nchunks); rest /= p.nchunks;
-    if (p.head_list) {
-        // chunks of `group` consecutive list entries take the place of the kv groups
-        const int nch = (p.index_heads + group - 1) / group;
-        w.slot = (int)(rest % nch) * group + hin;
-        w.b = (int)(rest / nch);
-        w.valid = w.valid && w.slot < p.index_heads;
-        w.h = w.valid ? p.head_list[w.slot] : 0;
-        w.hkv = w.h / group;
-    } else {
-        w.hkv = (int)(rest % p.hk);
-        w.b = (int)(rest / p.hk);
-        w.h = w.hkv * group + hin;
-        w.slot = w.h;
-    }
+    const int hc = (int)(rest % p.nhc);
+    w.b = (int)(rest / p.nhc);
+    w.kq = wave / p.gw;
+    w.slot = hc * p.gw + wave % p.gw;
+    w.wave_valid = w.valid && w.slot < p.index_heads;
+    w.h = w.wave_valid ? (p.head_list ? p.head_list[w.slot] : w.slot) : 0;
+    w.hkv = w.h / group;
     return w;
 }
 
@@ -125,22 +129,23 @@ __device__ __forceinline__ void load_k(const EstParams &p, const char *kb, int c
 template <typename T>
 __global__ __launch_bounds__(EST_THREADS, 3) void est_stats_kernel(const EstParams p) {
     __shared__ float lds_m[4][LQ], lds_l[4][LQ];
-    const WgId w = decode_wg(p);
-    if (!w.valid) return;
     const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const WgId w = decode_wg(p, wave, false);
+    if (!w.valid) return;
     const int l32 = lane & 31, g = lane >> 5;
-    const char *kb = p.k + ((long long)w.b * p.ks[0] + (long long)w.hkv * p.ks[1]) * 2;
-
-    Frag qf[2][8];
-    load_q(p, w, lane, qf);
+    const int nq = 4 / p.gw, klen = KC / nq;          // key sub-ranges per head, keys per wave
 
     // lane <-> query rows i = l32 and 32 + l32; regs <-> keys 8*(r/4) + 4*g + r%4 of the block
     float m_run[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.f, 0.f};
-    const int key_begin = w.chunk * KC + wave * (KC / 4);
+    if (w.wave_valid) {
+    const char *kb = p.k + ((long long)w.b * p.ks[0] + (long long)w.hkv * p.ks[1]) * 2;
+    Frag qf[2][8];
+    load_q(p, w, lane, qf);
+    const int key_begin = w.chunk * KC + w.kq * klen;
     const int qpos0 = p.n - p.last_q;          // absolute position of query row 0
     Frag kf[8], kn[8];
     load_k(p, kb, key_begin, lane, kn);
-    for (int blk = 0; blk < KC / 4 / 32; ++blk) {
+    for (int blk = 0; blk < klen / 32; ++blk) {
         const int c0 = key_begin + blk * 32;
         if (c0 >= p.n) break;
 #pragma unroll
@@ -164,10 +169,10 @@ __global__ __launch_bounds__(EST_THREADS, 3) void est_stats_kernel(const EstPara
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int tkc = 8 * (r >> 2) + (r & 3);
-                float s = st[nb][r] * p.scale_log2;
-                if (edge) s = (tkc <= hi) ? s : -INFINITY;
-                st[nb][r] = s;
-                mx = fmaxf(mx, s);
+                float sc = st[nb][r] * p.scale_log2;
+                if (edge) sc = (tkc <= hi) ? sc : -INFINITY;
+                st[nb][r] = sc;
+                mx = fmaxf(mx, sc);
             }
             const float m_new = fmaxf(m_run[nb], mx);
             const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
@@ -178,7 +183,8 @@ __global__ __launch_bounds__(EST_THREADS, 3) void est_stats_kernel(const EstPara
             m_run[nb] = m_new;
         }
     }
-    // merge the two lane halves, then the 4 waves
+    }
+    // merge the two lane halves, then the waves that share a head
 #pragma unroll
     for (int nb = 0; nb < 2; ++nb) {
         const float mo = __shfl_xor(m_run[nb], 32), lo = __shfl_xor(l_run[nb], 32);
@@ -192,19 +198,23 @@ __global__ __launch_bounds__(EST_THREADS, 3) void est_stats_kernel(const EstPara
         }
     }
     __syncthreads();
-    if (tid < LQ) {
-        float m = lds_m[0][tid], l = lds_l[0][tid];
-#pragma unroll
-        for (int wv = 1; wv < 4; ++wv) {
-            const float mo = lds_m[wv][tid], lo = lds_l[wv][tid];
-            const float m_new = fmaxf(m, mo);
-            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-            l = l * __builtin_amdgcn_exp2f(m - m_use) + lo * __builtin_amdgcn_exp2f(mo - m_use);
-            m = m_new;
+    // thread (hsub, row): the nq waves hsub, hsub + gw, ... hold the pieces of head hsub's row
+    const int hsub = tid / LQ, row = tid % LQ;
+    if (hsub < p.gw) {
+        const WgId wh = decode_wg(p, hsub, false);
+        if (wh.wave_valid) {
+            float m = lds_m[hsub][row], l = lds_l[hsub][row];
+            for (int kq = 1; kq < nq; ++kq) {
+                const float mo = lds_m[kq * p.gw + hsub][row], lo = lds_l[kq * p.gw + hsub][row];
+                const float m_new = fmaxf(m, mo);
+                const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+                l = l * __builtin_amdgcn_exp2f(m - m_use) + lo * __builtin_amdgcn_exp2f(mo - m_use);
+                m = m_new;
+            }
+            float *dst = p.stats + ((((long long)wh.b * p.index_heads + wh.slot) * p.nchunks + wh.chunk) * LQ + row) * 2;
+            dst[0] = m;
+            dst[1] = l;
         }
-        float *dst = p.stats + ((((long long)w.b * p.index_heads + w.slot) * p.nchunks + w.chunk) * LQ + tid) * 2;
-        dst[0] = m;
-        dst[1] = l;
     }
 }
 
@@ -233,7 +243,7 @@ __global__ __launch_bounds__(LQ) void est_reduce_kernel(const EstParams p) {
 // private per-wave window with plain read-modify-write (one wave, in-order LDS: no race).
 constexpr int TP = 33;                       // tile row pitch (floats)
 constexpr int TROWS = 94;                    // 32 rows of a half block, 31 zero rows above, 31 below
-constexpr int WWIN = KC / 4 + LQ;            // per-wave diagonal window (a quarter of the chunk + 64)
+constexpr int WWIN = KC + LQ;                // per-wave diagonal window: at most the whole chunk + 64
 
 // (min 2 waves per SIMD: caps the kernel at 256 registers; it is latency bound and one resident
 // wave per SIMD ran 1.4x slower)
@@ -242,19 +252,22 @@ __global__ __launch_bounds__(EST_THREADS, 2) void est_scores_kernel(const EstPar
     // the four waves' tiles overlap in their zero rows: wave w starts 63 rows after wave w-1
     __shared__ float lds_tile[(3 * 63 + TROWS) * TP];
     __shared__ float lds_wwin[4][WWIN];
-    const WgId w = decode_wg(p);
-    if (!w.valid) return;
     const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const WgId w = decode_wg(p, wave, true);
+    if (!w.valid) return;
     const int l32 = lane & 31, g = lane >> 5;
-    const char *kb = p.k + ((long long)w.b * p.ks[0] + (long long)w.hkv * p.ks[1]) * 2;
+    const int nq = 4 / p.gw, klen = KC / nq;          // key sub-ranges per head, keys per wave
+    const int wwin_len = klen + LQ;
     const long long bh = (long long)w.b * p.index_heads + w.slot;
     float *tile = lds_tile + wave * 63 * TP;
     float *wwin = lds_wwin[wave];
 
-    for (int i = lane; i < WWIN; i += 64) wwin[i] = 0.f;
+    for (int i = lane; i < wwin_len; i += 64) wwin[i] = 0.f;
     for (int i = tid; i < (3 * 63 + TROWS) * TP; i += EST_THREADS) lds_tile[i] = 0.f;
     __syncthreads();
 
+    if (w.wave_valid) {
+    const char *kb = p.k + ((long long)w.b * p.ks[0] + (long long)w.hkv * p.ks[1]) * 2;
     Frag qf[2][8];
     load_q(p, w, lane, qf);
     // lane <-> key; reg r of block mb <-> query row i = 32*mb + 8*(r/4) + 4*g + r%4
@@ -265,14 +278,13 @@ __global__ __launch_bounds__(EST_THREADS, 2) void est_scores_kernel(const EstPar
         for (int r = 0; r < 16; ++r)
             mrow[mb][r] = p.rowstat[bh * LQ + 32 * mb + 8 * (r >> 2) + 4 * g + (r & 3)];
 
-    const int chunk0 = w.chunk * KC;
-    const int key_begin = chunk0 + wave * (KC / 4);
+    const int key_begin = w.chunk * KC + w.kq * klen;
     const int qpos0 = p.n - p.last_q;
     const int rshift = LQ - p.last_q;          // rows are indexed as if last_q were 64
     float *vout = p.vertical + bh * p.n;
     Frag kf[8], kn[8];
     load_k(p, kb, key_begin, lane, kn);
-    for (int blk = 0; blk < KC / 4 / 32; ++blk) {
+    for (int blk = 0; blk < klen / 32; ++blk) {
         const int c0 = key_begin + blk * 32;
         if (c0 >= p.n) break;
 #pragma unroll
@@ -283,16 +295,16 @@ __global__ __launch_bounds__(EST_THREADS, 2) void est_scores_kernel(const EstPar
         float colsum = 0.f;
 #pragma unroll
         for (int mb = 0; mb < 2; ++mb) {
-            f32x16_t s;
+            f32x16_t sc;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) s[r] = 0.f;
+            for (int r = 0; r < 16; ++r) sc[r] = 0.f;
 #pragma unroll
-            for (int ks = 0; ks < 8; ++ks) s = mma<T>(qf[mb][ks], kf[ks], s);
+            for (int ks = 0; ks < 8; ++ks) sc = mma<T>(qf[mb][ks], kf[ks], sc);
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int il = 8 * (r >> 2) + 4 * g + (r & 3);      // row inside this 32-row half
                 const int i = 32 * mb + il;
-                float pr = __builtin_amdgcn_exp2f(fmaf(s[r], p.scale_log2, -mrow[mb][r]));
+                float pr = __builtin_amdgcn_exp2f(fmaf(sc[r], p.scale_log2, -mrow[mb][r]));
                 if (edge) pr = (c <= qpos0 + i && c < p.n) ? pr : 0.f;
                 colsum += pr;
                 tile[(31 + il) * TP + l32] = pr;
@@ -314,17 +326,20 @@ __global__ __launch_bounds__(EST_THREADS, 2) void est_scores_kernel(const EstPar
         colsum += __shfl_xor(colsum, 32);
         if (g == 0 && c < p.n) vout[c] = colsum;
     }
+    }
     __syncthreads();
-    // chunk window position q = (key - chunk0) + (last_q - 1 - i): wave wv contributes its slot q - 64*4*wv/4...
-    float *wout = p.win + (bh * p.nchunks + w.chunk) * WIN;
-    for (int q = tid; q < WIN; q += EST_THREADS) {
+    // chunk window of head hsub, position q = (key - chunk0) + (last_q - 1 - i): wave kq * gw + hsub
+    // contributes its slot q - kq * klen
+    for (int idx = tid; idx < p.gw * WIN; idx += EST_THREADS) {
+        const int hsub = idx / WIN, q = idx - hsub * WIN;
+        const WgId wh = decode_wg(p, hsub, true);
+        if (!wh.wave_valid) continue;
         float acc = 0.f;
-#pragma unroll
-        for (int wv = 0; wv < 4; ++wv) {
-            const int sl = q - wv * (KC / 4);
-            if (sl >= 0 && sl < WWIN) acc += lds_wwin[wv][sl];
+        for (int kq = 0; kq < nq; ++kq) {
+            const int sl = q - kq * klen;
+            if (sl >= 0 && sl < wwin_len) acc += lds_wwin[kq * p.gw + hsub][sl];
         }
-        wout[q] = acc;
+        p.win[(((long long)wh.b * p.index_heads + wh.slot) * p.nchunks + wh.chunk) * WIN + q] = acc;
     }
 }
 
@@ -374,9 +389,11 @@ int fill(EstParams &p, const void *q, const void *k, const int64_t *q_stride, co
     p.win = (float *)((char *)ws + stats_b + row_b);
     p.vertical = vertical; p.slash = slash;
     p.force_v = force_v; p.force_s = force_s;
+    // heads per workgroup: neighbours in head order that (mostly) share a kv head
     const int group = heads_q / heads_kv;
-    const long long grid_heads = head_list ? (long long)((index_heads + group - 1) / group) * group : heads_q;
-    p.total_wg = (long long)batch * grid_heads * p.nchunks;
+    p.gw = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);
+    p.nhc = (index_heads + p.gw - 1) / p.gw;
+    p.total_wg = (long long)batch * p.nhc * p.nchunks;
     p.head_list = head_list;
     p.index_heads = index_heads;
     return MINF_OK;
