@@ -125,7 +125,9 @@ int minf_vs_index_build_static(const int32_t *seqlens, const int32_t *vertical_i
  *   {batch, head, token} (head_dim stride is 1); heads_q % heads_kv == 0 and
  *   query head h reads kv head h / (heads_q / heads_kv) (no repeat_kv copy is
  *   needed; the reference always expands K/V first,
- *   minference/modules/forward.py:128-132).  head_dim must be 128.
+ *   minference/modules/forward.py:128-132).  head_dim must be 64 or 128 (the
+ *   reference's kernels accept 16/32/64/128, pit_sparse_flash_attention_v2.py:172;
+ *   smaller head dims are zero-padded to 64 by the caller).
  *   seqlens [batch] int32 may be NULL (= n for every batch).  Rows >= seqlen
  *   are written as zeros (the reference leaves its zeros_like buffer untouched).
  *   sm_scale multiplies q.k before the softmax (reference: head_dim^-0.5).

@@ -77,9 +77,8 @@ enum { MODE_VS = 0, MODE_BS = 1, MODE_ASHAPE = 2, MODE_DENSE = 3 };
 
 constexpr int BM = 64;        // query rows per workgroup
 constexpr int BN = 64;        // keys per tile
-constexpr int HD = 128;       // head_dim
+constexpr int HD_MAX = 128;   // head_dim: 128 or 64 (template parameter HD of the kernel)
 constexpr int NTHREADS = 128; // 2 wavefronts per 64-row block (x2 in the paired variant)
-constexpr int ROW_BYTES = HD * 2;
 // Scheduling constants (measured on MI355X): K fragments are read QK_AHEAD k-steps ahead of their
 // MFMAs; VALU_PER_MFMA softmax instructions are placed behind each of the first twelve PV MFMAs.
 constexpr int QK_AHEAD = 2;
@@ -176,7 +175,8 @@ struct Tile {
     int split;          // paired vertical-slash: each row block has a tile of its own in this step
 };
 constexpr int BS_PAIR_MAX = 512;   // longest block list the paired block-sparse walk keeps in LDS
-constexpr int VS_PAIR_MAX = 2048;  // longest vertical-slash block list the paired kernel merges in LDS
+// (the longest vertical-slash block list the paired kernel splits in LDS is what a K tile holds twice:
+// 2048 entries at head_dim 128, 1024 at 64)
 constexpr int VS_ONLY_MAX = 512;   // ... and the most entries of one list that the other one lacks
 
 template <int MODE>
@@ -265,12 +265,24 @@ __device__ __forceinline__ bool tile_on_list(const AttnParams &p, int m, int sta
     return ti >= t_lo || ti < ((p.n_init + BN - 1) >> 6);
 }
 
-template <typename T, int MODE, bool PAIR>
+template <typename T, int MODE, bool PAIR, int HD>
 __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_kernel(const AttnParams p) {
+    static_assert(HD == 128 || HD == 64, "head_dim 128 or 64");
+    constexpr int ROW_BYTES = HD * 2;                       // one token row of K / V / Q / O
+    constexpr int KS = HD / 16;                             // k-steps of S^T = K.Q^T
+    constexpr int NDB = HD / 32;                            // 32-row blocks of O^T
+    constexpr int NCH = ROW_BYTES / 16;                     // 16-byte chunks per row
+    constexpr int RPI = 64 / NCH;                           // tile rows one copy instruction fills (64 lanes x 16 B)
+    // LDS chunk permutations (conflict-free ds_read_b128 of 32 K rows / transpose reads of 4 V rows):
+    // 256-byte rows: K chunk ^ row%16, V chunk ^ 4*(row%4); 128-byte rows (two rows per bank sweep):
+    // K chunk ^ (row/2)%8, V chunk ^ 4*((row/2)%2)
+    auto swz_k = [](int row) { return HD == 128 ? (row & 15) : ((row >> 1) & 7); };
+    auto swz_v = [](int row) { return HD == 128 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); };
     constexpr int NT = PAIR ? 2 * NTHREADS : NTHREADS;      // threads per workgroup
     constexpr int CROWS = PAIR ? 16 : 32;                   // tile rows copied by one wave (shared tile)
     constexpr bool VSP = PAIR && MODE == MODE_VS;
     constexpr int TILE_BYTES = BN * ROW_BYTES;
+    constexpr int VS_PAIR_MAX = TILE_BYTES / 8;             // both staged lists fit the second K tile
     // separate LDS objects: the compiler then lets reads of one overtake copies into the other
     // paired vertical-slash: a second K and V tile (row block B's buffers in the steps in which each
     // row block has a tile of its own); before that, the second K tile stages the two block lists and
@@ -336,9 +348,9 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
     const bool have_rows = m < p.rows && row0 < seqlen;
     if (!have_rows) {
         if (m < p.rows)
-            for (int i = tid & (NTHREADS - 1); i < BM * 16; i += NTHREADS) {
-                int r = row0 + (i >> 4);
-                if (r < p.n) *reinterpret_cast<u32x4_t *>(o_base + (long long)r * p.os[2] * 2 + (i & 15) * 16) = u32x4_t{0u, 0u, 0u, 0u};
+            for (int i = tid & (NTHREADS - 1); i < BM * NCH; i += NTHREADS) {
+                int r = row0 + i / NCH;
+                if (r < p.n) *reinterpret_cast<u32x4_t *>(o_base + (long long)r * p.os[2] * 2 + (i % NCH) * 16) = u32x4_t{0u, 0u, 0u, 0u};
             }
         if (!PAIR || mA * BM >= seqlen) return;      // (wave-uniform; for a pair: both halves are past)
     }
@@ -350,12 +362,12 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
     const long long ridx = ((long long)b * p.index_heads + hs) * p.rows + min(m, p.rows - 1);
 
     // ---- Q fragments (B operand of S^T): row qrow, d = 16*ks + 8*g + 0..7 ----
-    Frag qf[8];
+    Frag qf[KS];
     {
         const bool ok = qrow < seqlen;
         const char *qp = q_base + (long long)(ok ? qrow : min(row0, seqlen - 1)) * p.qs[2] * 2 + g * 16;
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) {
+        for (int ks = 0; ks < KS; ++ks) {
             qf[ks].u = *reinterpret_cast<const u32x4_t *>(qp + ks * 32);
             if (!ok) qf[ks].u = u32x4_t{0u, 0u, 0u, 0u};
         }
@@ -546,14 +558,14 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
     // permutation is applied on the global side: lane (row, c') loads global chunk c' ^ swz(row).
     // Rows that do not exist (past seqlen, or padding of a gathered tile) are read from a clamped,
     // valid address: their scores are masked to -inf, so their probabilities are exactly 0.
-    const int cp_r = lane >> 4;                  // row inside the 4-row group
-    const int cp_c = lane & 15;                  // LDS chunk
+    const int cp_r = lane / NCH;                 // row inside the group of RPI rows one instruction fills
+    const int cp_c = lane % NCH;                 // LDS chunk
     // gathered tiles: lane l holds the token id of tile row l (one load per lane, issued an
     // iteration ahead); the copy fetches the ids of its own rows with wave shuffles
     int k_lane[4], v_lane;
 #pragma unroll
-    for (int jj = 0; jj < 4; ++jj) k_lane[jj] = cp_r * (int)k_row + ((cp_c ^ (4 * jj + cp_r)) << 4);
-    v_lane = cp_r * (int)v_row + ((cp_c ^ (cp_r << 2)) << 4);
+    for (int jj = 0; jj < 4; ++jj) k_lane[jj] = cp_r * (int)k_row + ((cp_c ^ swz_k(RPI * jj + cp_r)) << 4);
+    v_lane = cp_r * (int)v_row + ((cp_c ^ swz_v(cp_r)) << 4);
     auto gather_ids = [&](const Tile &t) -> int {
         if (MODE == MODE_VS && t.gathered) return p.ci[ridx * p.nnz_v + t.start + min(lane, max(t.nvalid, 1) - 1)];
         return 0;
@@ -573,13 +585,13 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
             // first row offset and step of this wave's part; in the paired vertical-slash kernel (two
             // copy shapes, K and V strides) they are made opaque so that the per-copy offsets are formed
             // with one scalar add each instead of living in two dozen loop-invariant scalar registers
-            int soff0 = CROWS * wsel * (int)rowstride, sstep = 4 * (int)rowstride;
+            int soff0 = CROWS * wsel * (int)rowstride, sstep = RPI * (int)rowstride;
             int lds0 = (int)(unsigned)(unsigned long long)(__attribute__((address_space(3))) char *)ldsbuf + CROWS * wsel * ROW_BYTES;
             if constexpr (VSP) asm volatile("" : "+s"(soff0), "+s"(sstep), "+s"(lds0));
 #pragma unroll
-            for (int j = 0; j < CROWS / 4; ++j) {
-                const int voff = is_v ? v_lane : k_lane[j & 3];
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(srd, (__attribute__((address_space(3))) void *)(unsigned long long)(unsigned)(lds0 + 4 * j * ROW_BYTES),
+            for (int j = 0; j < CROWS / RPI; ++j) {
+                const int voff = is_v ? v_lane : k_lane[j & 3];     // (the K permutation repeats every 16 rows)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(srd, (__attribute__((address_space(3))) void *)(unsigned long long)(unsigned)(lds0 + RPI * j * ROW_BYTES),
                                                          16, voff, soff0 + j * sstep, 0, 0);
             }
             return;
@@ -587,29 +599,29 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
         // three straight-line variants (a per-row select would turn into sixteen tiny branches).
         // The two rare ones recompute their per-lane rows and chunks on the spot (the empty asm
         // keeps the compiler from hoisting a dozen loop-invariant registers out of the tile loop).
-        int cp_r = lane >> 4, cp_c = lane & 15;
+        int cp_r = lane / NCH, cp_c = lane % NCH;
         asm volatile("" : "+v"(cp_r), "+v"(cp_c));
         if (gathered) {
 #pragma unroll
-            for (int j = 0; j < CROWS / 4; ++j) {
-                const int r = CROWS * wsel + 4 * j + cp_r;          // tile row
+            for (int j = 0; j < CROWS / RPI; ++j) {
+                const int r = CROWS * wsel + RPI * j + cp_r;        // tile row
                 const int tk = max(0, min(__shfl(idv, r), seqlen - 1));
-                const int c = is_v ? (cp_c ^ ((r & 3) << 2)) : (cp_c ^ (r & 15));
+                const int c = is_v ? (cp_c ^ swz_v(r)) : (cp_c ^ swz_k(r));
                 const char *gp = base + tk * rowstride + c * 16;
                 __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
-                                                 (__attribute__((address_space(3))) void *)(ldsbuf + (CROWS * wsel + 4 * j) * ROW_BYTES),
+                                                 (__attribute__((address_space(3))) void *)(ldsbuf + (CROWS * wsel + RPI * j) * ROW_BYTES),
                                                  16, 0, 0);
             }
             return;
         }
 #pragma unroll
-        for (int j = 0; j < CROWS / 4; ++j) {
-            const int r = CROWS * wsel + 4 * j + cp_r;
+        for (int j = 0; j < CROWS / RPI; ++j) {
+            const int r = CROWS * wsel + RPI * j + cp_r;
             const int tk = max(0, min(t.start + r, seqlen - 1));
-            const int c = is_v ? (cp_c ^ ((r & 3) << 2)) : (cp_c ^ (r & 15));
+            const int c = is_v ? (cp_c ^ swz_v(r)) : (cp_c ^ swz_k(r));
             const char *gp = base + tk * rowstride + c * 16;
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gp,
-                                             (__attribute__((address_space(3))) void *)(ldsbuf + (CROWS * wsel + 4 * j) * ROW_BYTES),
+                                             (__attribute__((address_space(3))) void *)(ldsbuf + (CROWS * wsel + RPI * j) * ROW_BYTES),
                                              16, 0, 0);
         }
     };
@@ -624,9 +636,9 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
     };
 
     // ---- accumulators -------------------------------------------------------
-    f32x16_t oacc[4];
+    f32x16_t oacc[NDB];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < NDB; ++i)
 #pragma unroll
         for (int r = 0; r < 16; ++r) oacc[i][r] = 0.f;
     float m_i = -INFINITY;   // running max (log2 domain, scaled)
@@ -634,24 +646,25 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
 
     // LDS read addresses that do not depend on the tile
     // K: row 32*blk + l32, logical chunk 2*ks + g -> physical chunk ^ (row % 16)
-    int k_rd_off[8];
+    int k_rd_off[KS];
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) k_rd_off[ks] = l32 * ROW_BYTES + (((2 * ks + g) ^ (l32 & 15)) << 4);
+    for (int ks = 0; ks < KS; ++ks) k_rd_off[ks] = l32 * ROW_BYTES + (((2 * ks + g) ^ swz_k(l32)) << 4);
     // V transpose read: row = 16*s + 8*jj + 4*g + rsub (row % 4 == rsub), logical chunk
     // 4*db + vc -> physical 4*(db ^ rsub) + vc
     const int v_rd_rsub = (lane & 15) >> 2;
     const int v_rd_vc = (((lane >> 4) & 1) << 1) + ((lane & 3) >> 1);
-    int v_rd_off[4];
+    int v_rd_off[NDB];
 #pragma unroll
-    for (int db = 0; db < 4; ++db)
-        v_rd_off[db] = (4 * g + v_rd_rsub) * ROW_BYTES + ((((db ^ v_rd_rsub) << 2) + v_rd_vc) << 4) + ((lane & 1) << 3);
+    for (int db = 0; db < NDB; ++db)
+        v_rd_off[db] = (4 * g + v_rd_rsub) * ROW_BYTES + ((((db << 2) + v_rd_vc) ^ swz_v(v_rd_rsub)) << 4) + ((lane & 1) << 3);
 
     // ---- S^T = K . Q^T for this wave's 32 query rows; K tile in kbuf.  EARLY (2-wave kernel, whose
     // waves all run this code): the tile's second barrier comes after k-step EARLY_B2, when every K
     // fragment has been read, and all V^T fragment reads are issued under the last four MFMAs.
-    auto qk_block = [&](const char *kbuf, const char *vbuf, f32x16_t &s0, f32x16_t &s1, Frag (&vf)[4][4], auto early_c) {
+    auto qk_block = [&](const char *kbuf, const char *vbuf, f32x16_t &s0, f32x16_t &s1, Frag (&vf)[4][NDB], auto early_c) {
         constexpr bool EARLY = decltype(early_c)::value;
-        Frag a0[8], a1[8];
+        constexpr int EARLY_AT = EARLY_B2 * KS / 8;       // the k-step after which every K fragment has been read
+        Frag a0[KS], a1[KS];
         __builtin_amdgcn_s_setprio(2);
 #pragma unroll
         for (int r = 0; r < 16; ++r) { s0[r] = 0.f; s1[r] = 0.f; }
@@ -664,8 +677,8 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) {
-            if (ks + QK_AHEAD < 8) {
+        for (int ks = 0; ks < KS; ++ks) {
+            if (ks + QK_AHEAD < KS) {
                 a0[ks + QK_AHEAD].u = *reinterpret_cast<const u32x4_t *>(kbuf + k_rd_off[ks + QK_AHEAD]);
                 a1[ks + QK_AHEAD].u = *reinterpret_cast<const u32x4_t *>(kbuf + k_rd_off[ks + QK_AHEAD] + 32 * ROW_BYTES);
             }
@@ -673,13 +686,13 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
             s1 = Mma<T>::mfma(frag_as<T>(a1[ks]), frag_as<T>(qf[ks]), s1);
             __builtin_amdgcn_sched_barrier(0);
             if constexpr (EARLY) {
-                if (ks == EARLY_B2) {
+                if (ks == EARLY_AT) {
                     __builtin_amdgcn_s_waitcnt(0x0f70);
                     __syncthreads();
 #pragma unroll
                     for (int s = 0; s < 4; ++s)
 #pragma unroll
-                        for (int db = 0; db < 4; ++db)
+                        for (int db = 0; db < NDB; ++db)
 #pragma unroll
                             for (int jj = 0; jj < 2; ++jj)
                                 vf[s][db].s4[jj] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
@@ -692,7 +705,7 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
 
     // ---- mask, online softmax, O^T += V^T . P^T.  READ_V: the V^T fragments have not been read yet
     // (4-wave variants, whose second barrier sits between the two blocks).
-    auto sm_pv_block = [&](const Tile &cur, const char *vbuf, f32x16_t &s0, f32x16_t &s1, Frag (&vf)[4][4], auto read_v_c) {
+    auto sm_pv_block = [&](const Tile &cur, const char *vbuf, f32x16_t &s0, f32x16_t &s1, Frag (&vf)[4][NDB], auto read_v_c) {
         constexpr bool READ_V = decltype(read_v_c)::value;
         // element (blk, r) of this lane is tile-local key tk = tkc + 4*g with the compile-time
         // part tkc = 32*blk + 8*(r/4) + r%4.  keep <=> tk <= hi && (tk > wlo || tk < slim).
@@ -744,7 +757,7 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
 #pragma unroll
         for (int s = 0; s < 4; ++s)
 #pragma unroll
-        for (int db = 0; db < 4; ++db)
+        for (int db = 0; db < NDB; ++db)
 #pragma unroll
             for (int jj = 0; jj < 2; ++jj)
                 vf[s][db].s4[jj] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
@@ -785,7 +798,7 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
         probs(0);
         if (__any(alpha != 1.0f)) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+            for (int i = 0; i < NDB; ++i)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
         }
@@ -800,12 +813,13 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
 #pragma unroll
             for (int s = 0; s < 4; ++s)
 #pragma unroll
-                for (int db = 0; db < 4; ++db)
+                for (int db = 0; db < NDB; ++db)
                     oacc[db] = Mma<T>::mfma(frag_as<T>(vf[s][db]), frag_as<T>(pfr[s]), oacc[db]);
+            // the softmax instructions of key groups 1..3 are spread behind the MFMAs of groups 0..2
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
+            for (int i = 0; i < 4 * NDB; ++i) {
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                if (i < 12) __builtin_amdgcn_sched_group_barrier(VALU_MASK, VALU_PER_MFMA, 0);
+                if (i < 3 * NDB) __builtin_amdgcn_sched_group_barrier(VALU_MASK, VALU_PER_MFMA * 4 / NDB, 0);
             }
         }
         __builtin_amdgcn_s_setprio(0);
@@ -845,9 +859,9 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
                 // offsets move in place, once)
                 vs_shifted = true;
 #pragma unroll
-                for (int ks = 0; ks < 8; ++ks) k_rd_off[ks] += half * TILE_BYTES;
+                for (int ks = 0; ks < KS; ++ks) k_rd_off[ks] += half * TILE_BYTES;
 #pragma unroll
-                for (int db = 0; db < 4; ++db) v_rd_off[db] += half * TILE_BYTES;
+                for (int db = 0; db < NDB; ++db) v_rd_off[db] += half * TILE_BYTES;
             }
         } else {
             copy_tile(cur, v_base, v_row, std::true_type{}, gt_cur, lds_v);
@@ -861,7 +875,7 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
         if constexpr (PAIR && (MODE == MODE_BS || MODE == MODE_VS)) active = have_rows && (half ? cur.on_b : cur.on_a);   // (split steps: on_a == on_b == own flag)
         else if constexpr (PAIR) active = have_rows && tile_on_list<MODE>(p, m, cur.start);
         f32x16_t s0, s1;
-        Frag vf[4][4];
+        Frag vf[4][NDB];
         if (active) qk_block(lds_k, lds_v, s0, s1, vf, std::integral_constant<bool, !PAIR>{});
         if constexpr (PAIR) {
             __builtin_amdgcn_s_waitcnt(0x0f70);      // vmcnt(0): this wave's part of V(it) is in LDS
@@ -886,7 +900,7 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
         char *ot = PAIR ? (half ? lds_v : lds_k) + wave * 32 * OP : (wave ? lds_v : lds_k);   // 32 rows per wave
         const bool live = qrow < seqlen;
 #pragma unroll
-        for (int db = 0; db < 4; ++db)
+        for (int db = 0; db < NDB; ++db)
 #pragma unroll
             for (int rq = 0; rq < 4; ++rq) {
                 union { T e[4]; u32x2_t u; } out4;
@@ -895,13 +909,13 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
                 *reinterpret_cast<u32x2_t *>(ot + l32 * OP + (32 * db + 8 * rq + 4 * g) * 2) = out4.u;
             }
         __builtin_amdgcn_wave_barrier();
-        // lane -> (row = 4*i + lane/16, chunk = lane%16)
+        // lane -> (row = RPI*i + lane/NCH, chunk = lane%NCH)
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int r = 4 * i + (lane >> 4);
+        for (int i = 0; i < 32 / RPI; ++i) {
+            const int r = RPI * i + lane / NCH;
             const int grow = row0 + wave * 32 + r;
-            const u32x4_t val = *reinterpret_cast<const u32x4_t *>(ot + r * OP + (lane & 15) * 16);
-            if (grow < p.n && have_rows) *reinterpret_cast<u32x4_t *>(o_base + (long long)grow * p.os[2] * 2 + (lane & 15) * 16) = val;
+            const u32x4_t val = *reinterpret_cast<const u32x4_t *>(ot + r * OP + (lane % NCH) * 16);
+            if (grow < p.n && have_rows) *reinterpret_cast<u32x4_t *>(o_base + (long long)grow * p.os[2] * 2 + (lane % NCH) * 16) = val;
         }
     }
 }
@@ -914,7 +928,7 @@ int check_tensors(const minf_qkvo *t) {
     if (!empty && (!t->q || !t->k || !t->v || !t->o)) return MINF_ERR_INVALID_ARG;
     if (t->heads_q % t->heads_kv != 0) return MINF_ERR_INVALID_ARG;
     if (t->head_list && t->index_heads <= 0) return MINF_ERR_INVALID_ARG;
-    if (t->head_dim != HD) return MINF_ERR_UNSUPPORTED;
+    if (t->head_dim != 128 && t->head_dim != 64) return MINF_ERR_UNSUPPORTED;
     if (t->dtype != MINF_BF16 && t->dtype != MINF_F16) return MINF_ERR_UNSUPPORTED;
     const void *ptrs[4] = {t->q, t->k, t->v, t->o};
     const int64_t *strides[4] = {t->q_stride, t->k_stride, t->v_stride, t->o_stride};
@@ -926,7 +940,7 @@ int check_tensors(const minf_qkvo *t) {
         if (strides[i][2] > (1 << 23)) return MINF_ERR_UNSUPPORTED;
         // rows must not overlap (expanded or interleaved views): the tile copies describe 64 rows of
         // a tile by one buffer descriptor of 64 x token stride bytes
-        if (t->n > 1 && strides[i][2] < HD) return MINF_ERR_UNSUPPORTED;
+        if (t->n > 1 && strides[i][2] < t->head_dim) return MINF_ERR_UNSUPPORTED;
     }
     return MINF_OK;
 }
@@ -950,7 +964,7 @@ void fill_params(AttnParams &p, const minf_qkvo *t) {
     p.descending = 0;
 }
 
-template <int MODE> int launch(AttnParams p, int dtype, void *stream) {
+template <int MODE, int HD> int launch_hd(AttnParams p, int dtype, void *stream) {
     if (p.batch == 0 || p.rows == 0) return MINF_OK;
     // every mode runs on the paired (4-wave) kernel, except block-sparse lists that are too long for
     // the paired walk's LDS copy: those run on the 2-wave kernel
@@ -969,17 +983,21 @@ template <int MODE> int launch(AttnParams p, int dtype, void *stream) {
     hipStream_t st = (hipStream_t)stream;
     if constexpr (CAN_PAIR) {
         if (pair) {
-            if (dtype == MINF_BF16) hipLaunchKernelGGL((attn_fwd_kernel<__bf16, MODE, true>), dim3((unsigned)grid), block, 0, st, p);
-            else hipLaunchKernelGGL((attn_fwd_kernel<_Float16, MODE, true>), dim3((unsigned)grid), block, 0, st, p);
+            if (dtype == MINF_BF16) hipLaunchKernelGGL((attn_fwd_kernel<__bf16, MODE, true, HD>), dim3((unsigned)grid), block, 0, st, p);
+            else hipLaunchKernelGGL((attn_fwd_kernel<_Float16, MODE, true, HD>), dim3((unsigned)grid), block, 0, st, p);
             return minf_launch_status();
         }
     }
     if constexpr (CAN_SINGLE) {
-        if (dtype == MINF_BF16) hipLaunchKernelGGL((attn_fwd_kernel<__bf16, MODE, false>), dim3((unsigned)grid), block, 0, st, p);
-        else hipLaunchKernelGGL((attn_fwd_kernel<_Float16, MODE, false>), dim3((unsigned)grid), block, 0, st, p);
+        if (dtype == MINF_BF16) hipLaunchKernelGGL((attn_fwd_kernel<__bf16, MODE, false, HD>), dim3((unsigned)grid), block, 0, st, p);
+        else hipLaunchKernelGGL((attn_fwd_kernel<_Float16, MODE, false, HD>), dim3((unsigned)grid), block, 0, st, p);
         return minf_launch_status();
     }
     return MINF_ERR_UNSUPPORTED;      // not reached: every mode has one of the two variants
+}
+
+template <int MODE> int launch(const AttnParams &p, const minf_qkvo *t, void *stream) {
+    return t->head_dim == 64 ? launch_hd<MODE, 64>(p, t->dtype, stream) : launch_hd<MODE, 128>(p, t->dtype, stream);
 }
 
 }  // namespace
@@ -997,7 +1015,7 @@ extern "C" int minf_vs_attn_fwd(const minf_qkvo *t, const int32_t *block_count,
     if (rows != p.rows) return MINF_ERR_INVALID_ARG;
     p.bc = block_count; p.bo = block_offset; p.cc = column_count; p.ci = column_index;
     p.nnz_s = nnz_s; p.nnz_v = nnz_v;
-    return launch<MODE_VS>(p, t->dtype, stream);
+    return launch<MODE_VS>(p, t, stream);
 }
 
 extern "C" int minf_bs_attn_fwd(const minf_qkvo *t, const int32_t *block_index, int rows,
@@ -1010,7 +1028,7 @@ extern "C" int minf_bs_attn_fwd(const minf_qkvo *t, const int32_t *block_index, 
     if (rows < p.rows) return MINF_ERR_INVALID_ARG;
     // block_index may have more rows than ceil(n/64) (the reference pads n first)
     p.bidx = block_index; p.max_blocks = max_blocks; p.bidx_rows = rows;
-    return launch<MODE_BS>(p, t->dtype, stream);
+    return launch<MODE_BS>(p, t, stream);
 }
 
 extern "C" int minf_ashape_attn_fwd(const minf_qkvo *t, int n_init, int n_local, void *stream) {
@@ -1020,7 +1038,7 @@ extern "C" int minf_ashape_attn_fwd(const minf_qkvo *t, int n_init, int n_local,
     AttnParams p;
     fill_params(p, t);
     p.n_init = n_init; p.n_local = n_local;
-    return launch<MODE_ASHAPE>(p, t->dtype, stream);
+    return launch<MODE_ASHAPE>(p, t, stream);
 }
 
 extern "C" int minf_trishape_attn_fwd(const minf_qkvo *t, int n_init, int n_local, int n_last, void *stream) {
@@ -1031,7 +1049,7 @@ extern "C" int minf_trishape_attn_fwd(const minf_qkvo *t, int n_init, int n_loca
     fill_params(p, t);
     p.n_init = n_init; p.n_local = n_local;
     p.dense_from = n_last < t->n ? t->n - n_last : 0;
-    return launch<MODE_ASHAPE>(p, t->dtype, stream);
+    return launch<MODE_ASHAPE>(p, t, stream);
 }
 
 extern "C" int minf_dense_attn_fwd(const minf_qkvo *t, void *stream) {
@@ -1039,5 +1057,5 @@ extern "C" int minf_dense_attn_fwd(const minf_qkvo *t, void *stream) {
     if (st) return st;
     AttnParams p;
     fill_params(p, t);
-    return launch<MODE_DENSE>(p, t->dtype, stream);
+    return launch<MODE_DENSE>(p, t, stream);
 }

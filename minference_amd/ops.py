@@ -23,7 +23,8 @@ import torch
 from . import _lib
 from .index import convert_vertical_slash_indexes
 
-_SUPPORTED_D = 128
+_SUPPORTED_D = 128            # head_dim of the estimation / block-index kernels, largest of the tile engine
+_NATIVE_D = (64, 128)         # head_dims the tile engine is instantiated for; others are zero-padded up
 
 
 def _prep(t: torch.Tensor) -> torch.Tensor:
@@ -67,7 +68,7 @@ class _Call:
     """Holds the (possibly cast/padded) tensors of one operator call and the
     filled ``minf_qkvo`` struct."""
 
-    def __init__(self, q, k, v, seqlens=None, need_out=True):
+    def __init__(self, q, k, v, seqlens=None, need_out=True, pad_to=None):
         _check_qkv(q, k, v)
         self.out_dtype = q.dtype
         self.head_dim = q.shape[-1]
@@ -79,23 +80,27 @@ class _Call:
         D = q.shape[-1]
         if D > _SUPPORTED_D:
             raise ValueError(f"head_dim {D} > {_SUPPORTED_D} is not supported")
-        if D < _SUPPORTED_D:
+        # the reference runs head_dim 16, 32, 64, 128 (pit_sparse_flash_attention_v2.py:172); here 64 and
+        # 128 are native, anything else is zero-padded to the next of the two (or to `pad_to`)
+        Dk = pad_to if pad_to else min(d for d in _NATIVE_D if d >= D)
+        if D < Dk:
             # zero columns change neither q.k nor the first D output columns
-            pad = _SUPPORTED_D - D
+            pad = Dk - D
             q = torch.nn.functional.pad(q, [0, pad])
             k = torch.nn.functional.pad(k, [0, pad])
             v = torch.nn.functional.pad(v, [0, pad])
+        self.kernel_dim = Dk
         self.q, self.k, self.v = _prep(q), _prep(k), _prep(v)
         B, H, N, _ = self.q.shape
         self.B, self.H, self.N, self.Hk = B, H, N, self.k.shape[1]
-        self.o = torch.empty((B, H, N, _SUPPORTED_D) if need_out else (1, 1, 1, _SUPPORTED_D),
+        self.o = torch.empty((B, H, N, Dk) if need_out else (1, 1, 1, Dk),
                              dtype=self.q.dtype, device=q.device)
         s = _lib.QKVO()
         s.q, s.k, s.v, s.o = self.q.data_ptr(), self.k.data_ptr(), self.v.data_ptr(), self.o.data_ptr()
         for name, t in (("q_stride", self.q), ("k_stride", self.k), ("v_stride", self.v), ("o_stride", self.o)):
             getattr(s, name)[:] = list(t.stride()[:3])
         s.batch, s.heads_q, s.heads_kv, s.n = B, H, self.Hk, N
-        s.head_dim = _SUPPORTED_D
+        s.head_dim = Dk
         s.dtype = _lib.MINF_BF16 if self.q.dtype == torch.bfloat16 else _lib.MINF_F16
         self.seqlens = seqlens
         s.seqlens = seqlens.data_ptr() if seqlens is not None else None
@@ -117,7 +122,7 @@ class _Call:
 
     def result(self):
         o = self.o
-        if self.head_dim != _SUPPORTED_D:
+        if self.head_dim != self.kernel_dim:
             o = o[..., : self.head_dim]
         if o.dtype != self.out_dtype:
             o = o.to(self.out_dtype)
@@ -189,7 +194,7 @@ def _build_block_index(query, key, top_k, block_size_M=64, block_size_N=64, forc
     rows = (n + 64 - n % 64) / 64, every row ascending."""
     if block_size_M != 64 or block_size_N != 64:
         raise ValueError("only 64x64 blocks are supported")
-    c = _Call(query, key, key, need_out=False)           # casts / pads head_dim exactly like the attention call
+    c = _Call(query, key, key, need_out=False, pad_to=_SUPPORTED_D)   # the block-index kernels take head_dim 128
     lib = _lib.load()
     rows = lib.minf_bs_block_index_rows(c.N)
     kk = min(int(top_k), rows)

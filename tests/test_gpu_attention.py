@@ -211,12 +211,74 @@ def test_strided_inputs_and_batch(gpu):
     check(out, ref, "strided")
 
 
-def test_head_dim_64_is_padded(gpu):
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("n,hq,hk", [(64, 1, 1), (300, 2, 2), (1000, 4, 1), (4100, 4, 2)])
+def test_head_dim_64_runs_natively(gpu, monkeypatch, dtype, n, hq, hk):
+    """head_dim 64 (reference: pit_sparse_flash_attention_v2.py:172, block_sparse_flash_attention.py:128
+    accept 16, 32, 64, 128) on the tile engine's own 64-wide instantiation: no padded copies of
+    q/k/v (torch.nn.functional.pad must not be called by the attention operators), all four tile
+    sources against the oracle, gathered columns and ragged tails included."""
+    import minference_amd as M
+    print(f"case d64 n={n} hq={hq} hk={hk} {dtype}", flush=True)
+    q, k, v = make(1, hq, hk, n, 60 + n, dtype, d=64)
+    qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
+    ke, ve = expand(k, hq), expand(v, hq)
+
+    def no_pad(*a, **kw):
+        raise AssertionError("head_dim 64 must not be zero-padded")
+    real_pad = torch.nn.functional.pad
+    monkeypatch.setattr(torch.nn.functional, "pad", no_pad)
+    out = M.dense_causal_attention(qg, kg, vg)
+    assert out.shape == q.shape and out.dtype == dtype
+    check(out, sdpa_causal(q, ke, ve), "d64 dense")
+    n_init, n_local = min(16, n), max(1, n // 3)
+    check(M.streaming_forward(qg, kg, vg, n_init, n_local), O.streaming_forward(q, ke, ve, n_init, n_local), "d64 a-shape")
+    nv, ns = min(n, 90), min(n, 130)
+    vi, si = gen.vs_index_inputs(hq, n, nv, ns, seed=n, force_v=min(4, nv), force_s=min(64, ns))
+    v_idx, s_idx = torch.from_numpy(vi), torch.from_numpy(np.ascontiguousarray(si))
+    out = M.vertical_slash_sparse_attention(qg, kg, vg, v_idx.to(gpu), s_idx.to(gpu))
+    check(out, O.vertical_slash_sparse_attention(q, ke, ve, v_idx, s_idx), "d64 vertical-slash")
+    monkeypatch.setattr(torch.nn.functional, "pad", real_pad)
+    # block-sparse: the index comes from the oracle (the block-index kernels take head_dim 128)
+    pad = 64 - (n & 63)
+    bi = O.bs_block_index(real_pad(q, [0, 0, 0, pad]), real_pad(ke, [0, 0, 0, pad]), 5)
+    out = M.block_sparse_attention_from_index(qg, kg, vg, bi.contiguous().to(gpu))
+    ref = torch.stack([O.masked_attention(q[0, h], ke[0, h], ve[0, h], O.bs_mask(bi[0, h].numpy(), n)) for h in range(hq)])[None]
+    check(out, ref, "d64 block-sparse")
+
+
+def test_head_dim_64_long_lists_and_the_whole_path(gpu):
+    """head_dim 64 at 20000 tokens through estimate -> top-k -> index -> attention (lists long enough
+    for the paired walk's common / leftover split and several gathered tiles per row block), and the
+    block_sparse operator end to end; sampled against the oracle on the indices the GPU produced."""
+    import minference_amd as M
+    n, hq, hk = 20000 + 13, 4, 2
+    q, k, v = make(1, hq, hk, n, 77, torch.bfloat16, d=64)
+    qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
+    v_idx, s_idx = M.estimate_vertical_slash(qg, kg, 700, 900)
+    out = M.vertical_slash_sparse_attention(qg, kg, vg, v_idx, s_idx)
+    for h in (0, 3):
+        kv = h // (hq // hk)
+        ref = O.vertical_slash_sparse_attention(q[:, h:h + 1], k[:, kv:kv + 1], v[:, kv:kv + 1], v_idx[:, h:h + 1].cpu(), s_idx[:, h:h + 1].cpu())
+        check(out[:, h:h + 1], ref, f"d64 whole path head {h}")
+    out = M.block_sparse_attention(qg, kg, vg, 20)
+    from minference_amd.ops import _build_block_index
+    bi = _build_block_index(qg, kg, 20)[0].cpu().numpy()
+    for h in (1, 2):
+        kv = h // (hq // hk)
+        ref = O.masked_attention(q[0, h], k[0, kv], v[0, kv], O.bs_mask(bi[h], n))[None, None]
+        check(out[:, h:h + 1], ref, f"d64 block_sparse head {h}")
+
+
+@pytest.mark.parametrize("d,kernel_d", [(32, 64), (16, 64), (96, 128)])
+def test_other_head_dims_are_zero_padded_to_the_next_instantiation(gpu, d, kernel_d):
     from minference_amd import dense_causal_attention
-    q, k, v = make(1, 2, 2, 300, 32, torch.bfloat16, d=64)
+    from minference_amd.ops import _Call
+    q, k, v = make(1, 2, 2, 300, 32 + d, torch.bfloat16, d=d)
+    assert _Call(q.to(gpu), k.to(gpu), v.to(gpu)).kernel_dim == kernel_d
     out = dense_causal_attention(q.to(gpu), k.to(gpu), v.to(gpu))
     assert out.shape == q.shape
-    check(out, sdpa_causal(q, k, v), "d64")
+    check(out, sdpa_causal(q, k, v), f"d{d}")
 
 
 def test_golden_fixtures(gpu):
