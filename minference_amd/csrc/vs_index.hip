@@ -611,7 +611,12 @@ static int index_build_tables(const int32_t *seqlens, const int32_t *vertical_id
                        dim3(256), 0, stream, workspace, nnz_s, rows);
     status = minf_launch_status();
     if (status != MINF_OK) return status;
-    hipLaunchKernelGGL(vs_index_fast_kernel, dim3((unsigned)nblk), dim3(IDX_WAVES * MINF_WAVE), 0,
+    // With zero-filled outputs the row-block pass is bound by its stores, and 24 resident waves per CU
+    // write faster than 32 (6-9 % at 128K-512K tokens: fewer rows in flight, better DRAM locality); the
+    // payload-only form is bound by its chains of dependent loads and wants every wave it can get.
+    // Unused dynamic LDS is the occupancy limiter: 3 KB static + 24000 B -> 6 workgroups per CU.
+    const unsigned occupancy_lds = zero_fill ? 24000u : 0u;
+    hipLaunchKernelGGL(vs_index_fast_kernel, dim3((unsigned)nblk), dim3(IDX_WAVES * MINF_WAVE), occupancy_lds,
                        stream, seqlens, vertical_idx, slash_idx, (const int32_t *)workspace,
                        block_count, block_offset, column_count, column_index, heads, rows, nnz_v, nnz_s,
                        zero_fill, error_flag, total);
