@@ -215,8 +215,8 @@ int minf_dense_attn_fwd(const minf_qkvo *t, void *stream);
  *   (slash[j] is the mass on the diagonal with offset n-1-j);
  *   then vertical[..., :force_vertical] = +inf and slash[..., n-force_slash:] = +inf
  *   (the reference forces 30 and 100; pass 0 to get the raw sums).
- * q [batch, heads_q, n, 128], k [batch, heads_kv, n, 128] as base pointer +
- * element strides {batch, head, token}; last_q <= 64 (clamped to n).
+ * q [batch, heads_q, n, head_dim], k [batch, heads_kv, n, head_dim] (head_dim 64 or 128) as base
+ * pointer + element strides {batch, head, token}; last_q <= 64 (clamped to n).
  * vertical, slash: [batch, heads_q, n] fp32, contiguous.
  * workspace: at least minf_vs_estimate_workspace_bytes() bytes, 16-byte aligned.
  */
@@ -306,7 +306,8 @@ int minf_topk_indices_pair_ragged(const float *scores_a, const int32_t *k_rows_a
  * force_diag_first != 0 additionally keeps the diagonal block and block 0 of every query block.
  *   rows = minf_bs_block_index_rows(n) = (n + 64 - n%64) / 64
  *   block_index [batch, heads_q, rows, min(top_k, rows)] int32, contiguous
- *   q [batch, heads_q, n, 128], k [batch, heads_kv, n, 128]: base pointer + element strides
+ *   q [batch, heads_q, n, head_dim], k [batch, heads_kv, n, head_dim] (head_dim 64 or 128): base
+ *   pointer + element strides
  *   workspace: minf_bs_block_index_workspace_bytes() bytes, 16-byte aligned
  */
 int minf_bs_block_index_rows(int n);

@@ -33,8 +33,9 @@ constexpr int HD = 128;
 constexpr int BLK = 64;
 
 struct PoolParams {
-    const char *x;            // [batch, heads, n, 128] 16-bit, element strides below
+    const char *x;            // [batch, heads, n, hd] 16-bit, element strides below
     long long xs[3];
+    int hd;                   // 64 or 128 input dims; the pooled rows are always 128 wide (zeros above hd)
     float *out;               // [batch*heads, rows, 128] fp32
     int heads, n, rows;
     int blk;                  // tokens per block: 64 or 32
@@ -69,7 +70,7 @@ template <typename T> __global__ __launch_bounds__(256) void bs_pool_kernel(cons
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const int tok = blk * p.blk + r4 + 16 * j;
-        if (16 * j < p.blk && tok < p.n) {
+        if (16 * j < p.blk && tok < p.n && c * 8 < p.hd) {
             const u32x4_t raw = *reinterpret_cast<const u32x4_t *>(base + (long long)tok * p.xs[2] * 2 + c * 16);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -177,7 +178,7 @@ int block_index_impl(const void *q, const void *k, const int64_t *q_stride, cons
     if (!head_list) index_heads = heads_q;
     if (batch < 0 || heads_q <= 0 || heads_kv <= 0 || n <= 0 || top_k <= 0) return MINF_ERR_INVALID_ARG;
     if (heads_q % heads_kv != 0) return MINF_ERR_INVALID_ARG;
-    if (head_dim != HD) return MINF_ERR_UNSUPPORTED;
+    if (head_dim != HD && head_dim != 64) return MINF_ERR_UNSUPPORTED;
     if (dtype != MINF_BF16 && dtype != MINF_F16) return MINF_ERR_UNSUPPORTED;
     if (((uintptr_t)q | (uintptr_t)k) & 15) return MINF_ERR_ALIGNMENT;
     for (int i = 0; i < 3; ++i)
@@ -196,8 +197,8 @@ int block_index_impl(const void *q, const void *k, const int64_t *q_stride, cons
     float *scores = (float *)ws;
     hipStream_t st = (hipStream_t)stream;
 
-    PoolParams pq{(const char *)q, {q_stride[0], q_stride[1], q_stride[2]}, qp, heads_q, n, rows, blk, head_list, index_heads};
-    PoolParams pk{(const char *)k, {k_stride[0], k_stride[1], k_stride[2]}, kp, heads_kv, n, rows, blk, nullptr, heads_kv};
+    PoolParams pq{(const char *)q, {q_stride[0], q_stride[1], q_stride[2]}, head_dim, qp, heads_q, n, rows, blk, head_list, index_heads};
+    PoolParams pk{(const char *)k, {k_stride[0], k_stride[1], k_stride[2]}, head_dim, kp, heads_kv, n, rows, blk, nullptr, heads_kv};
     if (dtype == MINF_BF16) {
         hipLaunchKernelGGL(bs_pool_kernel<__bf16>, dim3(rows, batch * index_heads), dim3(256), 0, st, pq);
         hipLaunchKernelGGL(bs_pool_kernel<__bf16>, dim3(rows, batch * heads_kv), dim3(256), 0, st, pk);

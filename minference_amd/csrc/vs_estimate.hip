@@ -30,6 +30,7 @@
 // before its fp32 softmax).
 #include "minf_common.h"
 #include <math.h>
+#include <type_traits>
 
 namespace {
 
@@ -42,7 +43,6 @@ constexpr int LQ = 64;          // query rows held per head (last_q <= LQ)
 constexpr int KC = 2048;        // keys per workgroup
 constexpr int EST_THREADS = 256;
 constexpr int WIN = KC + LQ;    // diagonal window of one chunk
-constexpr int HD = 128;
 
 struct EstParams {
     const char *q, *k;
@@ -103,7 +103,8 @@ __device__ __forceinline__ WgId decode_wg(const EstParams &p, int wave, bool rev
 }
 
 // Q fragments of one head: rows N-last_q+i, i = 32*blk + lane%32, d = 16*ks + 8*(lane/32) + 0..7
-__device__ __forceinline__ void load_q(const EstParams &p, const WgId &w, int lane, Frag (&qf)[2][8]) {
+template <int KS>
+__device__ __forceinline__ void load_q(const EstParams &p, const WgId &w, int lane, Frag (&qf)[2][KS]) {
     const int l32 = lane & 31, g = lane >> 5;
     const char *qb = p.q + ((long long)w.b * p.qs[0] + (long long)w.h * p.qs[1]) * 2;
 #pragma unroll
@@ -112,22 +113,24 @@ __device__ __forceinline__ void load_q(const EstParams &p, const WgId &w, int la
         const int row = min(max(p.n - p.last_q + i, 0), p.n - 1);
         const char *rp = qb + (long long)row * p.qs[2] * 2 + g * 16;
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) qf[blk][ks].u = *reinterpret_cast<const u32x4_t *>(rp + ks * 32);
+        for (int ks = 0; ks < KS; ++ks) qf[blk][ks].u = *reinterpret_cast<const u32x4_t *>(rp + ks * 32);
     }
 }
 
 // K fragments of one 32-key block starting at key c0 (rows clamped to n-1)
-__device__ __forceinline__ void load_k(const EstParams &p, const char *kb, int c0, int lane, Frag (&kf)[8]) {
+template <int KS>
+__device__ __forceinline__ void load_k(const EstParams &p, const char *kb, int c0, int lane, Frag (&kf)[KS]) {
     const int l32 = lane & 31, g = lane >> 5;
     const int row = min(c0 + l32, p.n - 1);
     const char *rp = kb + (long long)row * p.ks[2] * 2 + g * 16;
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) kf[ks].u = *reinterpret_cast<const u32x4_t *>(rp + ks * 32);
+    for (int ks = 0; ks < KS; ++ks) kf[ks].u = *reinterpret_cast<const u32x4_t *>(rp + ks * 32);
 }
 
 // ---------------------------------------------------------------- stats sweep
-template <typename T>
+template <typename T, int HD>
 __global__ __launch_bounds__(EST_THREADS, 3) void est_stats_kernel(const EstParams p) {
+    constexpr int KS = HD / 16;       // k-steps of one 32x32 score block
     __shared__ float lds_m[4][LQ], lds_l[4][LQ];
     const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const WgId w = decode_wg(p, wave, false);
@@ -139,17 +142,17 @@ __global__ __launch_bounds__(EST_THREADS, 3) void est_stats_kernel(const EstPara
     float m_run[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.f, 0.f};
     if (w.wave_valid) {
     const char *kb = p.k + ((long long)w.b * p.ks[0] + (long long)w.hkv * p.ks[1]) * 2;
-    Frag qf[2][8];
+    Frag qf[2][KS];
     load_q(p, w, lane, qf);
     const int key_begin = w.chunk * KC + w.kq * klen;
     const int qpos0 = p.n - p.last_q;          // absolute position of query row 0
-    Frag kf[8], kn[8];
+    Frag kf[KS], kn[KS];
     load_k(p, kb, key_begin, lane, kn);
     for (int blk = 0; blk < klen / 32; ++blk) {
         const int c0 = key_begin + blk * 32;
         if (c0 >= p.n) break;
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) kf[ks] = kn[ks];
+        for (int ks = 0; ks < KS; ++ks) kf[ks] = kn[ks];
         load_k(p, kb, min(c0 + 32, p.n - 1), lane, kn);      // next block, in flight during this one
         f32x16_t st[2];
 #pragma unroll
@@ -157,7 +160,7 @@ __global__ __launch_bounds__(EST_THREADS, 3) void est_stats_kernel(const EstPara
 #pragma unroll
             for (int r = 0; r < 16; ++r) st[nb][r] = 0.f;
 #pragma unroll
-            for (int ks = 0; ks < 8; ++ks) st[nb] = mma<T>(kf[ks], qf[nb][ks], st[nb]);
+            for (int ks = 0; ks < KS; ++ks) st[nb] = mma<T>(kf[ks], qf[nb][ks], st[nb]);
         }
         const bool edge = c0 + 31 > qpos0 || c0 + 32 > p.n;
 #pragma unroll
@@ -247,8 +250,9 @@ constexpr int WWIN = KC + LQ;                // per-wave diagonal window: at mos
 
 // (min 2 waves per SIMD: caps the kernel at 256 registers; it is latency bound and one resident
 // wave per SIMD ran 1.4x slower)
-template <typename T>
+template <typename T, int HD>
 __global__ __launch_bounds__(EST_THREADS, 2) void est_scores_kernel(const EstParams p) {
+    constexpr int KS = HD / 16;
     // the four waves' tiles overlap in their zero rows: wave w starts 63 rows after wave w-1
     __shared__ float lds_tile[(3 * 63 + TROWS) * TP];
     __shared__ float lds_wwin[4][WWIN];
@@ -268,7 +272,7 @@ __global__ __launch_bounds__(EST_THREADS, 2) void est_scores_kernel(const EstPar
 
     if (w.wave_valid) {
     const char *kb = p.k + ((long long)w.b * p.ks[0] + (long long)w.hkv * p.ks[1]) * 2;
-    Frag qf[2][8];
+    Frag qf[2][KS];
     load_q(p, w, lane, qf);
     // lane <-> key; reg r of block mb <-> query row i = 32*mb + 8*(r/4) + 4*g + r%4
     float mrow[2][16];
@@ -282,13 +286,13 @@ __global__ __launch_bounds__(EST_THREADS, 2) void est_scores_kernel(const EstPar
     const int qpos0 = p.n - p.last_q;
     const int rshift = LQ - p.last_q;          // rows are indexed as if last_q were 64
     float *vout = p.vertical + bh * p.n;
-    Frag kf[8], kn[8];
+    Frag kf[KS], kn[KS];
     load_k(p, kb, key_begin, lane, kn);
     for (int blk = 0; blk < klen / 32; ++blk) {
         const int c0 = key_begin + blk * 32;
         if (c0 >= p.n) break;
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) kf[ks] = kn[ks];
+        for (int ks = 0; ks < KS; ++ks) kf[ks] = kn[ks];
         load_k(p, kb, min(c0 + 32, p.n - 1), lane, kn);      // next block, in flight during this one
         const int c = c0 + l32;                 // this lane's key
         const bool edge = c0 + 31 > qpos0 || c0 + 32 > p.n;
@@ -299,7 +303,7 @@ __global__ __launch_bounds__(EST_THREADS, 2) void est_scores_kernel(const EstPar
 #pragma unroll
             for (int r = 0; r < 16; ++r) sc[r] = 0.f;
 #pragma unroll
-            for (int ks = 0; ks < 8; ++ks) sc = mma<T>(qf[mb][ks], kf[ks], sc);
+            for (int ks = 0; ks < KS; ++ks) sc = mma<T>(qf[mb][ks], kf[ks], sc);
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int il = 8 * (r >> 2) + 4 * g + (r & 3);      // row inside this 32-row half
@@ -367,7 +371,7 @@ int fill(EstParams &p, const void *q, const void *k, const int64_t *q_stride, co
     if (head_list && index_heads <= 0) return MINF_ERR_INVALID_ARG;
     if (!head_list) index_heads = heads_q;
     if (batch < 0 || heads_q <= 0 || heads_kv <= 0 || n <= 0 || heads_q % heads_kv) return MINF_ERR_INVALID_ARG;
-    if (head_dim != HD || (dtype != MINF_BF16 && dtype != MINF_F16)) return MINF_ERR_UNSUPPORTED;
+    if ((head_dim != 128 && head_dim != 64) || (dtype != MINF_BF16 && dtype != MINF_F16)) return MINF_ERR_UNSUPPORTED;
     if (last_q < 1 || last_q > LQ || force_v < 0 || force_s < 0) return MINF_ERR_INVALID_ARG;
     if (((uintptr_t)q & 15) || ((uintptr_t)k & 15)) return MINF_ERR_ALIGNMENT;
     for (int j = 0; j < 3; ++j)
@@ -423,11 +427,22 @@ static int estimate_launch(const void *q, const void *k, const int64_t *q_stride
     if (grid > 0x7fffffffLL) return MINF_ERR_UNSUPPORTED;
     hipStream_t s = (hipStream_t)stream;
     const long long bh = (long long)batch * p.index_heads;       // heads of the outputs
-    if (dtype == MINF_BF16) hipLaunchKernelGGL(est_stats_kernel<__bf16>, dim3((unsigned)grid), dim3(EST_THREADS), 0, s, p);
-    else hipLaunchKernelGGL(est_stats_kernel<_Float16>, dim3((unsigned)grid), dim3(EST_THREADS), 0, s, p);
+    const bool bf = dtype == MINF_BF16;
+    const dim3 g((unsigned)grid), b(EST_THREADS);
+    auto sweep = [&](auto stats_not_scores) {
+        constexpr bool STATS = decltype(stats_not_scores)::value;
+        auto go = [&](auto kern) { hipLaunchKernelGGL(kern, g, b, 0, s, p); };
+        if constexpr (STATS) {
+            if (head_dim == 128) { if (bf) go(est_stats_kernel<__bf16, 128>); else go(est_stats_kernel<_Float16, 128>); }
+            else                 { if (bf) go(est_stats_kernel<__bf16, 64>);  else go(est_stats_kernel<_Float16, 64>); }
+        } else {
+            if (head_dim == 128) { if (bf) go(est_scores_kernel<__bf16, 128>); else go(est_scores_kernel<_Float16, 128>); }
+            else                 { if (bf) go(est_scores_kernel<__bf16, 64>);  else go(est_scores_kernel<_Float16, 64>); }
+        }
+    };
+    sweep(std::true_type{});
     hipLaunchKernelGGL(est_reduce_kernel, dim3((unsigned)bh), dim3(LQ), 0, s, p);
-    if (dtype == MINF_BF16) hipLaunchKernelGGL(est_scores_kernel<__bf16>, dim3((unsigned)grid), dim3(EST_THREADS), 0, s, p);
-    else hipLaunchKernelGGL(est_scores_kernel<_Float16>, dim3((unsigned)grid), dim3(EST_THREADS), 0, s, p);
+    sweep(std::false_type{});
     hipLaunchKernelGGL(est_finalize_kernel, dim3((unsigned)((n + 255) / 256), (unsigned)bh), dim3(256), 0, s, p);
     return minf_launch_status();
 }

@@ -12,7 +12,7 @@ from __future__ import annotations
 import torch
 
 from . import _lib
-from .ops import _check_qkv, _narrow_fp32, _prep
+from .ops import _NATIVE_D, _check_qkv, _narrow_fp32, _prep
 
 LAST_Q = 64            # minference_forward.py:41
 FORCE_VERTICAL = 30    # :606
@@ -24,12 +24,13 @@ def _prep16(q, k):
         q, k = _narrow_fp32(q, k)          # fp16 when the values fit, else bf16
     elif q.dtype not in (torch.bfloat16, torch.float16):
         raise ValueError(f"unsupported dtype {q.dtype}")
-    if q.shape[-1] != 128:
-        if q.shape[-1] > 128:
-            raise ValueError("head_dim > 128 is not supported")
-        pad = 128 - q.shape[-1]
-        q = torch.nn.functional.pad(q, [0, pad])
-        k = torch.nn.functional.pad(k, [0, pad])
+    d = q.shape[-1]
+    if d > max(_NATIVE_D):
+        raise ValueError(f"head_dim > {max(_NATIVE_D)} is not supported")
+    dk = min(x for x in _NATIVE_D if x >= d)          # the kernels are built for head_dim 64 and 128
+    if d != dk:
+        q = torch.nn.functional.pad(q, [0, dk - d])
+        k = torch.nn.functional.pad(k, [0, dk - d])
     return _prep(q), _prep(k)
 
 
@@ -52,7 +53,7 @@ def vertical_slash_scores(q, k, last_q=LAST_Q, force_vertical=FORCE_VERTICAL, fo
     with torch.cuda.device(dev):
         st = lib.minf_vs_estimate(
             q16.data_ptr(), k16.data_ptr(), i64x3(*q16.stride()[:3]), i64x3(*k16.stride()[:3]),
-            B, H, Hk, N, 128, _lib.MINF_BF16 if q16.dtype == torch.bfloat16 else _lib.MINF_F16,
+            B, H, Hk, N, q16.shape[-1], _lib.MINF_BF16 if q16.dtype == torch.bfloat16 else _lib.MINF_F16,
             float(head_dim) ** -0.5, int(last_q), int(force_vertical), int(force_slash),
             vertical.data_ptr(), slash.data_ptr(), ws.data_ptr(), ws_bytes, _lib.stream_ptr(dev))
     _lib.check(st, "minf_vs_estimate")

@@ -23,7 +23,7 @@ import torch
 from . import _lib
 from .index import convert_vertical_slash_indexes
 
-_SUPPORTED_D = 128            # head_dim of the estimation / block-index kernels, largest of the tile engine
+_SUPPORTED_D = 128            # largest head_dim
 _NATIVE_D = (64, 128)         # head_dims the tile engine is instantiated for; others are zero-padded up
 
 
@@ -68,7 +68,7 @@ class _Call:
     """Holds the (possibly cast/padded) tensors of one operator call and the
     filled ``minf_qkvo`` struct."""
 
-    def __init__(self, q, k, v, seqlens=None, need_out=True, pad_to=None):
+    def __init__(self, q, k, v, seqlens=None, need_out=True):
         _check_qkv(q, k, v)
         self.out_dtype = q.dtype
         self.head_dim = q.shape[-1]
@@ -81,8 +81,8 @@ class _Call:
         if D > _SUPPORTED_D:
             raise ValueError(f"head_dim {D} > {_SUPPORTED_D} is not supported")
         # the reference runs head_dim 16, 32, 64, 128 (pit_sparse_flash_attention_v2.py:172); here 64 and
-        # 128 are native, anything else is zero-padded to the next of the two (or to `pad_to`)
-        Dk = pad_to if pad_to else min(d for d in _NATIVE_D if d >= D)
+        # 128 are native, anything else is zero-padded to the next of the two
+        Dk = min(d for d in _NATIVE_D if d >= D)
         if D < Dk:
             # zero columns change neither q.k nor the first D output columns
             pad = Dk - D
@@ -194,7 +194,7 @@ def _build_block_index(query, key, top_k, block_size_M=64, block_size_N=64, forc
     rows = (n + 64 - n % 64) / 64, every row ascending."""
     if block_size_M != 64 or block_size_N != 64:
         raise ValueError("only 64x64 blocks are supported")
-    c = _Call(query, key, key, need_out=False, pad_to=_SUPPORTED_D)   # the block-index kernels take head_dim 128
+    c = _Call(query, key, key, need_out=False)
     lib = _lib.load()
     rows = lib.minf_bs_block_index_rows(c.N)
     kk = min(int(top_k), rows)
@@ -207,7 +207,7 @@ def _build_block_index(query, key, top_k, block_size_M=64, block_size_N=64, forc
     ks = (ctypes.c_int64 * 3)(*c.k.stride()[:3])
     with torch.cuda.device(c.q.device):
         st = lib.minf_bs_block_index(c.q.data_ptr(), c.k.data_ptr(), qs, ks, c.B, c.H, c.Hk, c.N,
-                                     _SUPPORTED_D, c.struct.dtype, int(top_k), int(bool(force_diag_first)),
+                                     c.kernel_dim, c.struct.dtype, int(top_k), int(bool(force_diag_first)),
                                      out.data_ptr(), ws.data_ptr(), ws_bytes, _lib.stream_ptr(c.q.device))
     _lib.check(st, "minf_bs_block_index")
     return out

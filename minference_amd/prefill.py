@@ -77,18 +77,15 @@ def _mixed_layer(query_states, key_states, value_states, plan):
     The reference runs one operator call per head here (minference_forward.py:657-667)."""
     from . import _lib
     from .estimate import FORCE_SLASH, FORCE_VERTICAL, LAST_Q
-    from .ops import _Call, _SUPPORTED_D
+    from .ops import _Call
     import ctypes
     B, H, N, D = query_states.shape
     dev = query_states.device
     c = _Call(query_states, key_states, value_states)
-    # the estimation and block-index kernels take head_dim 128: a zero-padded q/k for them when the
-    # tile engine runs the model's head_dim natively
-    ce = c if c.kernel_dim == _SUPPORTED_D else _Call(query_states, key_states, key_states, need_out=False, pad_to=_SUPPORTED_D)
     lib = _lib.load()
     stream = _lib.stream_ptr(dev)
     i64x3 = _lib.c_i64 * 3
-    qs, ks = i64x3(*ce.q.stride()[:3]), i64x3(*ce.k.stride()[:3])
+    qs, ks = i64x3(*c.q.stride()[:3]), i64x3(*c.k.stride()[:3])
     rows = (N + 63) // 64
     keep = []                                             # tensors the enqueued kernels still read
 
@@ -115,7 +112,7 @@ def _mixed_layer(query_states, key_states, value_states, plan):
             slash = torch.empty((B, nh, N), dtype=torch.float32, device=dev)
             ws_bytes = lib.minf_vs_estimate_workspace_bytes(B, nh, N)
             ws = torch.empty((ws_bytes + 15) // 16 * 16, dtype=torch.uint8, device=dev)
-            st = lib.minf_vs_estimate_heads(ce.q.data_ptr(), ce.k.data_ptr(), qs, ks, B, H, c.Hk, N, _SUPPORTED_D,
+            st = lib.minf_vs_estimate_heads(c.q.data_ptr(), c.k.data_ptr(), qs, ks, B, H, c.Hk, N, c.kernel_dim,
                                             c.struct.dtype, float(D) ** -0.5, LAST_Q, FORCE_VERTICAL, FORCE_SLASH,
                                             slot.data_ptr(), nh, vertical.data_ptr(), slash.data_ptr(),
                                             ws.data_ptr(), ws_bytes, stream)
@@ -145,7 +142,7 @@ def _mixed_layer(query_states, key_states, value_states, plan):
             ws_bytes = lib.minf_bs_block_index_workspace_bytes(B, nh, c.Hk, N)
             ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
             bi = torch.empty((B, nh, brows, kk), dtype=torch.int32, device=dev)
-            st = lib.minf_bs_block_index_heads(ce.q.data_ptr(), ce.k.data_ptr(), qs, ks, B, H, c.Hk, N, _SUPPORTED_D,
+            st = lib.minf_bs_block_index_heads(c.q.data_ptr(), c.k.data_ptr(), qs, ks, B, H, c.Hk, N, c.kernel_dim,
                                                c.struct.dtype, 100, 0, slot.data_ptr(), nh, bi.data_ptr(),
                                                ws.data_ptr(), ws_bytes, stream)
             _lib.check(st, "minf_bs_block_index_heads")
@@ -161,7 +158,6 @@ def _mixed_layer(query_states, key_states, value_states, plan):
                 _lib.check(st, "minf_ashape_attn_fwd")
             keep.append(slot)
     c.select_heads(None)
-    keep.append(ce)
     out = c.result()
     # torch's caching allocator hands a freed block only to work enqueued later on the same stream, so
     # dropping `keep` here is safe for kernels that are still running

@@ -78,7 +78,7 @@ def test_argument_validation_of_the_index_estimate_and_search_entry_points(lib):
     assert lib.minf_vs_estimate(P, P, i3, i3, 1, 4, 4, 64, 128, 0, 0.1, 64, 30, 100, P, P, P, 16, None) == -4
     assert lib.minf_vs_estimate(P, P, bad, i3, 1, 4, 4, 64, 128, 0, 0.1, 64, 30, 100, P, P, P, 1 << 30, None) == -3
     assert lib.minf_vs_estimate(P, P, i3, i3, 1, 4, 4, 64, 128, 0, 0.1, 65, 30, 100, P, P, P, 1 << 30, None) == -1
-    assert lib.minf_vs_estimate(P, P, i3, i3, 1, 4, 4, 64, 64, 0, 0.1, 64, 30, 100, P, P, P, 1 << 30, None) == -2
+    assert lib.minf_vs_estimate(P, P, i3, i3, 1, 4, 4, 64, 96, 0, 0.1, 64, 30, 100, P, P, P, 1 << 30, None) == -2
     # block index: head counts, head_dim, workspace
     assert lib.minf_bs_block_index(P, P, i3, i3, 1, 4, 3, 64, 128, 0, 10, 0, P, P, 1 << 30, None) == -1
     assert lib.minf_bs_block_index(P, P, i3, i3, 1, 4, 4, 64, 256, 0, 10, 0, P, P, 1 << 30, None) == -2

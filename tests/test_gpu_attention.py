@@ -239,7 +239,7 @@ def test_head_dim_64_runs_natively(gpu, monkeypatch, dtype, n, hq, hk):
     out = M.vertical_slash_sparse_attention(qg, kg, vg, v_idx.to(gpu), s_idx.to(gpu))
     check(out, O.vertical_slash_sparse_attention(q, ke, ve, v_idx, s_idx), "d64 vertical-slash")
     monkeypatch.setattr(torch.nn.functional, "pad", real_pad)
-    # block-sparse: the index comes from the oracle (the block-index kernels take head_dim 128)
+    # block-sparse on an index from the oracle
     pad = 64 - (n & 63)
     bi = O.bs_block_index(real_pad(q, [0, 0, 0, pad]), real_pad(ke, [0, 0, 0, pad]), 5)
     out = M.block_sparse_attention_from_index(qg, kg, vg, bi.contiguous().to(gpu))
@@ -247,14 +247,20 @@ def test_head_dim_64_runs_natively(gpu, monkeypatch, dtype, n, hq, hk):
     check(out, ref, "d64 block-sparse")
 
 
-def test_head_dim_64_long_lists_and_the_whole_path(gpu):
+def test_head_dim_64_long_lists_and_the_whole_path(gpu, monkeypatch):
     """head_dim 64 at 20000 tokens through estimate -> top-k -> index -> attention (lists long enough
     for the paired walk's common / leftover split and several gathered tiles per row block), and the
-    block_sparse operator end to end; sampled against the oracle on the indices the GPU produced."""
+    block_sparse operator end to end (pooled block index included), none of it on zero-padded copies;
+    sampled against the oracle on the indices the GPU produced, and the block index against the
+    oracle's scores."""
     import minference_amd as M
     n, hq, hk = 20000 + 13, 4, 2
     q, k, v = make(1, hq, hk, n, 77, torch.bfloat16, d=64)
     qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
+
+    def no_pad(*a, **kw):
+        raise AssertionError("head_dim 64 must not be zero-padded")
+    monkeypatch.setattr(torch.nn.functional, "pad", no_pad)
     v_idx, s_idx = M.estimate_vertical_slash(qg, kg, 700, 900)
     out = M.vertical_slash_sparse_attention(qg, kg, vg, v_idx, s_idx)
     for h in (0, 3):
@@ -352,14 +358,15 @@ def _oracle_block_scores(q, k, hq, force):
     return p
 
 
-@pytest.mark.parametrize("n,top_k,hq,hk,force,dtype", [
-    (1024, 4, 2, 2, False, torch.bfloat16), (2000, 8, 4, 2, False, torch.bfloat16),
-    (640, 100, 1, 1, False, torch.float16), (4160, 16, 8, 2, True, torch.bfloat16),
-    (63, 3, 2, 1, False, torch.bfloat16), (8192, 100, 2, 1, True, torch.bfloat16)])
-def test_block_index_kernel_vs_oracle(gpu, n, top_k, hq, hk, force, dtype):
+@pytest.mark.parametrize("n,top_k,hq,hk,force,dtype,d", [
+    (1024, 4, 2, 2, False, torch.bfloat16, 128), (2000, 8, 4, 2, False, torch.bfloat16, 128),
+    (640, 100, 1, 1, False, torch.float16, 128), (4160, 16, 8, 2, True, torch.bfloat16, 128),
+    (63, 3, 2, 1, False, torch.bfloat16, 128), (8192, 100, 2, 1, True, torch.bfloat16, 128),
+    (2000, 8, 4, 2, False, torch.bfloat16, 64), (4160, 16, 2, 1, True, torch.float16, 64)])
+def test_block_index_kernel_vs_oracle(gpu, n, top_k, hq, hk, force, dtype, d):
     from minference_amd.ops import _build_block_index
-    print(f"case block-index n={n} top_k={top_k} hq={hq} hk={hk} force={force}", flush=True)
-    q, k, _ = make(1, hq, hk, n, 40, dtype)
+    print(f"case block-index n={n} top_k={top_k} hq={hq} hk={hk} force={force} d={d}", flush=True)
+    q, k, _ = make(1, hq, hk, n, 40, dtype, d=d)
     bi = _build_block_index(q.to(gpu), k.to(gpu), top_k, force_diag_first=force)
     R = (n + 64 - (n & 63)) // 64
     assert tuple(bi.shape) == (1, hq, R, min(top_k, R)) and bi.dtype == torch.int32

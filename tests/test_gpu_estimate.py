@@ -13,16 +13,23 @@ def expand(x, hq):
     return x.repeat_interleave(hq // x.shape[1], dim=1)
 
 
-@pytest.mark.parametrize("n,hq,hk,dtype", [
-    (64, 1, 1, torch.bfloat16), (100, 2, 1, torch.bfloat16), (1024, 4, 2, torch.bfloat16),
-    (3000, 2, 2, torch.float16), (5000, 4, 1, torch.bfloat16), (40, 1, 1, torch.bfloat16),
+@pytest.mark.parametrize("n,hq,hk,dtype,d", [
+    (64, 1, 1, torch.bfloat16, 128), (100, 2, 1, torch.bfloat16, 128), (1024, 4, 2, torch.bfloat16, 128),
+    (3000, 2, 2, torch.float16, 128), (5000, 4, 1, torch.bfloat16, 128), (40, 1, 1, torch.bfloat16, 128),
+    (100, 2, 1, torch.bfloat16, 64), (3000, 4, 2, torch.float16, 64), (5000, 4, 1, torch.bfloat16, 64),
+    (700, 2, 2, torch.bfloat16, 32),
 ])
-def test_scores_vs_oracle(gpu, n, hq, hk, dtype):
+def test_scores_vs_oracle(gpu, monkeypatch, n, hq, hk, dtype, d):
     from minference_amd.estimate import vertical_slash_scores
-    print(f"case est n={n} hq={hq} hk={hk} {dtype}", flush=True)
-    q, k, _ = gen.qkv(1, hq, hk, n, 128, seed=n, scale=1.0)
+    print(f"case est n={n} hq={hq} hk={hk} {dtype} d={d}", flush=True)
+    q, k, _ = gen.qkv(1, hq, hk, n, d, seed=n, scale=1.0)
     q, k = q.to(dtype), k.to(dtype)
+    if d in (64, 128):          # both are native instantiations: no zero-padded copies of q / k
+        def no_pad(*a, **kw):
+            raise AssertionError("native head_dim must not be zero-padded")
+        monkeypatch.setattr(torch.nn.functional, "pad", no_pad)
     vert, slash = vertical_slash_scores(q.to(gpu), k.to(gpu), force_vertical=0, force_slash=0)
+    monkeypatch.undo()
     rv, rs = O.estimate_scores(q, expand(k, hq))
     vert, slash = vert.cpu(), slash.cpu()
     lq = min(64, n)
