@@ -202,3 +202,73 @@ def test_config5_two_layer_llama3_8b_shape_at_262144_tokens(gpu, monkeypatch):
         err = (c["o"][m].float().cpu() - _rows_reference(c["q"][m].cpu(), c["k"], c["v"], mask)).abs()
         print(f"  max-abs {err.max().item():.3e} mean-abs {err.mean().item():.3e}", flush=True)
         assert err.max() <= 2e-2 and err.mean() <= 1e-3
+
+
+def test_vertical_slash_walks_that_are_not_split(gpu):
+    """The paired vertical-slash walk splits the two block lists of a workgroup into common entries and
+    leftovers only when both are strictly ascending, at most 2048 entries long and differ in at most
+    512 entries; everything else takes the walk in which each half follows its own list.  Three inputs
+    that force that walk, on sampled row blocks against the fp32 masked-dense oracle:
+    scattered slashes (more than 512 leftovers), one run of more than 2048 blocks, and block lists
+    handed over in descending order (the reference's kernel accepts any order,
+    pit_sparse_flash_attention_v2.py:84-117)."""
+    import minference_amd as M
+
+    def rel_check(tag, out_rows, ref_rows):
+        err = (out_rows.float().cpu() - ref_rows).abs()
+        scale = ref_rows.abs().max().item()
+        print(f"  {tag}: max-abs {err.max().item():.3e} mean-abs {err.mean().item():.3e} (max |ref| {scale:.3e})", flush=True)
+        assert err.max() <= 2e-2 * scale and err.mean() <= 1e-3 * scale, tag
+
+    def run(tag, n, hq, hk, nv, ns, vi, si, sample, seed):
+        # logits of standard deviation 2: a few dozen keys, spread over all tiles of a row's list, carry
+        # most of each row's weight, so a tile that is skipped, doubled or misplaced shows; with
+        # thousands of keys per row the outputs are small, hence the bound relative to max |ref|
+        q, k, v = gen.qkv(1, hq, hk, n, 128, seed=seed, scale=1.0)
+        q, k, v = (2.0 * q).bfloat16(), k.bfloat16(), v.bfloat16()
+        qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
+        seqlens = torch.full((1,), n, dtype=torch.int32, device=gpu)
+        v_idx, s_idx = torch.from_numpy(vi).to(gpu), torch.from_numpy(np.ascontiguousarray(si)).to(gpu)
+        bc, bo, cc, ci = M.convert_vertical_slash_indexes(seqlens, v_idx, s_idx, n, 64, 64, zero_fill=True)
+        out = M.vertical_slash_attention_from_index(qg, kg, vg, bc, bo, cc, ci, seqlens)
+        torch.cuda.synchronize()
+        for h, m in sample:
+            print(f"case {tag} head={h} row-block={m} blocks={int(bc[0, h, m])}", flush=True)
+            kv = h // (hq // hk)
+            _check_vs_row_block(f"{tag} head {h} row block {m}", out[0, h, m * 64: m * 64 + 64], q[0, h, m * 64: m * 64 + 64],
+                                k[0, kv], v[0, kv], vi[0, h].tolist(), si[0, h].tolist(),
+                                bc[0, h, m], bo[0, h, m].cpu().numpy(), cc[0, h, m], ci[0, h, m].cpu().numpy(), m, n)
+            nb, nc = int(bc[0, h, m]), int(cc[0, h, m])
+            mask = O.vs_mask_rows(nb, bo[0, h, m, :nb].tolist(), nc, ci[0, h, m, :nc].tolist(), m, n)
+            rel_check(f"{tag} head {h} row block {m} (relative)", out[0, h, m * 64: m * 64 + 64],
+                      _rows_reference(q[0, h, m * 64: m * 64 + 64], k[0, kv], v[0, kv], mask[:64]))
+        return (qg, kg, vg, seqlens, bc, bo, cc, ci, out)
+
+    # (a) 1100 uniformly drawn slashes over 128K tokens: mostly isolated blocks, so the lists of two
+    # neighbouring row blocks (one is the other moved by 64 keys) share few entries
+    n = 131072 + 64 * 3
+    vi, si = gen.vs_index_inputs(2, n, 500, 1100, seed=41)
+    rows = n // 64
+    qg, kg, vg, seqlens, bc, bo, cc, ci, out = run("scattered", n, 2, 1, 500, 1100, vi, si,
+                                                     [(0, rows - 1), (1, rows - 2), (0, 1700), (1, 1701), (1, 3)], 42)
+    la = set(bo[0, 0, rows - 2, : int(bc[0, 0, rows - 2])].tolist())
+    lb = set(bo[0, 0, rows - 1, : int(bc[0, 0, rows - 1])].tolist())
+    assert len(la - lb) > 512 and len(lb - la) > 512, (len(la - lb), len(lb - la))
+    # (c) the same lists in descending order: same mask, so the same rows within the tolerance
+    cnt = bc.long().unsqueeze(-1)
+    pos = torch.arange(bo.shape[-1], device=gpu).expand_as(bo)
+    rev = torch.where(pos < cnt, bo.gather(-1, (cnt - 1 - pos).clamp_(min=0)), bo)
+    out_rev = M.vertical_slash_attention_from_index(qg, kg, vg, bc, rev, cc, ci, seqlens)
+    err = (out_rev.float() - out.float()).abs()
+    scale = out.float().abs().max().item()
+    print(f"case descending lists: max-abs {err.max().item():.3e} (max |out| {scale:.3e})", flush=True)
+    assert err.max() <= 2e-2 * scale and err.mean() <= 1e-3 * scale
+    del qg, kg, vg, bc, bo, cc, ci, out, out_rev, rev, pos, cnt
+    torch.cuda.empty_cache()
+    # (b) slashes 37 apart over the whole context: one run per row block, more than 2048 blocks at the end
+    n = 64 * 2200
+    si = np.ascontiguousarray(np.arange(0, 37 * 3900, 37, dtype=np.int32)[::-1]).reshape(1, 1, -1)
+    vi = np.arange(0, 64, dtype=np.int32).reshape(1, 1, -1)
+    rows = n // 64
+    res = run("long run", n, 1, 1, 64, 3900, vi, si, [(0, rows - 1), (0, rows - 2), (0, 2100), (0, 5)], 43)
+    assert int(res[4].max()) > 2048
