@@ -26,9 +26,13 @@ def _check_vs_row_block(tag, out_rows, q_rows, k, v, v_list, s_list, bc_m, bo_m,
     assert int(bc_m) == len(rbo) and int(cc_m) == len(rci), tag
     assert bo_m[: len(rbo)].tolist() == rbo and ci_m[: len(rci)].tolist() == rci, tag
     mask = O.vs_mask_rows(len(rbo), rbo, len(rci), rci, m, n)
-    err = (out_rows.float().cpu() - _rows_reference(q_rows, k, v, mask[: q_rows.shape[0]])).abs()
-    print(f"  {tag}: max-abs {err.max().item():.3e} mean-abs {err.mean().item():.3e}", flush=True)
+    ref = _rows_reference(q_rows, k, v, mask[: q_rows.shape[0]])
+    err = (out_rows.float().cpu() - ref).abs()
+    scale = ref.abs().max().item()
+    print(f"  {tag}: max-abs {err.max().item():.3e} mean-abs {err.mean().item():.3e} (max |ref| {scale:.3e})", flush=True)
     assert err.max() <= 2e-2 and err.mean() <= 1e-3, tag
+    # and relative to the size of the outputs (rows that average over thousands of keys are small)
+    assert err.max() <= 2e-2 * scale and err.mean() <= 1e-3 * scale, tag
 
 
 def test_config3_index_at_524288_tokens(gpu):
@@ -214,12 +218,6 @@ def test_vertical_slash_walks_that_are_not_split(gpu):
     pit_sparse_flash_attention_v2.py:84-117)."""
     import minference_amd as M
 
-    def rel_check(tag, out_rows, ref_rows):
-        err = (out_rows.float().cpu() - ref_rows).abs()
-        scale = ref_rows.abs().max().item()
-        print(f"  {tag}: max-abs {err.max().item():.3e} mean-abs {err.mean().item():.3e} (max |ref| {scale:.3e})", flush=True)
-        assert err.max() <= 2e-2 * scale and err.mean() <= 1e-3 * scale, tag
-
     def run(tag, n, hq, hk, nv, ns, vi, si, sample, seed):
         # logits of standard deviation 2: a few dozen keys, spread over all tiles of a row's list, carry
         # most of each row's weight, so a tile that is skipped, doubled or misplaced shows; with
@@ -238,10 +236,6 @@ def test_vertical_slash_walks_that_are_not_split(gpu):
             _check_vs_row_block(f"{tag} head {h} row block {m}", out[0, h, m * 64: m * 64 + 64], q[0, h, m * 64: m * 64 + 64],
                                 k[0, kv], v[0, kv], vi[0, h].tolist(), si[0, h].tolist(),
                                 bc[0, h, m], bo[0, h, m].cpu().numpy(), cc[0, h, m], ci[0, h, m].cpu().numpy(), m, n)
-            nb, nc = int(bc[0, h, m]), int(cc[0, h, m])
-            mask = O.vs_mask_rows(nb, bo[0, h, m, :nb].tolist(), nc, ci[0, h, m, :nc].tolist(), m, n)
-            rel_check(f"{tag} head {h} row block {m} (relative)", out[0, h, m * 64: m * 64 + 64],
-                      _rows_reference(q[0, h, m * 64: m * 64 + 64], k[0, kv], v[0, kv], mask[:64]))
         return (qg, kg, vg, seqlens, bc, bo, cc, ci, out)
 
     # (a) 1100 uniformly drawn slashes over 128K tokens: mostly isolated blocks, so the lists of two

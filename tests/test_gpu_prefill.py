@@ -219,8 +219,11 @@ def test_config2_full_size_sampled_row_blocks(gpu):
         s = torch.where(torch.as_tensor(mask), s, torch.tensor(-torch.inf))
         ref = torch.softmax(s, dim=-1) @ v[0, 0].float()
         err = (out[0, h, r0:r1].float().cpu() - ref).abs()
-        print(f"  max-abs {err.max().item():.3e} mean-abs {err.mean().item():.3e}", flush=True)
+        scale = ref.abs().max().item()
+        print(f"  max-abs {err.max().item():.3e} mean-abs {err.mean().item():.3e} (max |ref| {scale:.3e})", flush=True)
         assert err.max() <= 2e-2 and err.mean() <= 1e-3
+        # and relative to the size of the outputs (rows that average over thousands of keys are small)
+        assert err.max() <= 2e-2 * scale and err.mean() <= 1e-3 * scale
 
 
 def test_one_million_tokens_sampled_row_blocks(gpu):
@@ -254,8 +257,11 @@ def test_one_million_tokens_sampled_row_blocks(gpu):
         s = torch.where(torch.as_tensor(mask), s, torch.tensor(-torch.inf))
         ref = torch.softmax(s, dim=-1) @ vf
         err = (out[0, h, r0:r1].float().cpu() - ref).abs()
-        print(f"  max-abs {err.max().item():.3e} mean-abs {err.mean().item():.3e}", flush=True)
+        scale = ref.abs().max().item()
+        print(f"  max-abs {err.max().item():.3e} mean-abs {err.mean().item():.3e} (max |ref| {scale:.3e})", flush=True)
         assert err.max() <= 2e-2 and err.mean() <= 1e-3
+        # and relative to the size of the outputs (rows that average over thousands of keys are small)
+        assert err.max() <= 2e-2 * scale and err.mean() <= 1e-3 * scale
 
 
 def _rows_reference(q_rows, k, v, mask):
@@ -298,9 +304,13 @@ def test_config4_full_size_sampled_row_blocks(gpu):
         for j in row[: min(m + 1, top_k)]:
             cols = np.arange(j * 64, min(j * 64 + 64, n))
             mask[:, cols] |= cols[None, :] <= rr[:, None]
-        err = (out[0, h, m * 64: m * 64 + 64].float().cpu() - _rows_reference(q[0, h, m * 64: m * 64 + 64], k[0, 0], v[0, 0], mask)).abs()
-        print(f"  max-abs {err.max().item():.3e} mean-abs {err.mean().item():.3e}", flush=True)
+        ref = _rows_reference(q[0, h, m * 64: m * 64 + 64], k[0, 0], v[0, 0], mask)
+        err = (out[0, h, m * 64: m * 64 + 64].float().cpu() - ref).abs()
+        scale = ref.abs().max().item()
+        print(f"  max-abs {err.max().item():.3e} mean-abs {err.mean().item():.3e} (max |ref| {scale:.3e})", flush=True)
         assert err.max() <= 2e-2 and err.mean() <= 1e-3
+        # and relative to the size of the outputs (rows that average over thousands of keys are small)
+        assert err.max() <= 2e-2 * scale and err.mean() <= 1e-3 * scale
 
 
 def test_config5_ashape_heads_full_size_sampled_row_blocks(gpu):
@@ -319,6 +329,10 @@ def test_config5_ashape_heads_full_size_sampled_row_blocks(gpu):
         r = np.arange(r0, r1)[:, None]
         c = np.arange(n)[None, :]
         mask = ((c <= r) & (c > r - n_local)) | ((c < n_init) & (c <= r - n_local))
-        err = (out[0, h, r0:r1].float().cpu() - _rows_reference(q[0, h, r0:r1], k[0, 0], v[0, 0], mask)).abs()
-        print(f"  max-abs {err.max().item():.3e} mean-abs {err.mean().item():.3e}", flush=True)
+        ref = _rows_reference(q[0, h, r0:r1], k[0, 0], v[0, 0], mask)
+        err = (out[0, h, r0:r1].float().cpu() - ref).abs()
+        scale = ref.abs().max().item()
+        print(f"  max-abs {err.max().item():.3e} mean-abs {err.mean().item():.3e} (max |ref| {scale:.3e})", flush=True)
         assert err.max() <= 2e-2 and err.mean() <= 1e-3
+        # and relative to the size of the outputs (rows that average over thousands of keys are small)
+        assert err.max() <= 2e-2 * scale and err.mean() <= 1e-3 * scale
