@@ -842,11 +842,24 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
         copy_tile(cur, k_base, k_row, std::false_type{}, gt_cur, lds_k);
     }
 
-    for (int it = 0; have_cur; ++it) {
+    // One step of the walk.  COMMON (paired vertical-slash only): this tile and the next one are both
+    // on the list of common entries -- shared, contiguous, never gathered -- so everything that deals
+    // with split steps, gathered tiles and the end of the walk drops out of the instruction stream;
+    // the general form serves every other step and every other mode.
+    auto step = [&](const int it, auto common_c) {
+        constexpr bool COMMON = decltype(common_c)::value;
         __builtin_amdgcn_s_waitcnt(0x0f70);      // vmcnt(0): this wave's part of K(it) is in LDS
         __syncthreads();
         bool have_nxt;
-        if constexpr (VSP) {
+        if constexpr (COMMON) {
+            vs_pref = vs_list(it + 2);
+            have_nxt = true;
+            nxt.gathered = 0; nxt.nvalid = BN; nxt.on_a = nxt.on_b = 1; nxt.split = 0;
+            nxt.start = vs_entry;
+            gt_nxt = 0;
+            cur.gathered = 0; cur.nvalid = BN; cur.on_a = cur.on_b = 1; cur.split = 0;
+            copy_rows(cur, v_base, v_row, std::true_type{}, 0, lds_v, std::integral_constant<int, CROWS>{}, wave_wg);
+        } else if constexpr (VSP) {
             // the merged list shares an LDS object with the V tiles: its entry is read while no copy
             // is in flight, so that the read never waits for one
             vs_pref = vs_list(it + 2);
@@ -872,7 +885,8 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
 
         // paired variant: is this tile on the list of this wave's row block ?
         bool active = true;
-        if constexpr (PAIR && (MODE == MODE_BS || MODE == MODE_VS)) active = have_rows && (half ? cur.on_b : cur.on_a);   // (split steps: on_a == on_b == own flag)
+        if constexpr (COMMON) active = have_rows;
+        else if constexpr (PAIR && (MODE == MODE_BS || MODE == MODE_VS)) active = have_rows && (half ? cur.on_b : cur.on_a);   // (split steps: on_a == on_b == own flag)
         else if constexpr (PAIR) active = have_rows && tile_on_list<MODE>(p, m, cur.start);
         f32x16_t s0, s1;
         Frag vf[4][NDB];
@@ -881,13 +895,20 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
             __builtin_amdgcn_s_waitcnt(0x0f70);      // vmcnt(0): this wave's part of V(it) is in LDS
             __syncthreads();
         }
-        if (have_nxt) copy_tile(nxt, k_base, k_row, std::false_type{}, gt_nxt, lds_k);
+        if constexpr (COMMON) copy_rows(nxt, k_base, k_row, std::false_type{}, 0, lds_k, std::integral_constant<int, CROWS>{}, wave_wg);
+        else if (have_nxt) copy_tile(nxt, k_base, k_row, std::false_type{}, gt_nxt, lds_k);
         if (active) sm_pv_block(cur, lds_v, s0, s1, vf, std::integral_constant<bool, PAIR>{});
         if constexpr (VSP) vs_entry = __builtin_amdgcn_readfirstlane(vs_pref);
         cur = nxt;
         gt_cur = gt_nxt;
         have_cur = have_nxt;
+    };
+    int it = 0;
+    if constexpr (VSP) {
+        // (a first step exists whenever there is a common entry; steps 0 .. vs_nc-2 have a common successor)
+        for (; it + 1 < vs_nc; ++it) step(it, std::true_type{});
     }
+    for (; have_cur; ++it) step(it, std::false_type{});
 
     // ---- epilogue: O = O^T / l, transposed through LDS so that every global store is 16 bytes
     // of one row and 16 lanes cover a whole 256-byte row ---------------------------------------
