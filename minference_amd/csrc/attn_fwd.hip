@@ -53,8 +53,9 @@
 //  * index entries (block offsets, column counts) are wave-uniform and read through the constant
 //    address space, i.e. scalar loads that do not queue behind the vector memory traffic; gathered
 //    column ids are fetched one per lane an iteration ahead and distributed with wave shuffles;
-//  * the running max is only raised when a tile exceeds it by more than 2^8 (probabilities stay
-//    below 2^8, far inside fp32/bf16 range), so most tiles skip the O^T rescale;
+//  * the running max is only raised when a tile exceeds it by more than 2^20 (bf16; 2^8 for f16
+//    operands, whose probabilities must stay inside the f16 range), so nearly all tiles skip the
+//    O^T rescale;
 //  * the cross-half max uses v_permlane32_swap, the row sums v_dot2 on the rounded probabilities
 //    (the same values the second MFMA consumes);
 //  * s_setprio raises the wave while it issues MFMAs;
@@ -86,6 +87,9 @@ constexpr int VALU_PER_MFMA = 6;
 // 2-wave kernel: the second barrier of a tile comes after this k-step of the QK loop (all K
 // fragments have been read by then), and the V^T fragment reads follow it under the last MFMAs
 constexpr int EARLY_B2 = 5;
+#ifndef LAZY_MAX_BF16
+#define LAZY_MAX_BF16 20.0f
+#endif
 constexpr int VALU_MASK = 0x402;             // sched_group_barrier classes: VALU | transcendental
 
 struct AttnParams {
@@ -779,7 +783,11 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
         }
         { const unsigned u = __float_as_uint(mx); auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false); mx = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1])); }
         const float cand = mx * p.scale_log2;
-        const bool grow = cand > m_i + 8.0f;
+        // lazy reference maximum: raised only when a tile exceeds it by more than LAZY_MAX powers of two
+        // (probabilities stay below 2^LAZY_MAX: 2^8 fits f16 with room for the row sums, bf16 has the
+        // exponent range of fp32)
+        constexpr float LAZY_MAX = std::is_same<T, __bf16>::value ? LAZY_MAX_BF16 : 8.0f;
+        const bool grow = cand > m_i + LAZY_MAX;
         const float m_new = grow ? cand : m_i;
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
         const float alpha = grow ? __builtin_amdgcn_exp2f(m_i - m_use) : 1.0f;
