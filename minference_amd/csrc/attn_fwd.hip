@@ -850,12 +850,20 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
         copy_tile(cur, k_base, k_row, std::false_type{}, gt_cur, lds_k);
     }
 
-    // One step of the walk.  COMMON (paired vertical-slash only): this tile and the next one are both
-    // on the list of common entries -- shared, contiguous, never gathered -- so everything that deals
-    // with split steps, gathered tiles and the end of the walk drops out of the instruction stream;
-    // the general form serves every other step and every other mode.
-    auto step = [&](const int it, auto common_c) {
-        constexpr bool COMMON = decltype(common_c)::value;
+    // One step of the walk, in three forms (the last two for paired vertical-slash lists only):
+    // general (kind 0) -- any tile, any successor, every mode;
+    // COMMON (kind 1) -- this tile and the next one are both on the list of common entries: shared,
+    // contiguous, never gathered;
+    // SPLIT (kind 2) -- this step and the next one are both split steps in which each row block
+    // visits a block entry of its own, fetched a step ahead: a leftover from the split lists in LDS
+    // or, when the lists were not split, an entry of its list in global memory (kind 2).
+    // In the two special forms everything that deals with the other cases drops out of the
+    // instruction stream (the general form costs about 1.7 times a COMMON step).
+    [[maybe_unused]] int sp_entry = 0;
+    [[maybe_unused]] const cint_ptr sp_list = as_const(p.bo) + ridx * p.nnz_s;      // this row block's list in global memory
+    auto step = [&](const int it, auto kind_c) {
+        constexpr int KIND = decltype(kind_c)::value;
+        constexpr bool COMMON = KIND == 1, SPLIT = KIND == 2;
         __builtin_amdgcn_s_waitcnt(0x0f70);      // vmcnt(0): this wave's part of K(it) is in LDS
         __syncthreads();
         bool have_nxt;
@@ -867,6 +875,16 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
             gt_nxt = 0;
             cur.gathered = 0; cur.nvalid = BN; cur.on_a = cur.on_b = 1; cur.split = 0;
             copy_rows(cur, v_base, v_row, std::true_type{}, 0, lds_v, std::integral_constant<int, CROWS>{}, wave_wg);
+        } else if constexpr (SPLIT) {
+            const int j = it - vs_nc;                      // this step's position in the leftover lists
+            if (vs_merged) vs_pref = vs_only[half * VS_ONLY_MAX + min(j + 2, VS_ONLY_MAX - 1)];
+            else vs_pref = sp_list[min(j + 2, p.nnz_s - 1)];
+            have_nxt = true;
+            nxt.gathered = 0; nxt.nvalid = BN; nxt.on_a = nxt.on_b = 1; nxt.split = 1;
+            nxt.start = sp_entry;
+            gt_nxt = 0;
+            cur.gathered = 0; cur.nvalid = BN; cur.on_a = cur.on_b = 1; cur.split = 1;
+            copy_rows(cur, v_base, v_row, std::true_type{}, 0, lds_v + half * TILE_BYTES, std::integral_constant<int, 32>{}, wave);
         } else if constexpr (VSP) {
             // the merged list shares an LDS object with the V tiles: its entry is read while no copy
             // is in flight, so that the read never waits for one
@@ -893,7 +911,7 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
 
         // paired variant: is this tile on the list of this wave's row block ?
         bool active = true;
-        if constexpr (COMMON) active = have_rows;
+        if constexpr (COMMON || SPLIT) active = have_rows;
         else if constexpr (PAIR && (MODE == MODE_BS || MODE == MODE_VS)) active = have_rows && (half ? cur.on_b : cur.on_a);   // (split steps: on_a == on_b == own flag)
         else if constexpr (PAIR) active = have_rows && tile_on_list<MODE>(p, m, cur.start);
         f32x16_t s0, s1;
@@ -904,9 +922,11 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
             __syncthreads();
         }
         if constexpr (COMMON) copy_rows(nxt, k_base, k_row, std::false_type{}, 0, lds_k, std::integral_constant<int, CROWS>{}, wave_wg);
+        else if constexpr (SPLIT) copy_rows(nxt, k_base, k_row, std::false_type{}, 0, lds_k + half * TILE_BYTES, std::integral_constant<int, 32>{}, wave);
         else if (have_nxt) copy_tile(nxt, k_base, k_row, std::false_type{}, gt_nxt, lds_k);
         if (active) sm_pv_block(cur, lds_v, s0, s1, vf, std::integral_constant<bool, PAIR>{});
-        if constexpr (VSP) vs_entry = __builtin_amdgcn_readfirstlane(vs_pref);
+        if constexpr (SPLIT) sp_entry = __builtin_amdgcn_readfirstlane(vs_pref);
+        else if constexpr (VSP) vs_entry = __builtin_amdgcn_readfirstlane(vs_pref);
         cur = nxt;
         gt_cur = gt_nxt;
         have_cur = have_nxt;
@@ -914,9 +934,28 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
     int it = 0;
     if constexpr (VSP) {
         // (a first step exists whenever there is a common entry; steps 0 .. vs_nc-2 have a common successor)
-        for (; it + 1 < vs_nc; ++it) step(it, std::true_type{});
+        for (; it + 1 < vs_nc; ++it) step(it, std::integral_constant<int, 1>{});
+        // block entries of their own that both row blocks still have (leftovers of the split, or the
+        // whole lists when they were not split): these steps run in the SPLIT form
+        const int nb_both = min(vs_na, vs_nb) - vs_nc;
+        if (nb_both >= 3 && have_cur) {
+            if (vs_nc > 0) {                               // from the last common tile to the first split step
+                step(it, std::integral_constant<int, 0>{});
+                ++it;
+            }
+            // cur is now each row block's entry 0, its K copy is on the way
+            if (!vs_shifted) {
+                vs_shifted = true;
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) k_rd_off[ks] += half * TILE_BYTES;
+#pragma unroll
+                for (int db = 0; db < NDB; ++db) v_rd_off[db] += half * TILE_BYTES;
+            }
+            sp_entry = vs_merged ? __builtin_amdgcn_readfirstlane(vs_only[half * VS_ONLY_MAX + 1]) : sp_list[1];
+            for (; it - vs_nc + 1 < nb_both; ++it) step(it, std::integral_constant<int, 2>{});
+        }
     }
-    for (; have_cur; ++it) step(it, std::false_type{});
+    for (; have_cur; ++it) step(it, std::integral_constant<int, 0>{});
 
     // ---- epilogue: O = O^T / l, transposed through LDS so that every global store is 16 bytes
     // of one row and 16 lanes cover a whole 256-byte row ---------------------------------------
