@@ -87,6 +87,9 @@ constexpr int VALU_PER_MFMA = 6;
 // 2-wave kernel: the second barrier of a tile comes after this k-step of the QK loop (all K
 // fragments have been read by then), and the V^T fragment reads follow it under the last MFMAs
 constexpr int EARLY_B2 = 5;
+#ifndef MAX_PERIOD
+#define MAX_PERIOD 8      // (a power of two) the row maximum is recomputed at least every MAX_PERIOD tiles
+#endif
 #ifndef LAZY_MAX_BF16
 #define LAZY_MAX_BF16 20.0f
 #endif
@@ -269,8 +272,26 @@ __device__ __forceinline__ bool tile_on_list(const AttnParams &p, int m, int sta
     return ti >= t_lo || ti < ((p.n_init + BN - 1) >> 6);
 }
 
-template <typename T, int MODE, bool PAIR, int HD>
-__global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_kernel(const AttnParams p) {
+// LDS of one workgroup (declared by the kernel, see attn_fwd_kernel): separate objects, so that the
+// compiler lets reads of one overtake copies into the other.
+template <int MODE, bool PAIR, int HD> struct AttnLds {
+    static constexpr bool VSP = PAIR && MODE == MODE_VS;
+    static constexpr int TILE_BYTES = BN * HD * 2;
+    static constexpr int NK = (VSP ? 2 : 1) * TILE_BYTES;
+    static constexpr int NLIST = PAIR && MODE == MODE_BS ? 2 * BS_PAIR_MAX : 1;
+    static constexpr int NONLY = VSP ? 2 * VS_ONLY_MAX : 1;
+};
+
+// The whole walk of one workgroup.  EVERY_MAX: the row maximum is computed for every tile; otherwise
+// only where it is needed (see sm_pv_block), and the function returns true -- for the whole
+// workgroup -- when a row sum left the safe range, i.e. when the walk has to be run again with
+// EVERY_MAX (the output it wrote is then overwritten).
+template <typename T, int MODE, bool PAIR, int HD, bool EVERY_MAX>
+__device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[AttnLds<MODE, PAIR, HD>::NK],
+                                          char (&lds_v)[AttnLds<MODE, PAIR, HD>::NK],
+                                          int (&lds_list)[AttnLds<MODE, PAIR, HD>::NLIST],
+                                          int (&vs_only)[AttnLds<MODE, PAIR, HD>::NONLY], int (&vs_wsum)[4], int &vs_bad,
+                                          int &lds_redo) {
     static_assert(HD == 128 || HD == 64, "head_dim 128 or 64");
     constexpr int ROW_BYTES = HD * 2;                       // one token row of K / V / Q / O
     constexpr int KS = HD / 16;                             // k-steps of S^T = K.Q^T
@@ -287,12 +308,9 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
     constexpr bool VSP = PAIR && MODE == MODE_VS;
     constexpr int TILE_BYTES = BN * ROW_BYTES;
     constexpr int VS_PAIR_MAX = TILE_BYTES / 8;             // both staged lists fit the second K tile
-    // separate LDS objects: the compiler then lets reads of one overtake copies into the other
     // paired vertical-slash: a second K and V tile (row block B's buffers in the steps in which each
     // row block has a tile of its own); before that, the second K tile stages the two block lists and
     // the second V tile holds their merge
-    __shared__ __attribute__((aligned(16))) char lds_k[(VSP ? 2 : 1) * TILE_BYTES];
-    __shared__ __attribute__((aligned(16))) char lds_v[(VSP ? 2 : 1) * TILE_BYTES];
     char *const lds_k1 = lds_k + (VSP ? TILE_BYTES : 0);
     char *const lds_v1 = lds_v + (VSP ? TILE_BYTES : 0);
 
@@ -303,7 +321,7 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
     // heads that share K/V also share an L2.
     const long long per_xcd = (p.total_wg + 7) >> 3;
     const long long logical = (long long)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    if (logical >= p.total_wg) return;
+    if (logical >= p.total_wg) return false;
     const int group = p.hq / p.hk;
     long long rest = logical;
     const int hin = (int)(rest % group); rest /= group;
@@ -322,7 +340,7 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
         const int ch = (int)(rest % nch);
         b = (int)(rest / nch);
         hs = ch * group + hin;
-        if (hs >= p.index_heads) return;             // padding of the last chunk (workgroup-uniform)
+        if (hs >= p.index_heads) return false;       // padding of the last chunk (workgroup-uniform)
         h = as_const(p.head_list)[hs];
         hkv = h / group;
     } else {
@@ -356,7 +374,7 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
                 int r = row0 + i / NCH;
                 if (r < p.n) *reinterpret_cast<u32x4_t *>(o_base + (long long)r * p.os[2] * 2 + (i % NCH) * 16) = u32x4_t{0u, 0u, 0u, 0u};
             }
-        if (!PAIR || mA * BM >= seqlen) return;      // (wave-uniform; for a pair: both halves are past)
+        if (!PAIR || mA * BM >= seqlen) return false;   // (wave-uniform; for a pair: both halves are past)
     }
 
     const char *q_base = p.q + ((long long)b * p.qs[0] + (long long)h * p.qs[1]) * 2;
@@ -365,6 +383,7 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
     const long long k_row = p.ks[2] * 2, v_row = p.vs[2] * 2;
     const long long ridx = ((long long)b * p.index_heads + hs) * p.rows + min(m, p.rows - 1);
 
+    constexpr bool every_max = EVERY_MAX;
     // ---- Q fragments (B operand of S^T): row qrow, d = 16*ks + 8*g + 0..7 ----
     Frag qf[KS];
     {
@@ -377,10 +396,11 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
         }
     }
 
+    // The row maximum of a tile is only computed when it is needed (see sm_pv_block); a walk whose
+    // row sums leave the safe range is run again with the maximum computed for every tile.
     int nblk = 0;
     // Paired block-sparse: both row blocks' lists (ascending block ids) are parked in LDS and walked
     // as one merged sequence; a block that is on both lists is copied and visited once.
-    __shared__ int lds_list[PAIR && MODE == MODE_BS ? 2 * BS_PAIR_MAX : 1];
     int bs_na = 0, bs_nb = 0, bs_ia = 0, bs_ib = 0;
     if constexpr (PAIR && MODE == MODE_BS) {
         bs_na = min(mA + 1, p.max_blocks);
@@ -407,10 +427,7 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
     [[maybe_unused]] int vs_na = 0, vs_nb = 0, vs_cca = 0, vs_ccb = 0, vs_nc = 0;
     [[maybe_unused]] bool vs_merged = false;
     [[maybe_unused]] long long vs_ra = 0, vs_rb = 0;
-    __shared__ int vs_only[VSP ? 2 * VS_ONLY_MAX : 1];        // [row block][entries the other list lacks]
     if constexpr (VSP) {
-        __shared__ int vs_wsum[4];
-        __shared__ int vs_bad;
         const bool b_exists = 2 * mslot + 1 < p.rows && (2 * mslot + 1) * BM < seqlen;
         vs_ra = ((long long)b * p.index_heads + hs) * p.rows + mA;
         vs_rb = b_exists ? vs_ra + 1 : vs_ra;
@@ -646,6 +663,7 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
 #pragma unroll
         for (int r = 0; r < 16; ++r) oacc[i][r] = 0.f;
     float m_i = -INFINITY;   // running max (log2 domain, scaled)
+    int sm_steps = 0;        // tiles this wave has put through the softmax
     float l_i = 0.f;         // this lane's share of the running sum
 
     // LDS read addresses that do not depend on the tile
@@ -768,6 +786,13 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
                     (__attribute__((address_space(3))) short4_t *)(vbuf + v_rd_off[db] + (16 * s + 8 * jj) * ROW_BYTES));
         }
         // ---- online softmax (exp2 domain) -------------------------------------
+        // The reference maximum m_i of a row only has to keep exp2 inside the range of fp32 (bf16 has the
+        // same exponent range), so most tiles take it as it is: no row maximum, no rescale factor.  It
+        // is recomputed where a row has none yet (first tile, fully masked tiles), every MAX_PERIOD steps,
+        // and for every tile of a walk that is run again because a row sum left the safe range (which
+        // takes a row whose scores rise by more than a hundred powers of two within MAX_PERIOD tiles).
+        float alpha = 1.0f, m_use = m_i;
+        if (every_max || ((sm_steps++ & (MAX_PERIOD - 1)) == 0) || __any(m_i == -INFINITY)) {
         float mx;
         {
             // four independent chains of three-operand maxima (8 scores each)
@@ -783,15 +808,15 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
         }
         { const unsigned u = __float_as_uint(mx); auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false); mx = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1])); }
         const float cand = mx * p.scale_log2;
-        // lazy reference maximum: raised only when a tile exceeds it by more than LAZY_MAX powers of two
-        // (probabilities stay below 2^LAZY_MAX: 2^8 fits f16 with room for the row sums, bf16 has the
-        // exponent range of fp32)
+        // lazy: raised only when a tile exceeds it by more than LAZY_MAX powers of two (probabilities of
+        // f16 operands must stay inside the f16 range: 2^8 leaves room for the row sums)
         constexpr float LAZY_MAX = std::is_same<T, __bf16>::value ? LAZY_MAX_BF16 : 8.0f;
         const bool grow = cand > m_i + LAZY_MAX;
         const float m_new = grow ? cand : m_i;
-        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = grow ? __builtin_amdgcn_exp2f(m_i - m_use) : 1.0f;
+        m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        alpha = grow ? __builtin_amdgcn_exp2f(m_i - m_use) : 1.0f;
         m_i = m_new;
+        }
         float psum = 0.f;
         Frag pfr[4];
         // probabilities of key group q (16 keys): registers 8*(q%2) .. +7 of s0 (q < 2) / s1
@@ -964,6 +989,8 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
         const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
         // pitch: 8-byte lane writes spread over all banks (four waves only fit without the pad)
         constexpr int OP = PAIR ? ROW_BYTES : ROW_BYTES + 8;
+        // a row sum at 2^100 or beyond (or no number at all): some probability may have overflowed
+        if (!every_max && __any(!(l_tot < 0x1p100f)) && lane == 0) lds_redo = 1;
         __syncthreads();                                  // K/V tiles no longer needed
         char *ot = PAIR ? (half ? lds_v : lds_k) + wave * 32 * OP : (wave ? lds_v : lds_k);   // 32 rows per wave
         const bool live = qrow < seqlen;
@@ -985,6 +1012,30 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
             const u32x4_t val = *reinterpret_cast<const u32x4_t *>(ot + r * OP + (lane % NCH) * 16);
             if (grow < p.n && have_rows) *reinterpret_cast<u32x4_t *>(o_base + (long long)grow * p.os[2] * 2 + (lane % NCH) * 16) = val;
         }
+    }
+    // (the flag was written before the barrier at the head of the epilogue)
+    return !every_max && lds_redo != 0;                   // (workgroup-uniform)
+}
+
+template <typename T, int MODE, bool PAIR, int HD>
+__global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_kernel(const AttnParams p) {
+    typedef AttnLds<MODE, PAIR, HD> L;
+    __shared__ __attribute__((aligned(16))) char lds_k[L::NK];
+    __shared__ __attribute__((aligned(16))) char lds_v[L::NK];
+    __shared__ int lds_list[L::NLIST];       // paired block-sparse: the two block lists
+    __shared__ int vs_only[L::NONLY];        // paired vertical-slash: [row block][entries the other list lacks]
+    __shared__ int vs_wsum[4];
+    __shared__ int vs_bad;
+    __shared__ int lds_redo;
+    if (threadIdx.x == 0) lds_redo = 0;      // (ordered before its readers by the barriers of the walk)
+    if constexpr (std::is_same<T, __bf16>::value) {
+        if (attn_walk<T, MODE, PAIR, HD, false>(p, lds_k, lds_v, lds_list, vs_only, vs_wsum, vs_bad, lds_redo)) {
+            __syncthreads();                 // everyone has read the flag and is done with LDS
+            attn_walk<T, MODE, PAIR, HD, true>(p, lds_k, lds_v, lds_list, vs_only, vs_wsum, vs_bad, lds_redo);
+        }
+    } else {
+        // f16 probabilities have no headroom above the lazy threshold: the maximum of every tile
+        attn_walk<T, MODE, PAIR, HD, true>(p, lds_k, lds_v, lds_list, vs_only, vs_wsum, vs_bad, lds_redo);
     }
 }
 

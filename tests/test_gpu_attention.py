@@ -48,6 +48,33 @@ def test_dense_causal_vs_sdpa(gpu, dtype, n, hq, hk):
     check(out, sdpa_causal(q, expand(k, hq), expand(v, hq)), "dense")
 
 
+@pytest.mark.parametrize("hot_key", [300, 520, 70])
+def test_scores_far_above_the_first_tiles_are_walked_again(gpu, hot_key):
+    """One key whose score lies ~290 powers of two above everything before it: the fast walk takes its
+    reference maximum from earlier tiles and overflows exp2, which it has to notice and repair by
+    walking the row blocks again with the maximum of every tile (hot_key 300: inside the tiles
+    that skip the maximum; 520: at a tile that computes it; 70: in the second tile)."""
+    from minference_amd import dense_causal_attention, vertical_slash_sparse_attention
+    n, hq, hk = 1024, 2, 1
+    print(f"case rising scores hot_key={hot_key}", flush=True)
+    g = torch.Generator().manual_seed(5)
+    q = 0.1 * torch.randn(1, hq, n, 128, generator=g) + 4.25
+    k = 0.1 * torch.randn(1, hk, n, 128, generator=g)
+    v = torch.randn(1, hk, n, 128, generator=g)
+    k[0, 0, hot_key] += 4.25
+    q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
+    ref = sdpa_causal(q, expand(k, hq), expand(v, hq))
+    out = dense_causal_attention(q.to(gpu), k.to(gpu), v.to(gpu))
+    check(out, ref, "dense, rising scores")
+    # the same key as a vertical line next to a local band of 128 diagonals: the gathered column
+    # tile comes last in the walk of every row block
+    v_idx = torch.tensor([0, 1, 2, hot_key], dtype=torch.int32).expand(1, hq, 4).contiguous()
+    s_idx = torch.arange(127, -1, -1, dtype=torch.int32).expand(1, hq, -1).contiguous()
+    out = vertical_slash_sparse_attention(q.to(gpu), k.to(gpu), v.to(gpu), v_idx.to(gpu), s_idx.to(gpu))
+    ref = O.vertical_slash_sparse_attention(q, expand(k, hq), expand(v, hq), v_idx, s_idx)
+    check(out, ref, "vertical-slash, rising scores")
+
+
 @pytest.mark.parametrize("n,nv,ns,hq,hk,seed", [
     (1024, 40, 60, 2, 2, 0), (2048, 100, 300, 4, 1, 1), (1500, 30, 50, 2, 2, 2), (700, 200, 20, 1, 1, 3),
 ])
