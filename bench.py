@@ -190,7 +190,11 @@ def sensitivity_lines(args, torch, gen, M, dev, n, hq, hk):
       over the whole context and almost everything is covered;
     * scattered: the index lists of BASELINE config 3's generator at this length with 600 slashes
       (0..63 forced, the rest uniform) and 1000 uniform verticals: block lists made of many short
-      runs and 14-16 gathered column tiles per row block."""
+      runs and 14-16 gathered column tiles per row block.  Neighbouring row blocks and the heads of a
+      kv group share almost none of these tiles, so every visited tile is its own 32 KB of K and V:
+      `kv_tile_fetch_tbs` = tiles x 32 KiB / time is what the memory system behind the LDS delivers,
+      and it is at the level of the HBM peak -- this case is bound by memory, not by the matrix pipe
+      (at 64 FLOP per fetched byte, 8 TB/s caps it at 512 TFLOP/s without cache hits)."""
     import numpy as np
     rows = (n + 63) // 64
     causal_tiles = hq * rows * (rows + 1) // 2
@@ -225,7 +229,8 @@ def sensitivity_lines(args, torch, gen, M, dev, n, hq, hk):
     ms = timed(lambda: M.vertical_slash_attention_from_index(q, k, v, bc, bo, cc, ci, seqlens), 3)
     out["scattered"] = {"coverage": round(tiles / causal_tiles, 4), "attention_ms": round(ms, 3),
                         "gathered_tile_share": round(gathered / tiles, 4),
-                        "tflops_on_computed_tiles": round(tiles * TILE_FLOP / ms / 1e9, 1)}
+                        "tflops_on_computed_tiles": round(tiles * TILE_FLOP / ms / 1e9, 1),
+                        "kv_tile_fetch_tbs": round(tiles * 2 * 64 * 128 * 2 / ms / 1e9, 2), "bound": "hbm"}
     return out
 
 
