@@ -7,14 +7,14 @@
 // a tile that is on both lists is copied into LDS once for 128 query rows, a tile that only one of
 // them visits is copied by that half into buffers of its own while the other half does the same
 // with a tile of its list.  For dense causal and A-shape / tri-shape the lists are analytic and
-// differ by at most their ends; block-sparse lists are merged on the fly; vertical-slash lists are
-// split into common and leftover entries once, in LDS, before the tile loop.  Besides halving the
+// differ by at most their ends; vertical-slash and block-sparse lists are split into common and
+// leftover entries once, in LDS, before the tile loop.  Besides halving the
 // copies of shared tiles, the lockstep is what keeps long scattered lists fast: row block m+1's
 // list is row block m's shifted by 64 keys, so what one half fetches now the other fetched a step
 // ago and finds in L2 (measured +23..38 % on lists of several hundred blocks, +1 % on the
-// cache-friendly benchmark layer, against one 2-wave workgroup per row block).  The 2-wave form
-// (one workgroup per 64-row block) remains for block-sparse lists longer than the paired walk
-// keeps in LDS.
+// cache-friendly benchmark layer, against one 2-wave workgroup per row block).  Every launch uses
+// this paired form; the kernel's 2-wave form (PAIR = false: one workgroup per 64-row block) is what
+// those comparisons were measured against and is not instantiated.
 // Everything is computed in the TRANSPOSED orientation so that softmax statistics are per lane:
 //
 //   S^T[token][qrow] = K_tile . Q^T      v_mfma_f32_32x32x16 (A = K from LDS, B = Q in VGPRs)
@@ -179,11 +179,10 @@ struct Tile {
     int gathered;       // 0/1
     int nvalid;         // gathered: number of valid list entries in this tile
     int on_a, on_b;     // paired walks: is the tile on the list of row block A / B
-    int split;          // paired vertical-slash: each row block has a tile of its own in this step
+    int split;          // paired list walks: each row block has a tile of its own in this step
 };
-constexpr int BS_PAIR_MAX = 512;   // longest block list the paired block-sparse walk keeps in LDS
-// (the longest vertical-slash block list the paired kernel splits in LDS is what a K tile holds twice:
-// 2048 entries at head_dim 128, 1024 at 64)
+// (the longest block list the paired kernel splits in LDS is what a K tile holds twice: 2048 entries
+// at head_dim 128, 1024 at 64)
 constexpr int VS_ONLY_MAX = 512;   // ... and the most entries of one list that the other one lacks
 
 template <int MODE>
@@ -275,10 +274,9 @@ __device__ __forceinline__ bool tile_on_list(const AttnParams &p, int m, int sta
 // LDS of one workgroup (declared by the kernel, see attn_fwd_kernel): separate objects, so that the
 // compiler lets reads of one overtake copies into the other.
 template <int MODE, bool PAIR, int HD> struct AttnLds {
-    static constexpr bool VSP = PAIR && MODE == MODE_VS;
+    static constexpr bool VSP = PAIR && (MODE == MODE_VS || MODE == MODE_BS);      // walks of two block lists
     static constexpr int TILE_BYTES = BN * HD * 2;
     static constexpr int NK = (VSP ? 2 : 1) * TILE_BYTES;
-    static constexpr int NLIST = PAIR && MODE == MODE_BS ? 2 * BS_PAIR_MAX : 1;
     static constexpr int NONLY = VSP ? 2 * VS_ONLY_MAX : 1;
 };
 
@@ -289,7 +287,6 @@ template <int MODE, bool PAIR, int HD> struct AttnLds {
 template <typename T, int MODE, bool PAIR, int HD, bool EVERY_MAX>
 __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[AttnLds<MODE, PAIR, HD>::NK],
                                           char (&lds_v)[AttnLds<MODE, PAIR, HD>::NK],
-                                          int (&lds_list)[AttnLds<MODE, PAIR, HD>::NLIST],
                                           int (&vs_only)[AttnLds<MODE, PAIR, HD>::NONLY], int (&vs_wsum)[4], int &vs_bad,
                                           int &lds_redo) {
     static_assert(HD == 128 || HD == 64, "head_dim 128 or 64");
@@ -305,10 +302,13 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
     auto swz_v = [](int row) { return HD == 128 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); };
     constexpr int NT = PAIR ? 2 * NTHREADS : NTHREADS;      // threads per workgroup
     constexpr int CROWS = PAIR ? 16 : 32;                   // tile rows copied by one wave (shared tile)
-    constexpr bool VSP = PAIR && MODE == MODE_VS;
+    // VSP: the paired walk of two block lists -- the vertical-slash block lists, or the block-sparse
+    // lists (block numbers, i.e. key starts / 64; no columns)
+    constexpr bool VSP = PAIR && (MODE == MODE_VS || MODE == MODE_BS);
+    constexpr int LIST_SCALE = MODE == MODE_BS ? BN : 1;     // list entry -> first key of the block
     constexpr int TILE_BYTES = BN * ROW_BYTES;
     constexpr int VS_PAIR_MAX = TILE_BYTES / 8;             // both staged lists fit the second K tile
-    // paired vertical-slash: a second K and V tile (row block B's buffers in the steps in which each
+    // paired list walks (vertical-slash, block-sparse): a second K and V tile (row block B's buffers in the steps in which each
     // row block has a tile of its own); before that, the second K tile stages the two block lists and
     // the second V tile holds their merge
     char *const lds_k1 = lds_k + (VSP ? TILE_BYTES : 0);
@@ -399,18 +399,8 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
     // The row maximum of a tile is only computed when it is needed (see sm_pv_block); a walk whose
     // row sums leave the safe range is run again with the maximum computed for every tile.
     int nblk = 0;
-    // Paired block-sparse: both row blocks' lists (ascending block ids) are parked in LDS and walked
-    // as one merged sequence; a block that is on both lists is copied and visited once.
-    int bs_na = 0, bs_nb = 0, bs_ia = 0, bs_ib = 0;
-    if constexpr (PAIR && MODE == MODE_BS) {
-        bs_na = min(mA + 1, p.max_blocks);
-        bs_nb = (2 * mslot + 1 < p.rows && (2 * mslot + 1) * BM < seqlen) ? min(mA + 2, p.max_blocks) : 0;
-        const long long rbase = ((long long)b * p.index_heads + hs) * p.bidx_rows;
-        for (int i = tid; i < bs_na; i += NT) lds_list[i] = p.bidx[(rbase + mA) * p.max_blocks + i];
-        for (int i = tid; i < bs_nb; i += NT) lds_list[BS_PAIR_MAX + i] = p.bidx[(rbase + mA + 1) * p.max_blocks + i];
-        __syncthreads();
-    }
-    // Paired vertical-slash: the block lists of the two row blocks (ascending key starts; those of
+    // Paired list walks (vertical-slash block lists, block-sparse lists scaled to key starts): the
+    // block lists of the two row blocks (ascending key starts; vertical-slash lists of
     // neighbouring row blocks are each other's translate by 64 keys wherever no entry is clipped, so
     // runs of blocks share all but their ends) are split ONCE, by all 256 threads, before the tile
     // loop: both lists are staged in LDS, every entry looks itself up in the other list by binary
@@ -424,24 +414,34 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
     // Lists that are too long for LDS or not strictly ascending are not split: each half then walks
     // its whole list in split steps (still in lockstep with its neighbour, which is what keeps the
     // neighbour's tiles in L2 when the lists are long and scattered).
+    // where the block lists live: [batch, heads, list_rows, list_w]
+    [[maybe_unused]] const int *const list_base = MODE == MODE_BS ? p.bidx : p.bo;
+    [[maybe_unused]] const int list_w = MODE == MODE_BS ? p.max_blocks : p.nnz_s;
+    [[maybe_unused]] const int list_rows = MODE == MODE_BS ? p.bidx_rows : p.rows;
     [[maybe_unused]] int vs_na = 0, vs_nb = 0, vs_cca = 0, vs_ccb = 0, vs_nc = 0;
     [[maybe_unused]] bool vs_merged = false;
     [[maybe_unused]] long long vs_ra = 0, vs_rb = 0;
     if constexpr (VSP) {
         const bool b_exists = 2 * mslot + 1 < p.rows && (2 * mslot + 1) * BM < seqlen;
-        vs_ra = ((long long)b * p.index_heads + hs) * p.rows + mA;
+        vs_ra = ((long long)b * p.index_heads + hs) * list_rows + mA;
         vs_rb = b_exists ? vs_ra + 1 : vs_ra;
-        vs_na = max(0, min(as_const(p.bc)[vs_ra], p.nnz_s));
-        vs_cca = max(0, min(as_const(p.cc)[vs_ra], p.nnz_v));
-        vs_nb = b_exists ? max(0, min(as_const(p.bc)[vs_rb], p.nnz_s)) : 0;
-        vs_ccb = b_exists ? max(0, min(as_const(p.cc)[vs_rb], p.nnz_v)) : 0;
+        if constexpr (MODE == MODE_BS) {
+            // row block m visits the first min(m + 1, max_blocks) entries of its row; no columns
+            vs_na = min(mA + 1, p.max_blocks);
+            vs_nb = b_exists ? min(mA + 2, p.max_blocks) : 0;
+        } else {
+            vs_na = max(0, min(as_const(p.bc)[vs_ra], p.nnz_s));
+            vs_cca = max(0, min(as_const(p.cc)[vs_ra], p.nnz_v));
+            vs_nb = b_exists ? max(0, min(as_const(p.bc)[vs_rb], p.nnz_s)) : 0;
+            vs_ccb = b_exists ? max(0, min(as_const(p.cc)[vs_rb], p.nnz_v)) : 0;
+        }
         if (vs_na <= VS_PAIR_MAX && vs_nb <= VS_PAIR_MAX && vs_na > 0 && vs_nb > 0) {
             int *rawA = reinterpret_cast<int *>(lds_k1), *rawB = rawA + VS_PAIR_MAX;
             int *common = reinterpret_cast<int *>(lds_v1);
-            const int *ga = p.bo + vs_ra * p.nnz_s, *gb = p.bo + vs_rb * p.nnz_s;
+            const int *ga = list_base + vs_ra * list_w, *gb = list_base + vs_rb * list_w;
             if (tid == 0) vs_bad = 0;
-            for (int i = tid; i < vs_na; i += NT) rawA[i] = ga[i];
-            for (int i = tid; i < vs_nb; i += NT) rawB[i] = gb[i];
+            for (int i = tid; i < vs_na; i += NT) rawA[i] = ga[i] * LIST_SCALE;
+            for (int i = tid; i < vs_nb; i += NT) rawB[i] = gb[i] * LIST_SCALE;
             __syncthreads();
             bool bad = false;                              // the look-ups need strictly ascending lists
             for (int i = tid; i + 1 < vs_na; i += NT) bad |= rawA[i + 1] <= rawA[i];
@@ -492,21 +492,6 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
             }
         }
     }
-    auto bs_merge_next = [&]() -> Tile {      // one step of the merged walk (wave-uniform)
-        Tile t;
-        t.gathered = 0;
-        t.nvalid = BN;
-        const int xa = bs_ia < bs_na ? __builtin_amdgcn_readfirstlane(lds_list[min(bs_ia, BS_PAIR_MAX - 1)]) : 0x7fffffff;
-        const int xb = bs_ib < bs_nb ? __builtin_amdgcn_readfirstlane(lds_list[BS_PAIR_MAX + min(bs_ib, BS_PAIR_MAX - 1)]) : 0x7fffffff;
-        const int x = min(xa, xb);
-        t.on_a = xa == x && bs_ia < bs_na;
-        t.on_b = xb == x && bs_ib < bs_nb;
-        bs_ia += t.on_a;
-        bs_ib += t.on_b;
-        t.start = x * BN;
-        return t;
-    };
-    // the merged walk ends when both lists are used up (its length is not known in advance)
     int ntiles = 0;
     // paired vertical-slash: vs_nc common steps, then the split steps: per half its leftover block
     // entries (from LDS when the lists were split, else its whole list from global memory) and its
@@ -521,22 +506,19 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
         vs_nt_mine = have_rows ? (half ? nt_b : nt_a) : 0;
         ntiles = vs_nc + max(nt_a, nt_b);
     }
-    else if constexpr (!(PAIR && MODE == MODE_BS))
+    else
         ntiles = PAIR ? pair_tile_count<MODE>(p, mA, mB, nblk) : tile_count<MODE>(p, ridx, m, nblk);
-    auto more_tiles = [&](int it) -> bool {   // is there a tile number `it` ?
-        if constexpr (PAIR && MODE == MODE_BS) return bs_ia < bs_na || bs_ib < bs_nb;
-        else return it < ntiles;
-    };
+    auto more_tiles = [&](int it) -> bool { return it < ntiles; };   // is there a tile number `it` ?
     // paired vertical-slash: entry it+1 of the common list sits in a scalar when step `it` starts; the
     // LDS read of entry it+2 is issued at the top of step `it` (no tile copy is in flight there: the
     // list shares an LDS object with the V tiles and must not wait for one) and turns into the next
     // scalar at the end of the step, its latency hidden behind the tile's work
     [[maybe_unused]] int vs_entry = 0, vs_pref = 0;
+    // this row block's own list in global memory (walked directly when the lists were not split)
+    [[maybe_unused]] const cint_ptr sp_list = as_const(list_base) + (((long long)b * p.index_heads + hs) * list_rows + min(m, p.rows - 1)) * list_w;
     auto vs_list = [&](int i) -> int { return reinterpret_cast<const int *>(lds_v1)[min(i, 2 * VS_PAIR_MAX - 1)]; };
     auto tile_of = [&](int it) -> Tile {      // called with it = 0, 1, 2, ... in order
-        if constexpr (PAIR && MODE == MODE_BS) {
-            return bs_merge_next();
-        } else if constexpr (VSP) {
+        if constexpr (VSP) {
             Tile t;
             t.gathered = 0;
             t.nvalid = BN;
@@ -551,7 +533,7 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
                 t.start = 0;
                 if (j < vs_nb_mine) {
                     if (vs_merged) t.start = __builtin_amdgcn_readfirstlane(vs_only[half * VS_ONLY_MAX + j]);
-                    else t.start = as_const(p.bo)[ridx * p.nnz_s + j];
+                    else t.start = sp_list[j] * LIST_SCALE;
                 } else if (j < vs_nt_mine) {
                     t.gathered = 1;
                     t.start = (j - vs_nb_mine) * BN;
@@ -875,7 +857,7 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
         copy_tile(cur, k_base, k_row, std::false_type{}, gt_cur, lds_k);
     }
 
-    // One step of the walk, in three forms (the last two for paired vertical-slash lists only):
+    // One step of the walk, in three forms (the last two for the paired list walks only):
     // general (kind 0) -- any tile, any successor, every mode;
     // COMMON (kind 1) -- this tile and the next one are both on the list of common entries: shared,
     // contiguous, never gathered;
@@ -885,7 +867,6 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
     // In the two special forms everything that deals with the other cases drops out of the
     // instruction stream (the general form costs about 1.7 times a COMMON step).
     [[maybe_unused]] int sp_entry = 0;
-    [[maybe_unused]] const cint_ptr sp_list = as_const(p.bo) + ridx * p.nnz_s;      // this row block's list in global memory
     auto step = [&](const int it, auto kind_c) {
         constexpr int KIND = decltype(kind_c)::value;
         constexpr bool COMMON = KIND == 1, SPLIT = KIND == 2;
@@ -903,7 +884,7 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
         } else if constexpr (SPLIT) {
             const int j = it - vs_nc;                      // this step's position in the leftover lists
             if (vs_merged) vs_pref = vs_only[half * VS_ONLY_MAX + min(j + 2, VS_ONLY_MAX - 1)];
-            else vs_pref = sp_list[min(j + 2, p.nnz_s - 1)];
+            else vs_pref = sp_list[min(j + 2, list_w - 1)] * LIST_SCALE;
             have_nxt = true;
             nxt.gathered = 0; nxt.nvalid = BN; nxt.on_a = nxt.on_b = 1; nxt.split = 1;
             nxt.start = sp_entry;
@@ -976,7 +957,7 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
 #pragma unroll
                 for (int db = 0; db < NDB; ++db) v_rd_off[db] += half * TILE_BYTES;
             }
-            sp_entry = vs_merged ? __builtin_amdgcn_readfirstlane(vs_only[half * VS_ONLY_MAX + 1]) : sp_list[1];
+            sp_entry = vs_merged ? __builtin_amdgcn_readfirstlane(vs_only[half * VS_ONLY_MAX + 1]) : sp_list[1] * LIST_SCALE;
             for (; it - vs_nc + 1 < nb_both; ++it) step(it, std::integral_constant<int, 2>{});
         }
     }
@@ -1022,20 +1003,19 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
     typedef AttnLds<MODE, PAIR, HD> L;
     __shared__ __attribute__((aligned(16))) char lds_k[L::NK];
     __shared__ __attribute__((aligned(16))) char lds_v[L::NK];
-    __shared__ int lds_list[L::NLIST];       // paired block-sparse: the two block lists
-    __shared__ int vs_only[L::NONLY];        // paired vertical-slash: [row block][entries the other list lacks]
+    __shared__ int vs_only[L::NONLY];        // paired list walks: [row block][entries the other list lacks]
     __shared__ int vs_wsum[4];
     __shared__ int vs_bad;
     __shared__ int lds_redo;
     if (threadIdx.x == 0) lds_redo = 0;      // (ordered before its readers by the barriers of the walk)
     if constexpr (std::is_same<T, __bf16>::value) {
-        if (attn_walk<T, MODE, PAIR, HD, false>(p, lds_k, lds_v, lds_list, vs_only, vs_wsum, vs_bad, lds_redo)) {
+        if (attn_walk<T, MODE, PAIR, HD, false>(p, lds_k, lds_v, vs_only, vs_wsum, vs_bad, lds_redo)) {
             __syncthreads();                 // everyone has read the flag and is done with LDS
-            attn_walk<T, MODE, PAIR, HD, true>(p, lds_k, lds_v, lds_list, vs_only, vs_wsum, vs_bad, lds_redo);
+            attn_walk<T, MODE, PAIR, HD, true>(p, lds_k, lds_v, vs_only, vs_wsum, vs_bad, lds_redo);
         }
     } else {
         // f16 probabilities have no headroom above the lazy threshold: the maximum of every tile
-        attn_walk<T, MODE, PAIR, HD, true>(p, lds_k, lds_v, lds_list, vs_only, vs_wsum, vs_bad, lds_redo);
+        attn_walk<T, MODE, PAIR, HD, true>(p, lds_k, lds_v, vs_only, vs_wsum, vs_bad, lds_redo);
     }
 }
 
@@ -1085,11 +1065,8 @@ void fill_params(AttnParams &p, const minf_qkvo *t) {
 
 template <int MODE, int HD> int launch_hd(AttnParams p, int dtype, void *stream) {
     if (p.batch == 0 || p.rows == 0) return MINF_OK;
-    // every mode runs on the paired (4-wave) kernel, except block-sparse lists that are too long for
-    // the paired walk's LDS copy: those run on the 2-wave kernel
-    constexpr bool CAN_PAIR = true;
-    constexpr bool CAN_SINGLE = MODE == MODE_BS;
-    const bool pair = CAN_PAIR && (MODE != MODE_BS || p.max_blocks <= BS_PAIR_MAX);
+    // every mode runs on the paired (4-wave) kernel
+    constexpr bool pair = true;
     // heads of the grid: all of them, or the selected ones rounded up to whole chunks of hq / hk
     const int group = p.hq / p.hk;
     const long long grid_heads = p.head_list ? (long long)((p.index_heads + group - 1) / group) * group : p.hq;
@@ -1100,19 +1077,9 @@ template <int MODE, int HD> int launch_hd(AttnParams p, int dtype, void *stream)
     if (grid > 0x7fffffffLL) return MINF_ERR_UNSUPPORTED;
     const dim3 block(pair ? 2 * NTHREADS : NTHREADS);
     hipStream_t st = (hipStream_t)stream;
-    if constexpr (CAN_PAIR) {
-        if (pair) {
-            if (dtype == MINF_BF16) hipLaunchKernelGGL((attn_fwd_kernel<__bf16, MODE, true, HD>), dim3((unsigned)grid), block, 0, st, p);
-            else hipLaunchKernelGGL((attn_fwd_kernel<_Float16, MODE, true, HD>), dim3((unsigned)grid), block, 0, st, p);
-            return minf_launch_status();
-        }
-    }
-    if constexpr (CAN_SINGLE) {
-        if (dtype == MINF_BF16) hipLaunchKernelGGL((attn_fwd_kernel<__bf16, MODE, false, HD>), dim3((unsigned)grid), block, 0, st, p);
-        else hipLaunchKernelGGL((attn_fwd_kernel<_Float16, MODE, false, HD>), dim3((unsigned)grid), block, 0, st, p);
-        return minf_launch_status();
-    }
-    return MINF_ERR_UNSUPPORTED;      // not reached: every mode has one of the two variants
+    if (dtype == MINF_BF16) hipLaunchKernelGGL((attn_fwd_kernel<__bf16, MODE, pair, HD>), dim3((unsigned)grid), block, 0, st, p);
+    else hipLaunchKernelGGL((attn_fwd_kernel<_Float16, MODE, pair, HD>), dim3((unsigned)grid), block, 0, st, p);
+    return minf_launch_status();
 }
 
 template <int MODE> int launch(const AttnParams &p, const minf_qkvo *t, void *stream) {
