@@ -12,9 +12,8 @@
 // copies of shared tiles, the lockstep is what keeps long scattered lists fast: row block m+1's
 // list is row block m's shifted by 64 keys, so what one half fetches now the other fetched a step
 // ago and finds in L2 (measured +23..38 % on lists of several hundred blocks, +1 % on the
-// cache-friendly benchmark layer, against one 2-wave workgroup per row block).  Every launch uses
-// this paired form; the kernel's 2-wave form (PAIR = false: one workgroup per 64-row block) is what
-// those comparisons were measured against and is not instantiated.
+// cache-friendly benchmark layer, against an earlier form of this kernel with one 2-wave workgroup
+// per row block).
 // Everything is computed in the TRANSPOSED orientation so that softmax statistics are per lane:
 //
 //   S^T[token][qrow] = K_tile . Q^T      v_mfma_f32_32x32x16 (A = K from LDS, B = Q in VGPRs)
@@ -36,14 +35,13 @@
 // the 64 tile rows, a scalar row offset and one of five loop-invariant per-lane offsets: no vector
 // instruction per copy and 8 cycles less issue time per copy than the 64-bit-address form, which
 // remains for gathered and clamped rows (global_load_lds_dwordx4).  32-68 KB of LDS and <= 256 registers
-// keep two waves per SIMD resident (two 4-wave or four 2-wave workgroups per CU).
+// keep two waves per SIMD resident (two 4-wave workgroups per CU).
 //
 // One iteration of a wave (two workgroup barriers per tile, single buffers):
 //   wait own K(it) copies; barrier (all of K(it) visible, everyone done with V(it-1))
 //   issue V(it) copy; S^T = K.Q^T with the K fragments read two k-steps ahead of their MFMAs
-//   wait own V(it) copies; barrier (all of V(it) visible, everyone done with K(it)) -- in the 2-wave
-//   kernel already before the last four QK MFMAs, with all V^T fragment reads issued under them
-//   issue K(it+1) copy; (paired variant: read all V^T fragments;) row max; exponentials of keys 0..15
+//   wait own V(it) copies; barrier (all of V(it) visible, everyone done with K(it))
+//   issue K(it+1) copy; read all V^T fragments; row max where it is needed; exponentials of keys 0..15
 //   O^T += V^T.P^T with the exponentials of key group s+1 (16 keys) placed behind the MFMAs of
 //   group s
 // The compiler's own schedule read every fragment right before its MFMA (full LDS latency exposed
@@ -55,7 +53,7 @@
 //    column ids are fetched one per lane an iteration ahead and distributed with wave shuffles;
 //  * the running max is only raised when a tile exceeds it by more than 2^20 (bf16; 2^8 for f16
 //    operands, whose probabilities must stay inside the f16 range), so nearly all tiles skip the
-//    O^T rescale;
+//    O^T rescale; for bf16 the row maximum is not even computed in most tiles (see sm_pv_block);
 //  * the cross-half max uses v_permlane32_swap, the row sums v_dot2 on the rounded probabilities
 //    (the same values the second MFMA consumes);
 //  * s_setprio raises the wave while it issues MFMAs;
@@ -79,14 +77,11 @@ enum { MODE_VS = 0, MODE_BS = 1, MODE_ASHAPE = 2, MODE_DENSE = 3 };
 constexpr int BM = 64;        // query rows per workgroup
 constexpr int BN = 64;        // keys per tile
 constexpr int HD_MAX = 128;   // head_dim: 128 or 64 (template parameter HD of the kernel)
-constexpr int NTHREADS = 128; // 2 wavefronts per 64-row block (x2 in the paired variant)
+constexpr int NTHREADS = 128; // 2 wavefronts per 64-row block, two row blocks per workgroup
 // Scheduling constants (measured on MI355X): K fragments are read QK_AHEAD k-steps ahead of their
 // MFMAs; VALU_PER_MFMA softmax instructions are placed behind each of the first twelve PV MFMAs.
 constexpr int QK_AHEAD = 2;
 constexpr int VALU_PER_MFMA = 6;
-// 2-wave kernel: the second barrier of a tile comes after this k-step of the QK loop (all K
-// fragments have been read by then), and the V^T fragment reads follow it under the last MFMAs
-constexpr int EARLY_B2 = 5;
 #ifndef MAX_PERIOD
 #define MAX_PERIOD 8      // (a power of two) the row maximum is recomputed at least every MAX_PERIOD tiles
 #endif
@@ -185,58 +180,7 @@ struct Tile {
 // at head_dim 128, 1024 at 64)
 constexpr int VS_ONLY_MAX = 512;   // ... and the most entries of one list that the other one lacks
 
-template <int MODE>
-__device__ __forceinline__ int tile_count(const AttnParams &p, long long ridx, int m, int &nblk) {
-    if constexpr (MODE == MODE_VS) {
-        // counts are clamped to the list widths: a bad count must not turn into a read past the row
-        nblk = max(0, min(as_const(p.bc)[ridx], p.nnz_s));
-        return nblk + ((max(0, min(as_const(p.cc)[ridx], p.nnz_v)) + BN - 1) >> 6);
-    } else if constexpr (MODE == MODE_BS) {
-        nblk = min(m + 1, p.max_blocks);
-        return nblk;
-    } else if constexpr (MODE == MODE_ASHAPE) {
-        if (m * BM + BM - 1 >= p.dense_from) {     // block holds dense rows: every causal tile
-            nblk = m + 1;
-            return nblk;
-        }
-        // window tiles t_lo..m, preceded by the sink tiles that lie before t_lo
-        int lo_key = m * BM - p.n_local + 1;
-        int t_lo = lo_key > 0 ? (lo_key >> 6) : 0;
-        int sink_tiles = (p.n_init + BN - 1) >> 6;
-        nblk = min(sink_tiles, t_lo);            // number of leading sink tiles
-        return nblk + (m - t_lo + 1);
-    } else {
-        nblk = m + 1;
-        return nblk;
-    }
-}
-
-template <int MODE>
-__device__ __forceinline__ Tile tile_at(const AttnParams &p, long long ridx, int m, int nblk, int it) {
-    Tile t;
-    t.gathered = 0;
-    t.nvalid = BN;
-    if constexpr (MODE == MODE_VS) {
-        if (it < nblk) {
-            t.start = as_const(p.bo)[ridx * p.nnz_s + it];
-        } else {
-            t.gathered = 1;
-            t.start = (it - nblk) * BN;
-            t.nvalid = min(BN, min(as_const(p.cc)[ridx], p.nnz_v) - t.start);
-        }
-    } else if constexpr (MODE == MODE_BS) {
-        t.start = as_const(p.bidx)[((ridx / p.rows) * p.bidx_rows + m) * p.max_blocks + it] * BN;
-    } else if constexpr (MODE == MODE_ASHAPE) {
-        int lo_key = m * BM - p.n_local + 1;
-        int t_lo = lo_key > 0 ? (lo_key >> 6) : 0;
-        t.start = (it < nblk ? it : t_lo + (it - nblk)) * BN;
-    } else {
-        t.start = it * BN;
-    }
-    return t;
-}
-
-// Paired variant: one workgroup of 4 waves covers the row blocks mA = 2*mp and mB = mA + 1.  It
+// One workgroup of 4 waves covers the row blocks mA = 2*mp and mB = mA + 1.  It
 // walks the union of their two tile lists once, so every K/V tile is copied into LDS once for 128
 // query rows; a half skips the tiles that are not on its own list.  For dense causal and A-shape /
 // tri-shape the lists are analytic and differ by at most the ends (the three helpers below); for
@@ -273,8 +217,8 @@ __device__ __forceinline__ bool tile_on_list(const AttnParams &p, int m, int sta
 
 // LDS of one workgroup (declared by the kernel, see attn_fwd_kernel): separate objects, so that the
 // compiler lets reads of one overtake copies into the other.
-template <int MODE, bool PAIR, int HD> struct AttnLds {
-    static constexpr bool VSP = PAIR && (MODE == MODE_VS || MODE == MODE_BS);      // walks of two block lists
+template <int MODE, int HD> struct AttnLds {
+    static constexpr bool VSP = MODE == MODE_VS || MODE == MODE_BS;      // walks of two block lists
     static constexpr int TILE_BYTES = BN * HD * 2;
     static constexpr int NK = (VSP ? 2 : 1) * TILE_BYTES;
     static constexpr int NONLY = VSP ? 2 * VS_ONLY_MAX : 1;
@@ -284,10 +228,10 @@ template <int MODE, bool PAIR, int HD> struct AttnLds {
 // only where it is needed (see sm_pv_block), and the function returns true -- for the whole
 // workgroup -- when a row sum left the safe range, i.e. when the walk has to be run again with
 // EVERY_MAX (the output it wrote is then overwritten).
-template <typename T, int MODE, bool PAIR, int HD, bool EVERY_MAX>
-__device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[AttnLds<MODE, PAIR, HD>::NK],
-                                          char (&lds_v)[AttnLds<MODE, PAIR, HD>::NK],
-                                          int (&vs_only)[AttnLds<MODE, PAIR, HD>::NONLY], int (&vs_wsum)[4], int &vs_bad,
+template <typename T, int MODE, int HD, bool EVERY_MAX>
+__device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[AttnLds<MODE, HD>::NK],
+                                          char (&lds_v)[AttnLds<MODE, HD>::NK],
+                                          int (&vs_only)[AttnLds<MODE, HD>::NONLY], int (&vs_wsum)[4], int &vs_bad,
                                           int &lds_redo) {
     static_assert(HD == 128 || HD == 64, "head_dim 128 or 64");
     constexpr int ROW_BYTES = HD * 2;                       // one token row of K / V / Q / O
@@ -300,11 +244,11 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
     // K chunk ^ (row/2)%8, V chunk ^ 4*((row/2)%2)
     auto swz_k = [](int row) { return HD == 128 ? (row & 15) : ((row >> 1) & 7); };
     auto swz_v = [](int row) { return HD == 128 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); };
-    constexpr int NT = PAIR ? 2 * NTHREADS : NTHREADS;      // threads per workgroup
-    constexpr int CROWS = PAIR ? 16 : 32;                   // tile rows copied by one wave (shared tile)
+    constexpr int NT = 2 * NTHREADS;                        // threads per workgroup
+    constexpr int CROWS = 16;                               // tile rows copied by one wave (shared tile)
     // VSP: the paired walk of two block lists -- the vertical-slash block lists, or the block-sparse
     // lists (block numbers, i.e. key starts / 64; no columns)
-    constexpr bool VSP = PAIR && (MODE == MODE_VS || MODE == MODE_BS);
+    constexpr bool VSP = MODE == MODE_VS || MODE == MODE_BS;
     constexpr int LIST_SCALE = MODE == MODE_BS ? BN : 1;     // list entry -> first key of the block
     constexpr int TILE_BYTES = BN * ROW_BYTES;
     constexpr int VS_PAIR_MAX = TILE_BYTES / 8;             // both staged lists fit the second K tile
@@ -329,7 +273,7 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
     // modes have near-constant work per row block once the context is long and then measure 1 %
     // faster in ascending order; up to 64K tokens their early row blocks are still growing and the
     // descending order wins for vertical-slash lists (+4 % at 16K, +1.7 % at 32K): the launcher picks.
-    const int rows_wg = PAIR ? (p.rows + 1) >> 1 : p.rows;           // row-block slots per (batch, head)
+    const int rows_wg = (p.rows + 1) >> 1;                           // row-block pairs per (batch, head)
     const int mi = (int)(rest % rows_wg); rest /= rows_wg;
     const int mslot = p.descending ? rows_wg - 1 - mi : mi;
     int hkv, b, h, hs;                               // hs: head position in the index tensors
@@ -353,10 +297,10 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
     const int tid = (int)threadIdx.x;
     const int lane = tid & 63;
     const int wave_wg = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: keep it in an SGPR
-    const int half = PAIR ? wave_wg >> 1 : 0;                        // which row block of the pair
-    const int wave = PAIR ? wave_wg & 1 : wave_wg;                   // wave inside the row block
-    const int m = PAIR ? 2 * mslot + half : mslot;
-    const int mA = PAIR ? 2 * mslot : mslot, mB = PAIR ? min(mA + 1, p.rows - 1) : mslot;
+    const int half = wave_wg >> 1;                                   // which row block of the pair
+    const int wave = wave_wg & 1;                                    // wave inside the row block
+    const int m = 2 * mslot + half;
+    const int mA = 2 * mslot, mB = min(mA + 1, p.rows - 1);
     const int l32 = lane & 31;
     const int g = lane >> 5;
 
@@ -365,7 +309,7 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
     const int qrow = row0 + wave * 32 + l32;          // this lane's query row
     char *o_base = p.o + ((long long)b * p.os[0] + (long long)h * p.os[1]) * 2;
 
-    // row block past the sequence: zeros (16 B per lane-step); in the paired variant the other
+    // row block past the sequence: zeros (16 B per lane-step); the other
     // half may still have work, so this half stays for the copies and barriers without tiles
     const bool have_rows = m < p.rows && row0 < seqlen;
     if (!have_rows) {
@@ -374,7 +318,7 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
                 int r = row0 + i / NCH;
                 if (r < p.n) *reinterpret_cast<u32x4_t *>(o_base + (long long)r * p.os[2] * 2 + (i % NCH) * 16) = u32x4_t{0u, 0u, 0u, 0u};
             }
-        if (!PAIR || mA * BM >= seqlen) return false;   // (wave-uniform; for a pair: both halves are past)
+        if (mA * BM >= seqlen) return false;            // (workgroup-uniform: both halves are past)
     }
 
     const char *q_base = p.q + ((long long)b * p.qs[0] + (long long)h * p.qs[1]) * 2;
@@ -507,7 +451,7 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
         ntiles = vs_nc + max(nt_a, nt_b);
     }
     else
-        ntiles = PAIR ? pair_tile_count<MODE>(p, mA, mB, nblk) : tile_count<MODE>(p, ridx, m, nblk);
+        ntiles = pair_tile_count<MODE>(p, mA, mB, nblk);
     auto more_tiles = [&](int it) -> bool { return it < ntiles; };   // is there a tile number `it` ?
     // paired vertical-slash: entry it+1 of the common list sits in a scalar when step `it` starts; the
     // LDS read of entry it+2 is issued at the top of step `it` (no tile copy is in flight there: the
@@ -541,15 +485,13 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
                 }
             }
             return t;
-        } else if constexpr (PAIR) {
+        } else {
             Tile t;
             t.gathered = 0;
             t.nvalid = BN;
             t.on_a = t.on_b = 1;
             t.start = pair_tile_start<MODE>(p, mA, mB, nblk, it);
             return t;
-        } else {
-            return tile_at<MODE>(p, ridx, m, nblk, it);
         }
     };
 
@@ -662,12 +604,8 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
     for (int db = 0; db < NDB; ++db)
         v_rd_off[db] = (4 * g + v_rd_rsub) * ROW_BYTES + ((((db << 2) + v_rd_vc) ^ swz_v(v_rd_rsub)) << 4) + ((lane & 1) << 3);
 
-    // ---- S^T = K . Q^T for this wave's 32 query rows; K tile in kbuf.  EARLY (2-wave kernel, whose
-    // waves all run this code): the tile's second barrier comes after k-step EARLY_B2, when every K
-    // fragment has been read, and all V^T fragment reads are issued under the last four MFMAs.
-    auto qk_block = [&](const char *kbuf, const char *vbuf, f32x16_t &s0, f32x16_t &s1, Frag (&vf)[4][NDB], auto early_c) {
-        constexpr bool EARLY = decltype(early_c)::value;
-        constexpr int EARLY_AT = EARLY_B2 * KS / 8;       // the k-step after which every K fragment has been read
+    // ---- S^T = K . Q^T for this wave's 32 query rows; K tile in kbuf.
+    auto qk_block = [&](const char *kbuf, f32x16_t &s0, f32x16_t &s1) {
         Frag a0[KS], a1[KS];
         __builtin_amdgcn_s_setprio(2);
 #pragma unroll
@@ -689,28 +627,13 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
             s0 = Mma<T>::mfma(frag_as<T>(a0[ks]), frag_as<T>(qf[ks]), s0);
             s1 = Mma<T>::mfma(frag_as<T>(a1[ks]), frag_as<T>(qf[ks]), s1);
             __builtin_amdgcn_sched_barrier(0);
-            if constexpr (EARLY) {
-                if (ks == EARLY_AT) {
-                    __builtin_amdgcn_s_waitcnt(0x0f70);
-                    __syncthreads();
-#pragma unroll
-                    for (int s = 0; s < 4; ++s)
-#pragma unroll
-                        for (int db = 0; db < NDB; ++db)
-#pragma unroll
-                            for (int jj = 0; jj < 2; ++jj)
-                                vf[s][db].s4[jj] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                                    (__attribute__((address_space(3))) short4_t *)(vbuf + v_rd_off[db] + (16 * s + 8 * jj) * ROW_BYTES));
-                }
-            }
         }
         __builtin_amdgcn_s_setprio(0);
     };
 
-    // ---- mask, online softmax, O^T += V^T . P^T.  READ_V: the V^T fragments have not been read yet
-    // (4-wave variants, whose second barrier sits between the two blocks).
-    auto sm_pv_block = [&](const Tile &cur, const char *vbuf, f32x16_t &s0, f32x16_t &s1, Frag (&vf)[4][NDB], auto read_v_c) {
-        constexpr bool READ_V = decltype(read_v_c)::value;
+    // ---- mask, V^T fragment reads, online softmax, O^T += V^T . P^T
+    auto sm_pv_block = [&](const Tile &cur, const char *vbuf, f32x16_t &s0, f32x16_t &s1) {
+        Frag vf[4][NDB];
         // element (blk, r) of this lane is tile-local key tk = tkc + 4*g with the compile-time
         // part tkc = 32*blk + 8*(r/4) + r%4.  keep <=> tk <= hi && (tk > wlo || tk < slim).
         bool need_mask;
@@ -753,7 +676,7 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
             }
         }
 
-        if constexpr (READ_V) {
+        {
         // All V^T fragments of the tile are read here, in one scheduling region with the row-max
         // chain: the PV block below is bound by its vector instructions, so every LDS read moved out
         // of it shortens it (+3 % for the 24 reads that used to sit between its MFMAs), and the reads
@@ -915,22 +838,19 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
             gt_nxt = gather_ids(nxt);
         }
 
-        // paired variant: is this tile on the list of this wave's row block ?
+        // is this tile on the list of this wave's row block ?
         bool active = true;
         if constexpr (COMMON || SPLIT) active = have_rows;
-        else if constexpr (PAIR && (MODE == MODE_BS || MODE == MODE_VS)) active = have_rows && (half ? cur.on_b : cur.on_a);   // (split steps: on_a == on_b == own flag)
-        else if constexpr (PAIR) active = have_rows && tile_on_list<MODE>(p, m, cur.start);
+        else if constexpr (VSP) active = have_rows && (half ? cur.on_b : cur.on_a);   // (split steps: on_a == on_b == own flag)
+        else active = have_rows && tile_on_list<MODE>(p, m, cur.start);
         f32x16_t s0, s1;
-        Frag vf[4][NDB];
-        if (active) qk_block(lds_k, lds_v, s0, s1, vf, std::integral_constant<bool, !PAIR>{});
-        if constexpr (PAIR) {
-            __builtin_amdgcn_s_waitcnt(0x0f70);      // vmcnt(0): this wave's part of V(it) is in LDS
-            __syncthreads();
-        }
+        if (active) qk_block(lds_k, s0, s1);
+        __builtin_amdgcn_s_waitcnt(0x0f70);          // vmcnt(0): this wave's part of V(it) is in LDS
+        __syncthreads();
         if constexpr (COMMON) copy_rows(nxt, k_base, k_row, std::false_type{}, 0, lds_k, std::integral_constant<int, CROWS>{}, wave_wg);
         else if constexpr (SPLIT) copy_rows(nxt, k_base, k_row, std::false_type{}, 0, lds_k + half * TILE_BYTES, std::integral_constant<int, 32>{}, wave);
         else if (have_nxt) copy_tile(nxt, k_base, k_row, std::false_type{}, gt_nxt, lds_k);
-        if (active) sm_pv_block(cur, lds_v, s0, s1, vf, std::integral_constant<bool, PAIR>{});
+        if (active) sm_pv_block(cur, lds_v, s0, s1);
         if constexpr (SPLIT) sp_entry = __builtin_amdgcn_readfirstlane(vs_pref);
         else if constexpr (VSP) vs_entry = __builtin_amdgcn_readfirstlane(vs_pref);
         cur = nxt;
@@ -969,11 +889,11 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
         float l_tot = l_i + __shfl_xor(l_i, 32);
         const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
         // pitch: 8-byte lane writes spread over all banks (four waves only fit without the pad)
-        constexpr int OP = PAIR ? ROW_BYTES : ROW_BYTES + 8;
+        constexpr int OP = ROW_BYTES;
         // a row sum at 2^100 or beyond (or no number at all): some probability may have overflowed
         if (!every_max && __any(!(l_tot < 0x1p100f)) && lane == 0) lds_redo = 1;
         __syncthreads();                                  // K/V tiles no longer needed
-        char *ot = PAIR ? (half ? lds_v : lds_k) + wave * 32 * OP : (wave ? lds_v : lds_k);   // 32 rows per wave
+        char *ot = (half ? lds_v : lds_k) + wave * 32 * OP;    // 32 rows per wave
         const bool live = qrow < seqlen;
 #pragma unroll
         for (int db = 0; db < NDB; ++db)
@@ -998,9 +918,9 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
     return !every_max && lds_redo != 0;                   // (workgroup-uniform)
 }
 
-template <typename T, int MODE, bool PAIR, int HD>
-__global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_kernel(const AttnParams p) {
-    typedef AttnLds<MODE, PAIR, HD> L;
+template <typename T, int MODE, int HD>
+__global__ __launch_bounds__(2 * NTHREADS, 2) void attn_fwd_kernel(const AttnParams p) {
+    typedef AttnLds<MODE, HD> L;
     __shared__ __attribute__((aligned(16))) char lds_k[L::NK];
     __shared__ __attribute__((aligned(16))) char lds_v[L::NK];
     __shared__ int vs_only[L::NONLY];        // paired list walks: [row block][entries the other list lacks]
@@ -1009,13 +929,13 @@ __global__ __launch_bounds__(PAIR ? 2 * NTHREADS : NTHREADS, 2) void attn_fwd_ke
     __shared__ int lds_redo;
     if (threadIdx.x == 0) lds_redo = 0;      // (ordered before its readers by the barriers of the walk)
     if constexpr (std::is_same<T, __bf16>::value) {
-        if (attn_walk<T, MODE, PAIR, HD, false>(p, lds_k, lds_v, vs_only, vs_wsum, vs_bad, lds_redo)) {
+        if (attn_walk<T, MODE, HD, false>(p, lds_k, lds_v, vs_only, vs_wsum, vs_bad, lds_redo)) {
             __syncthreads();                 // everyone has read the flag and is done with LDS
-            attn_walk<T, MODE, PAIR, HD, true>(p, lds_k, lds_v, vs_only, vs_wsum, vs_bad, lds_redo);
+            attn_walk<T, MODE, HD, true>(p, lds_k, lds_v, vs_only, vs_wsum, vs_bad, lds_redo);
         }
     } else {
         // f16 probabilities have no headroom above the lazy threshold: the maximum of every tile
-        attn_walk<T, MODE, PAIR, HD, true>(p, lds_k, lds_v, vs_only, vs_wsum, vs_bad, lds_redo);
+        attn_walk<T, MODE, HD, true>(p, lds_k, lds_v, vs_only, vs_wsum, vs_bad, lds_redo);
     }
 }
 
@@ -1065,20 +985,18 @@ void fill_params(AttnParams &p, const minf_qkvo *t) {
 
 template <int MODE, int HD> int launch_hd(AttnParams p, int dtype, void *stream) {
     if (p.batch == 0 || p.rows == 0) return MINF_OK;
-    // every mode runs on the paired (4-wave) kernel
-    constexpr bool pair = true;
     // heads of the grid: all of them, or the selected ones rounded up to whole chunks of hq / hk
     const int group = p.hq / p.hk;
     const long long grid_heads = p.head_list ? (long long)((p.index_heads + group - 1) / group) * group : p.hq;
-    p.total_wg = (long long)p.batch * grid_heads * (pair ? (p.rows + 1) / 2 : p.rows);
+    p.total_wg = (long long)p.batch * grid_heads * ((p.rows + 1) / 2);
     p.descending = MODE == MODE_DENSE || (MODE == MODE_VS && p.rows <= 1024);
     const long long per_xcd = (p.total_wg + 7) >> 3;
     const long long grid = per_xcd * 8;
     if (grid > 0x7fffffffLL) return MINF_ERR_UNSUPPORTED;
-    const dim3 block(pair ? 2 * NTHREADS : NTHREADS);
+    const dim3 block(2 * NTHREADS);
     hipStream_t st = (hipStream_t)stream;
-    if (dtype == MINF_BF16) hipLaunchKernelGGL((attn_fwd_kernel<__bf16, MODE, pair, HD>), dim3((unsigned)grid), block, 0, st, p);
-    else hipLaunchKernelGGL((attn_fwd_kernel<_Float16, MODE, pair, HD>), dim3((unsigned)grid), block, 0, st, p);
+    if (dtype == MINF_BF16) hipLaunchKernelGGL((attn_fwd_kernel<__bf16, MODE, HD>), dim3((unsigned)grid), block, 0, st, p);
+    else hipLaunchKernelGGL((attn_fwd_kernel<_Float16, MODE, HD>), dim3((unsigned)grid), block, 0, st, p);
     return minf_launch_status();
 }
 
