@@ -14,9 +14,9 @@
 //            registers, one (max, sum) pair per row per 2048-key chunk;
 //   reduce : combine the chunk pairs into M_i = max_i + log2(sum_i);
 //   scores : S = Q.K^T    -> lane <-> key: p = exp2(s - M_row); column sums are
-//            in-lane adds (+ one cross-half shuffle); for the diagonal sums each wave parks
-//            its 64x32 probability block in LDS and every lane walks one diagonal with
-//            conflict-free strided reads (no atomics); the per-chunk window is written out whole;
+//            in-lane adds (+ one cross-half shuffle); the diagonal sums are formed in registers
+//            with whole-wave lane shifts (one DPP add per query row, see est_scores_kernel; no
+//            LDS tile, no atomics); the per-chunk window is written out whole;
 //   finalize: stitch the chunk windows together (each diagonal gets at most two
 //            pieces, added in a fixed order) and apply the forced +inf entries.
 // Work split: a workgroup owns one 2048-key chunk of one group of up to four query heads that are
@@ -168,20 +168,23 @@ __global__ __launch_bounds__(EST_THREADS, 3) void est_stats_kernel(const EstPara
             const int i = 32 * nb + l32;
             // key c is visible to row i iff c <= qpos0 + i, c < n, i < last_q
             const int hi = (i < p.last_q ? min(qpos0 + i, p.n - 1) : -1) - c0 - 4 * g;
-            float mx = -INFINITY;
+            if (edge) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int tkc = 8 * (r >> 2) + (r & 3);
-                float sc = st[nb][r] * p.scale_log2;
-                if (edge) sc = (tkc <= hi) ? sc : -INFINITY;
-                st[nb][r] = sc;
-                mx = fmaxf(mx, sc);
+                for (int r = 0; r < 16; ++r) {
+                    const int tkc = 8 * (r >> 2) + (r & 3);
+                    st[nb][r] = (tkc <= hi) ? st[nb][r] : -INFINITY;
+                }
             }
-            const float m_new = fmaxf(m_run[nb], mx);
+            // maximum of the raw scores (the scale is positive), three operands at a time
+            float mx = fmaxf(fmaxf(st[nb][0], st[nb][1]), st[nb][2]);
+#pragma unroll
+            for (int r = 3; r + 1 < 16; r += 2) mx = fmaxf(fmaxf(mx, st[nb][r]), st[nb][r + 1]);
+            mx = fmaxf(mx, st[nb][15]);
+            const float m_new = fmaxf(m_run[nb], mx * p.scale_log2);
             const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
             float sum = 0.f;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) sum += __builtin_amdgcn_exp2f(st[nb][r] - m_use);
+            for (int r = 0; r < 16; ++r) sum += __builtin_amdgcn_exp2f(fmaf(st[nb][r], p.scale_log2, -m_use));
             l_run[nb] = l_run[nb] * __builtin_amdgcn_exp2f(m_run[nb] - m_use) + sum;
             m_run[nb] = m_new;
         }
@@ -239,22 +242,25 @@ __global__ __launch_bounds__(LQ) void est_reduce_kernel(const EstParams p) {
 }
 
 // --------------------------------------------------------------- scores sweep
-// Diagonal sums without LDS float atomics (those run at a fraction of a lane per clock):
-// every wave parks its 64 x 32 probability block in a private LDS tile with a row pitch of
-// 33 floats, then lane d walks "its" diagonal (row i, key i + d) with conflict-free strided
-// reads -- 64 lanes cover d = -63..0, a second pass d = 1..31 -- and adds the 95 sums into a
-// private per-wave window with plain read-modify-write (one wave, in-order LDS: no race).
-constexpr int TP = 33;                       // tile row pitch (floats)
-constexpr int TROWS = 94;                    // 32 rows of a half block, 31 zero rows above, 31 below
+// Diagonal sums in registers.  A 32 x 32 probability block has one key per lane (n = lane % 32) and
+// its rows in registers, two per register (row il in lanes 0-31, row il + 4 in lanes 32-63).
+// v_permlane32_swap against a zero register turns each register into two 64-lane vectors "row il
+// in lanes 0-31, zeros above"; then  acc = shift_up_one_lane(acc) + row_i  for i = 0 .. 31 (one
+// v_add_f32 with the whole-wave DPP shift wave_shr:1 per row) leaves in lane L the sum of the
+// diagonal n - i = L - 31: 16 swaps + 32 adds per block instead of 32 LDS writes, 64 LDS reads and
+// 64 adds (LDS float atomics, tried first, run at a fraction of a lane per clock).  The 63 sums
+// are added into a private per-wave window in LDS with plain read-modify-write (one wave,
+// in-order LDS: no race).
 constexpr int WWIN = KC + LQ;                // per-wave diagonal window: at most the whole chunk + 64
+__device__ __forceinline__ float wave_shr1(float x) {      // lane L <- lane L - 1, lane 0 <- 0
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x138, 0xf, 0xf, true));
+}
 
 // (min 2 waves per SIMD: caps the kernel at 256 registers; it is latency bound and one resident
 // wave per SIMD ran 1.4x slower)
 template <typename T, int HD>
 __global__ __launch_bounds__(EST_THREADS, 2) void est_scores_kernel(const EstParams p) {
     constexpr int KS = HD / 16;
-    // the four waves' tiles overlap in their zero rows: wave w starts 63 rows after wave w-1
-    __shared__ float lds_tile[(3 * 63 + TROWS) * TP];
     __shared__ float lds_wwin[4][WWIN];
     const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const WgId w = decode_wg(p, wave, true);
@@ -263,11 +269,9 @@ __global__ __launch_bounds__(EST_THREADS, 2) void est_scores_kernel(const EstPar
     const int nq = 4 / p.gw, klen = KC / nq;          // key sub-ranges per head, keys per wave
     const int wwin_len = klen + LQ;
     const long long bh = (long long)w.b * p.index_heads + w.slot;
-    float *tile = lds_tile + wave * 63 * TP;
     float *wwin = lds_wwin[wave];
 
     for (int i = lane; i < wwin_len; i += 64) wwin[i] = 0.f;
-    for (int i = tid; i < (3 * 63 + TROWS) * TP; i += EST_THREADS) lds_tile[i] = 0.f;
     __syncthreads();
 
     if (w.wave_valid) {
@@ -297,6 +301,7 @@ __global__ __launch_bounds__(EST_THREADS, 2) void est_scores_kernel(const EstPar
         const int c = c0 + l32;                 // this lane's key
         const bool edge = c0 + 31 > qpos0 || c0 + 32 > p.n;
         float colsum = 0.f;
+        float pr[2][16];
 #pragma unroll
         for (int mb = 0; mb < 2; ++mb) {
             f32x16_t sc;
@@ -308,24 +313,41 @@ __global__ __launch_bounds__(EST_THREADS, 2) void est_scores_kernel(const EstPar
             for (int r = 0; r < 16; ++r) {
                 const int il = 8 * (r >> 2) + 4 * g + (r & 3);      // row inside this 32-row half
                 const int i = 32 * mb + il;
-                float pr = __builtin_amdgcn_exp2f(fmaf(sc[r], p.scale_log2, -mrow[mb][r]));
-                if (edge) pr = (c <= qpos0 + i && c < p.n) ? pr : 0.f;
-                colsum += pr;
-                tile[(31 + il) * TP + l32] = pr;
+                float x = __builtin_amdgcn_exp2f(fmaf(sc[r], p.scale_log2, -mrow[mb][r]));
+                if (edge) x = (c <= qpos0 + i && c < p.n) ? x : 0.f;
+                colsum += x;
+                pr[mb][r] = x;
             }
-            __builtin_amdgcn_wave_barrier();
-            // the 32x32 block has 63 diagonals d = n - il in [-31, 31]; lane <-> d + 31 walks its
-            // diagonal through rows n + 31 - lane, i.e. tile rows n + 62 - lane: rows outside
-            // [31, 62] are never written and stay zero, so no lane needs a bounds test and every
-            // read address is one per-lane base plus a constant
-            const float *dp = tile + (62 - min(lane, 62)) * TP;
-            float ds = 0.f;
+        }
+        // the 63 diagonals d = n - il in [-31, 31] of each 32 x 32 block: rows in ascending order,
+        // one lane shift between two rows, the two blocks' chains interleaved
+        float dacc[2] = {0.f, 0.f};
 #pragma unroll
-            for (int n = 0; n < 32; ++n) ds += dp[n * (TP + 1)];
-            // global diagonal: key - row = (32*blk + n) - (32*mb + il) -> window slot + 63 - rshift
+        for (int q4 = 0; q4 < 4; ++q4) {
+            float lo[2][4], hi[2][4];
+#pragma unroll
+            for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(pr[mb][4 * q4 + j]), 0u, false, false);
+                    lo[mb][j] = __uint_as_float(sw[0]);      // row 8*q4 + j     in lanes 0-31, zeros above
+                    hi[mb][j] = __uint_as_float(sw[1]);      // row 8*q4 + 4 + j in lanes 0-31, zeros above
+                }
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int mb = 0; mb < 2; ++mb) dacc[mb] = wave_shr1(dacc[mb]) + lo[mb][j];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int mb = 0; mb < 2; ++mb) dacc[mb] = wave_shr1(dacc[mb]) + hi[mb][j];
+        }
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb) {
+            // lane <-> d + 31; global diagonal: key - row = (32*blk + n) - (32*mb + il) -> window
+            // slot + 63 - rshift
             const int slot = 32 * blk + lane + 32 - 32 * mb - rshift;
-            if (lane < 63 && slot >= 0) wwin[slot] += ds;
-            __builtin_amdgcn_wave_barrier();
+            if (lane < 63 && slot >= 0) wwin[slot] += dacc[mb];
         }
         colsum += __shfl_xor(colsum, 32);
         if (g == 0 && c < p.n) vout[c] = colsum;
