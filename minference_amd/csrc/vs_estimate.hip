@@ -127,6 +127,70 @@ __device__ __forceinline__ void load_k(const EstParams &p, const char *kb, int c
     for (int ks = 0; ks < KS; ++ks) kf[ks].u = *reinterpret_cast<const u32x4_t *>(rp + ks * 32);
 }
 
+// K tiles shared through LDS.  When the heads of a workgroup read the same kv head (the usual
+// case: the query heads of a kv group), the waves that sweep the same keys fetch every 32-key
+// block of K once, together, straight into LDS (buffer_load ... lds, 16 bytes per lane, whole rows:
+// fully coalesced) and read their MFMA operand fragments from there, instead of every wave
+// fetching the same rows from global memory in 32-byte pieces.  Two buffers per key stream: the
+// next block is on its way while this one is scored; one workgroup barrier per block.
+// Rows are 2*HD bytes; their 16-byte chunks are XOR-permuted on the global-address side so that the
+// fragment reads of 32 rows hit distinct banks (HD 128: chunk ^ row%16; HD 64: chunk ^ (row/2)%8).
+template <int HD> struct KShare {
+    static constexpr int ROWB = HD * 2, NCH = ROWB / 16, RPI = 64 / NCH, TILE = 32 * ROWB;
+    static constexpr int MAXI = 16 / RPI;                    // copy instructions per wave at gw == 2
+    static __device__ __forceinline__ int swz(int row) { return HD == 128 ? (row & 15) : ((row >> 1) & 7); }
+    const char *kb;            // K of the common kv head
+    char *tiles;               // this stream's two tiles
+    long long rowstride;       // bytes
+    int n, rows_w, row0_w, ninstr;
+    int voff[MAXI];
+    __device__ __forceinline__ void init(const EstParams &p, const char *kb_, char *tiles_, int lane, int ws) {
+        kb = kb_; tiles = tiles_; rowstride = p.ks[2] * 2; n = p.n;
+        rows_w = 32 / p.gw; row0_w = rows_w * ws; ninstr = rows_w / RPI;
+        const int rin = lane / NCH, ch = lane % NCH;
+#pragma unroll
+        for (int j = 0; j < MAXI; ++j) voff[j] = rin * (int)rowstride + ((ch ^ swz(row0_w + RPI * j + rin)) << 4);
+    }
+    // this wave's share of the block of keys c0 .. c0+31 -> buffer `buf` (rows >= n are not fetched:
+    // their scores are masked by the callers)
+    __device__ __forceinline__ void copy(int c0, int buf) const {
+#if defined(__HIP_DEVICE_COMPILE__)      // (the LDS-DMA builtins do not exist in the host pass, which would
+                                         // then drop the kernels that use this function without a word)
+        if (c0 >= n) return;
+        const char *tb = kb + (long long)c0 * rowstride;
+        const int nrows = min(32, n - c0);
+        const __amdgpu_buffer_rsrc_t srd = __builtin_amdgcn_make_buffer_rsrc((void *)tb, 0, (nrows - 1) * (int)rowstride + ROWB, 0x00020000);
+        const int lds0 = (int)(unsigned)(unsigned long long)(__attribute__((address_space(3))) char *)(tiles + buf * TILE) + row0_w * ROWB;
+#pragma unroll
+        for (int j = 0; j < MAXI; ++j)
+            if (j < ninstr)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(srd, (__attribute__((address_space(3))) void *)(unsigned long long)(unsigned)(lds0 + RPI * j * ROWB),
+                                                         16, voff[j], (row0_w + RPI * j) * (int)rowstride, 0, 0);
+#endif
+    }
+    template <int KS> __device__ __forceinline__ void frags(int buf, int lane, Frag (&kf)[KS]) const {
+        const int l32 = lane & 31, g = lane >> 5;
+        const char *t = tiles + buf * TILE + l32 * ROWB;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) kf[ks].u = *reinterpret_cast<const u32x4_t *>(t + (((2 * ks + g) ^ swz(l32)) << 4));
+    }
+};
+
+// Do the (valid) heads of this workgroup read one kv head?  -> that head, or -1.  (All waves call
+// this; it contains a workgroup barrier.)
+__device__ __forceinline__ int common_kv_head(const EstParams &p, const WgId &w, int wave, int lane, int (&lds_hkv)[4]) {
+    if (lane == 0) lds_hkv[wave] = w.wave_valid ? w.hkv : -1;
+    __syncthreads();
+    int common = -1;
+    bool same = true;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        const int h = lds_hkv[v];
+        if (h >= 0) { if (common < 0) common = h; else same = same && h == common; }
+    }
+    return (p.gw >= 2 && same) ? common : -1;
+}
+
 // ---------------------------------------------------------------- stats sweep
 template <typename T, int HD>
 __global__ __launch_bounds__(EST_THREADS, 3) void est_stats_kernel(const EstParams p) {
@@ -140,20 +204,16 @@ __global__ __launch_bounds__(EST_THREADS, 3) void est_stats_kernel(const EstPara
 
     // lane <-> query rows i = l32 and 32 + l32; regs <-> keys 8*(r/4) + 4*g + r%4 of the block
     float m_run[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.f, 0.f};
-    if (w.wave_valid) {
-    const char *kb = p.k + ((long long)w.b * p.ks[0] + (long long)w.hkv * p.ks[1]) * 2;
+    __shared__ __attribute__((aligned(16))) char lds_kt[2][2 * KShare<HD>::TILE];
+    __shared__ int lds_hkv[4];
+    const int kv_common = common_kv_head(p, w, wave, lane, lds_hkv);       // (workgroup-uniform)
     Frag qf[2][KS];
-    load_q(p, w, lane, qf);
+    if (w.wave_valid) load_q(p, w, lane, qf);
     const int key_begin = w.chunk * KC + w.kq * klen;
     const int qpos0 = p.n - p.last_q;          // absolute position of query row 0
-    Frag kf[KS], kn[KS];
-    load_k(p, kb, key_begin, lane, kn);
-    for (int blk = 0; blk < klen / 32; ++blk) {
-        const int c0 = key_begin + blk * 32;
-        if (c0 >= p.n) break;
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) kf[ks] = kn[ks];
-        load_k(p, kb, min(c0 + 32, p.n - 1), lane, kn);      // next block, in flight during this one
+    const int nblk = klen / 32;
+    // scores one 32-key block whose K fragments are in kf
+    auto score_block = [&](int c0, const Frag (&kf)[KS]) {
         f32x16_t st[2];
 #pragma unroll
         for (int nb = 0; nb < 2; ++nb) {
@@ -188,7 +248,34 @@ __global__ __launch_bounds__(EST_THREADS, 3) void est_stats_kernel(const EstPara
             l_run[nb] = l_run[nb] * __builtin_amdgcn_exp2f(m_run[nb] - m_use) + sum;
             m_run[nb] = m_new;
         }
-    }
+    };
+    if (kv_common >= 0) {
+        KShare<HD> ks_;
+        ks_.init(p, p.k + ((long long)w.b * p.ks[0] + (long long)kv_common * p.ks[1]) * 2, lds_kt[w.kq & 1], lane, wave % p.gw);
+        ks_.copy(key_begin, 0);
+        for (int blk = 0; blk < nblk; ++blk) {
+            const int c0 = key_begin + blk * 32;
+            __builtin_amdgcn_s_waitcnt(0x0f70);      // vmcnt(0): this wave's share of block blk is in LDS
+            __syncthreads();                         // ... and everybody's; everyone is done with block blk-1
+            if (blk + 1 < nblk) ks_.copy(c0 + 32, (blk + 1) & 1);
+            if (w.wave_valid && c0 < p.n) {
+                Frag kf[KS];
+                ks_.template frags<KS>(blk & 1, lane, kf);
+                score_block(c0, kf);
+            }
+        }
+    } else if (w.wave_valid) {
+        const char *kb = p.k + ((long long)w.b * p.ks[0] + (long long)w.hkv * p.ks[1]) * 2;
+        Frag kf[KS], kn[KS];
+        load_k(p, kb, key_begin, lane, kn);
+        for (int blk = 0; blk < nblk; ++blk) {
+            const int c0 = key_begin + blk * 32;
+            if (c0 >= p.n) break;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) kf[ks] = kn[ks];
+            load_k(p, kb, min(c0 + 32, p.n - 1), lane, kn);      // next block, in flight during this one
+            score_block(c0, kf);
+        }
     }
     // merge the two lane halves, then the waves that share a head
 #pragma unroll
@@ -274,30 +361,27 @@ __global__ __launch_bounds__(EST_THREADS, 2) void est_scores_kernel(const EstPar
     for (int i = lane; i < wwin_len; i += 64) wwin[i] = 0.f;
     __syncthreads();
 
-    if (w.wave_valid) {
-    const char *kb = p.k + ((long long)w.b * p.ks[0] + (long long)w.hkv * p.ks[1]) * 2;
+    __shared__ __attribute__((aligned(16))) char lds_kt[2][2 * KShare<HD>::TILE];
+    __shared__ int lds_hkv[4];
+    const int kv_common = common_kv_head(p, w, wave, lane, lds_hkv);       // (workgroup-uniform)
     Frag qf[2][KS];
-    load_q(p, w, lane, qf);
     // lane <-> key; reg r of block mb <-> query row i = 32*mb + 8*(r/4) + 4*g + r%4
     float mrow[2][16];
+    if (w.wave_valid) {
+        load_q(p, w, lane, qf);
 #pragma unroll
-    for (int mb = 0; mb < 2; ++mb)
+        for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-            mrow[mb][r] = p.rowstat[bh * LQ + 32 * mb + 8 * (r >> 2) + 4 * g + (r & 3)];
-
+            for (int r = 0; r < 16; ++r)
+                mrow[mb][r] = p.rowstat[bh * LQ + 32 * mb + 8 * (r >> 2) + 4 * g + (r & 3)];
+    }
     const int key_begin = w.chunk * KC + w.kq * klen;
     const int qpos0 = p.n - p.last_q;
     const int rshift = LQ - p.last_q;          // rows are indexed as if last_q were 64
     float *vout = p.vertical + bh * p.n;
-    Frag kf[KS], kn[KS];
-    load_k(p, kb, key_begin, lane, kn);
-    for (int blk = 0; blk < klen / 32; ++blk) {
-        const int c0 = key_begin + blk * 32;
-        if (c0 >= p.n) break;
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) kf[ks] = kn[ks];
-        load_k(p, kb, min(c0 + 32, p.n - 1), lane, kn);      // next block, in flight during this one
+    const int nblk = klen / 32;
+    // scores one 32-key block whose K fragments are in kf -> this lane's column sum (both lane halves)
+    auto score_block = [&](int blk, int c0, const Frag (&kf)[KS]) -> float {
         const int c = c0 + l32;                 // this lane's key
         const bool edge = c0 + 31 > qpos0 || c0 + 32 > p.n;
         float colsum = 0.f;
@@ -310,15 +394,21 @@ __global__ __launch_bounds__(EST_THREADS, 2) void est_scores_kernel(const EstPar
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) sc = mma<T>(qf[mb][ks], kf[ks], sc);
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int il = 8 * (r >> 2) + 4 * g + (r & 3);      // row inside this 32-row half
-                const int i = 32 * mb + il;
-                float x = __builtin_amdgcn_exp2f(fmaf(sc[r], p.scale_log2, -mrow[mb][r]));
-                if (edge) x = (c <= qpos0 + i && c < p.n) ? x : 0.f;
-                colsum += x;
-                pr[mb][r] = x;
-            }
+            for (int r = 0; r < 16; ++r) pr[mb][r] = __builtin_amdgcn_exp2f(fmaf(sc[r], p.scale_log2, -mrow[mb][r]));
         }
+        if (edge) {      // (a block of its own, kept one by the empty asm: merged into the straight-line code
+                         // the 32 compares and selects would run for every block)
+            asm volatile("");
+#pragma unroll
+            for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int i = 32 * mb + 8 * (r >> 2) + 4 * g + (r & 3);      // query row
+                    pr[mb][r] = (c <= qpos0 + i && c < p.n) ? pr[mb][r] : 0.f;
+                }
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) colsum += pr[0][r] + pr[1][r];
         // the 63 diagonals d = n - il in [-31, 31] of each 32 x 32 block: rows in ascending order,
         // one lane shift between two rows, the two blocks' chains interleaved
         float dacc[2] = {0.f, 0.f};
@@ -349,9 +439,42 @@ __global__ __launch_bounds__(EST_THREADS, 2) void est_scores_kernel(const EstPar
             const int slot = 32 * blk + lane + 32 - 32 * mb - rshift;
             if (lane < 63 && slot >= 0) wwin[slot] += dacc[mb];
         }
-        colsum += __shfl_xor(colsum, 32);
-        if (g == 0 && c < p.n) vout[c] = colsum;
-    }
+        return colsum + __shfl_xor(colsum, 32);
+    };
+    if (kv_common >= 0) {
+        KShare<HD> ks_;
+        ks_.init(p, p.k + ((long long)w.b * p.ks[0] + (long long)kv_common * p.ks[1]) * 2, lds_kt[w.kq & 1], lane, wave % p.gw);
+        ks_.copy(key_begin, 0);
+        float cs_prev = 0.f;                         // column sum of the previous block, stored a block later
+        int c_prev = -1;                             // (so that no store is waited for with the copies)
+        for (int blk = 0; blk < nblk; ++blk) {
+            const int c0 = key_begin + blk * 32;
+            __builtin_amdgcn_s_waitcnt(0x0f70);      // vmcnt(0): this wave's share of block blk is in LDS
+            __syncthreads();                         // ... and everybody's; everyone is done with block blk-1
+            if (c_prev >= 0 && g == 0 && c_prev < p.n) vout[c_prev] = cs_prev;
+            if (blk + 1 < nblk) ks_.copy(c0 + 32, (blk + 1) & 1);
+            c_prev = -1;
+            if (w.wave_valid && c0 < p.n) {
+                Frag kf[KS];
+                ks_.template frags<KS>(blk & 1, lane, kf);
+                cs_prev = score_block(blk, c0, kf);
+                c_prev = c0 + l32;
+            }
+        }
+        if (c_prev >= 0 && g == 0 && c_prev < p.n) vout[c_prev] = cs_prev;
+    } else if (w.wave_valid) {
+        const char *kb = p.k + ((long long)w.b * p.ks[0] + (long long)w.hkv * p.ks[1]) * 2;
+        Frag kf[KS], kn[KS];
+        load_k(p, kb, key_begin, lane, kn);
+        for (int blk = 0; blk < nblk; ++blk) {
+            const int c0 = key_begin + blk * 32;
+            if (c0 >= p.n) break;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) kf[ks] = kn[ks];
+            load_k(p, kb, min(c0 + 32, p.n - 1), lane, kn);      // next block, in flight during this one
+            const float cs = score_block(blk, c0, kf);
+            if (g == 0 && c0 + l32 < p.n) vout[c0 + l32] = cs;
+        }
     }
     __syncthreads();
     // chunk window of head hsub, position q = (key - chunk0) + (last_q - 1 - i): wave kq * gw + hsub
@@ -451,21 +574,23 @@ static int estimate_launch(const void *q, const void *k, const int64_t *q_stride
     const long long bh = (long long)batch * p.index_heads;       // heads of the outputs
     const bool bf = dtype == MINF_BF16;
     const dim3 g((unsigned)grid), b(EST_THREADS);
-    auto sweep = [&](auto stats_not_scores) {
-        constexpr bool STATS = decltype(stats_not_scores)::value;
-        auto go = [&](auto kern) { hipLaunchKernelGGL(kern, g, b, 0, s, p); };
-        if constexpr (STATS) {
-            if (head_dim == 128) { if (bf) go(est_stats_kernel<__bf16, 128>); else go(est_stats_kernel<_Float16, 128>); }
-            else                 { if (bf) go(est_stats_kernel<__bf16, 64>);  else go(est_stats_kernel<_Float16, 64>); }
-        } else {
-            if (head_dim == 128) { if (bf) go(est_scores_kernel<__bf16, 128>); else go(est_scores_kernel<_Float16, 128>); }
-            else                 { if (bf) go(est_scores_kernel<__bf16, 64>);  else go(est_scores_kernel<_Float16, 64>); }
-        }
-    };
-    sweep(std::true_type{});
+    // (plain launches: a kernel template whose body holds lambdas is not instantiated for the host
+    // when its address is only taken inside a generic lambda)
+#define EST_LAUNCH(kernel)                                                                          \
+    do {                                                                                            \
+        if (head_dim == 128) {                                                                      \
+            if (bf) hipLaunchKernelGGL((kernel<__bf16, 128>), g, b, 0, s, p);                       \
+            else hipLaunchKernelGGL((kernel<_Float16, 128>), g, b, 0, s, p);                        \
+        } else {                                                                                    \
+            if (bf) hipLaunchKernelGGL((kernel<__bf16, 64>), g, b, 0, s, p);                        \
+            else hipLaunchKernelGGL((kernel<_Float16, 64>), g, b, 0, s, p);                         \
+        }                                                                                           \
+    } while (0)
+    EST_LAUNCH(est_stats_kernel);
     hipLaunchKernelGGL(est_reduce_kernel, dim3((unsigned)bh), dim3(LQ), 0, s, p);
-    sweep(std::false_type{});
+    EST_LAUNCH(est_scores_kernel);
     hipLaunchKernelGGL(est_finalize_kernel, dim3((unsigned)((n + 255) / 256), (unsigned)bh), dim3(256), 0, s, p);
+#undef EST_LAUNCH
     return minf_launch_status();
 }
 
