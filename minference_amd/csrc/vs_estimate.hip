@@ -12,7 +12,8 @@
 // score tile for free):
 //   stats  : S^T = K.Q^T  -> lane <-> query row: running max / sum-of-exp in
 //            registers, one (max, sum) pair per row per 2048-key chunk;
-//   reduce : combine the chunk pairs into M_i = max_i + log2(sum_i);
+//   (every workgroup of the second sweep first combines the chunk pairs of its heads into the row
+//   constants M_i = max_i + log2(sum_i): no kernel in between)
 //   scores : S = Q.K^T    -> lane <-> key: p = exp2(s - M_row); column sums are
 //            in-lane adds (+ one cross-half shuffle); the diagonal sums are formed in registers
 //            with whole-wave lane shifts (one DPP add per query row, see est_scores_kernel; no
@@ -51,7 +52,7 @@ struct EstParams {
     float scale_log2;
     int nchunks;
     float *stats;               // [B, Hq, nchunks, LQ, 2]
-    float *rowstat;             // [B, Hq, LQ]
+    float *rowstat;             // [B, Hq, LQ] (part of the workspace layout; no longer used)
     float *win;                 // [B, Hq, nchunks, WIN]
     float *vertical, *slash;    // [B, Hq, N]
     int force_v, force_s;
@@ -311,23 +312,6 @@ __global__ __launch_bounds__(EST_THREADS, 3) void est_stats_kernel(const EstPara
     }
 }
 
-// ------------------------------------------------------------- chunk reduction
-__global__ __launch_bounds__(LQ) void est_reduce_kernel(const EstParams p) {
-    const long long bh = blockIdx.x;
-    const int i = (int)threadIdx.x;
-    const float *src = p.stats + (bh * p.nchunks * LQ + i) * 2;
-    float m = -INFINITY, l = 0.f;
-    for (int c = 0; c < p.nchunks; ++c) {
-        const float mo = src[(long long)c * LQ * 2], lo = src[(long long)c * LQ * 2 + 1];
-        const float m_new = fmaxf(m, mo);
-        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        l = l * __builtin_amdgcn_exp2f(m - m_use) + lo * __builtin_amdgcn_exp2f(mo - m_use);
-        m = m_new;
-    }
-    // rows that do not exist (i >= last_q) get +inf so that every probability is 0
-    p.rowstat[bh * LQ + i] = (i < p.last_q && l > 0.f) ? m + __builtin_amdgcn_logf(l) : INFINITY;
-}
-
 // --------------------------------------------------------------- scores sweep
 // Diagonal sums in registers.  A 32 x 32 probability block has one key per lane (n = lane % 32) and
 // its rows in registers, two per register (row il in lanes 0-31, row il + 4 in lanes 32-63).
@@ -367,13 +351,41 @@ __global__ __launch_bounds__(EST_THREADS, 2) void est_scores_kernel(const EstPar
     Frag qf[2][KS];
     // lane <-> key; reg r of block mb <-> query row i = 32*mb + 8*(r/4) + 4*g + r%4
     float mrow[2][16];
+    // Row constants M_i = max_i + log2(sum_i) of this wave's head, from the chunk statistics of the
+    // first sweep (lane <-> row; every workgroup of a head repeats this small reduction instead of a
+    // kernel of its own in between); rows that do not exist (i >= last_q) get +inf so that every
+    // probability is 0.
+    __shared__ float lds_row[4][LQ];
     if (w.wave_valid) {
         load_q(p, w, lane, qf);
+        // two passes of independent loads (sixteen in flight) instead of one chain of dependent
+        // rescales: the maximum over the chunks, then the sum of the chunk sums scaled to it
+        const float2 *src = reinterpret_cast<const float2 *>(p.stats) + bh * p.nchunks * LQ + lane;
+        float m = -INFINITY, l = 0.f;
+        for (int c0 = 0; c0 < p.nchunks; c0 += 16) {
+            float2 v[16];
+#pragma unroll
+            for (int j = 0; j < 16; ++j) v[j] = src[(long long)min(c0 + j, p.nchunks - 1) * LQ];
+#pragma unroll
+            for (int j = 0; j < 16; ++j) m = fmaxf(m, v[j].x);
+        }
+        const float m_use = (m == -INFINITY) ? 0.f : m;
+        for (int c0 = 0; c0 < p.nchunks; c0 += 16) {
+            float2 v[16];
+#pragma unroll
+            for (int j = 0; j < 16; ++j) v[j] = src[(long long)min(c0 + j, p.nchunks - 1) * LQ];
+#pragma unroll
+            for (int j = 0; j < 16; ++j) l += (c0 + j < p.nchunks) ? v[j].y * __builtin_amdgcn_exp2f(v[j].x - m_use) : 0.f;
+        }
+        lds_row[wave][lane] = (lane < p.last_q && l > 0.f) ? m + __builtin_amdgcn_logf(l) : INFINITY;
+    }
+    __syncthreads();
+    if (w.wave_valid) {
 #pragma unroll
         for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
             for (int r = 0; r < 16; ++r)
-                mrow[mb][r] = p.rowstat[bh * LQ + 32 * mb + 8 * (r >> 2) + 4 * g + (r & 3)];
+                mrow[mb][r] = lds_row[wave][32 * mb + 8 * (r >> 2) + 4 * g + (r & 3)];
     }
     const int key_begin = w.chunk * KC + w.kq * klen;
     const int qpos0 = p.n - p.last_q;
@@ -382,6 +394,13 @@ __global__ __launch_bounds__(EST_THREADS, 2) void est_scores_kernel(const EstPar
     const int nblk = klen / 32;
     // scores one 32-key block whose K fragments are in kf -> this lane's column sum (both lane halves)
     auto score_block = [&](int blk, int c0, const Frag (&kf)[KS]) -> float {
+        // The block adds to 95 slots of the diagonal window, as two disjoint ranges: s1 + (0..63) and,
+        // in lanes 32..62, s2 = s1 + 32.  Their old values are read now, a block's work ahead of the
+        // add (window slot of lane L, row half mb: 32*blk + L + 32 - 32*mb - rshift = key - row + 63 - rshift).
+        const int s1 = 32 * blk + lane - rshift, s2 = s1 + 32;
+        const bool ok1 = s1 >= 0, ok2 = lane >= 32 && lane < 63 && s2 >= 0;
+        const float w1 = ok1 ? wwin[s1] : 0.f;
+        const float w2 = ok2 ? wwin[s2] : 0.f;
         const int c = c0 + l32;                 // this lane's key
         const bool edge = c0 + 31 > qpos0 || c0 + 32 > p.n;
         float colsum = 0.f;
@@ -432,12 +451,14 @@ __global__ __launch_bounds__(EST_THREADS, 2) void est_scores_kernel(const EstPar
 #pragma unroll
                 for (int mb = 0; mb < 2; ++mb) dacc[mb] = wave_shr1(dacc[mb]) + hi[mb][j];
         }
-#pragma unroll
-        for (int mb = 0; mb < 2; ++mb) {
-            // lane <-> d + 31; global diagonal: key - row = (32*blk + n) - (32*mb + il) -> window
-            // slot + 63 - rshift
-            const int slot = 32 * blk + lane + 32 - 32 * mb - rshift;
-            if (lane < 63 && slot >= 0) wwin[slot] += dacc[mb];
+        // lane L of dacc[mb] is diagonal d = L - 31 of row half mb (lane 63 holds nothing).  Half 1 goes
+        // to s1 + L; half 0 lies 32 slots higher: its lanes 0..31 join the upper lanes of half 1, its
+        // lanes 32..62 go to s2.
+        {
+            auto sw = __builtin_amdgcn_permlane32_swap(0u, __float_as_uint(dacc[0]), false, false);
+            const float v1 = dacc[1] + __uint_as_float(sw[0]);      // (0 | lanes 0..31 of half 0)
+            if (ok1) wwin[s1] = w1 + v1;
+            if (ok2) wwin[s2] = w2 + dacc[0];
         }
         return colsum + __shfl_xor(colsum, 32);
     };
@@ -587,7 +608,6 @@ static int estimate_launch(const void *q, const void *k, const int64_t *q_stride
         }                                                                                           \
     } while (0)
     EST_LAUNCH(est_stats_kernel);
-    hipLaunchKernelGGL(est_reduce_kernel, dim3((unsigned)bh), dim3(LQ), 0, s, p);
     EST_LAUNCH(est_scores_kernel);
     hipLaunchKernelGGL(est_finalize_kernel, dim3((unsigned)((n + 255) / 256), (unsigned)bh), dim3(256), 0, s, p);
 #undef EST_LAUNCH
