@@ -6,10 +6,11 @@
 //   slash[j]    = sum_i P[i, i + j + 1 - last_q]     (diagonal sums; j <-> offset N-1-j)
 // (reference minference/modules/minference_forward.py:599-614 and :110-116).
 //
-// Two sweeps over K, both on v_mfma_f32_32x32x16 with K and Q fragments read
-// straight from global memory in operand layout (no LDS staging; the same
-// registers serve as A or B operand, so swapping the operands transposes the
-// score tile for free):
+// Two sweeps over K, both on v_mfma_f32_32x32x16 with K and Q fragments in operand layout (the
+// same registers serve as A or B operand, so swapping the operands transposes the score tile for
+// free).  Q fragments are read straight from global memory; a K block is read straight from global
+// memory too when the waves of a workgroup score different kv heads, and otherwise fetched once
+// per workgroup into LDS (LDS-DMA, double buffered) and read from there by all four waves:
 //   stats  : S^T = K.Q^T  -> lane <-> query row: running max / sum-of-exp in
 //            registers, one (max, sum) pair per row per 2048-key chunk;
 //   (every workgroup of the second sweep first combines the chunk pairs of its heads into the row
