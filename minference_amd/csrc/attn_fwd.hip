@@ -340,8 +340,6 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
         }
     }
 
-    // The row maximum of a tile is only computed when it is needed (see sm_pv_block); a walk whose
-    // row sums leave the safe range is run again with the maximum computed for every tile.
     int nblk = 0;
     // Paired list walks (vertical-slash block lists, block-sparse lists scaled to key starts): the
     // block lists of the two row blocks (ascending key starts; vertical-slash lists of
