@@ -63,9 +63,9 @@ def test_scores_far_above_the_first_tiles_are_walked_again(gpu, hot_key):
     v = torch.randn(1, hk, n, 128, generator=g)
     k[0, 0, hot_key] += 4.25
     q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
-    ref = sdpa_causal(q, expand(k, hq), expand(v, hq))
+    ref_dense = sdpa_causal(q, expand(k, hq), expand(v, hq))
     out = dense_causal_attention(q.to(gpu), k.to(gpu), v.to(gpu))
-    check(out, ref, "dense, rising scores")
+    check(out, ref_dense, "dense, rising scores")
     # the same key as a vertical line next to a local band of 128 diagonals: the gathered column
     # tile comes last in the walk of every row block
     v_idx = torch.tensor([0, 1, 2, hot_key], dtype=torch.int32).expand(1, hq, 4).contiguous()
@@ -73,6 +73,16 @@ def test_scores_far_above_the_first_tiles_are_walked_again(gpu, hot_key):
     out = vertical_slash_sparse_attention(q.to(gpu), k.to(gpu), v.to(gpu), v_idx.to(gpu), s_idx.to(gpu))
     ref = O.vertical_slash_sparse_attention(q, expand(k, hq), expand(v, hq), v_idx, s_idx)
     check(out, ref, "vertical-slash, rising scores")
+    # sink + window: the hot key enters each row block's walk through the window (or, at 70, is a sink key)
+    from minference_amd import block_sparse_attention_from_index, streaming_forward
+    out = streaming_forward(q.to(gpu), k.to(gpu), v.to(gpu), 128, 512)
+    check(out, O.streaming_forward(q, expand(k, hq), expand(v, hq), 128, 512), "a-shape, rising scores")
+    # block lists that hold every causal block (the walk of the common / leftover entries)
+    rows = n // 64 + 1
+    bi = torch.arange(rows, dtype=torch.int32).expand(1, hq, rows, rows).contiguous()
+    bi = torch.minimum(bi, torch.arange(rows, dtype=torch.int32)[None, None, :, None])
+    out = block_sparse_attention_from_index(q.to(gpu), k.to(gpu), v.to(gpu), bi.to(gpu))
+    check(out, ref_dense, "block-sparse, rising scores")
 
 
 @pytest.mark.parametrize("n,nv,ns,hq,hk,seed", [
