@@ -20,6 +20,7 @@ namespace {
 
 constexpr int TK_THREADS = 1024;
 constexpr int TK_WAVES = TK_THREADS / 64;
+constexpr int TK_DEPTH = 16;          // independent 16-byte loads per thread in the sweeps
 
 __device__ __forceinline__ unsigned order_key(float x) {
     unsigned u = __float_as_uint(x);
@@ -58,7 +59,7 @@ __global__ __launch_bounds__(TK_THREADS) void topk_kernel(const TopkProblem p0, 
     // exponents, so most lanes of a wave hit the same bin; with one copy per bank they neither
     // serialise on one address nor conflict on a bank
     __shared__ unsigned hist[256 * 32];
-    __shared__ unsigned bins[256];
+    __shared__ unsigned bins[4];             // bin counts of waves 0..3
     __shared__ unsigned sh_prefix, sh_need;
     __shared__ int sh_last;
     __shared__ int wave_gt[TK_WAVES], wave_eq[TK_WAVES];
@@ -83,14 +84,15 @@ __global__ __launch_bounds__(TK_THREADS) void topk_kernel(const TopkProblem p0, 
             const unsigned u = order_key(xv);
             if ((u & mask) == prefix) atomicAdd(&hist[(((u >> shift) & 255u) << 5) + (lane & 31)], 1u);
         };
-        // 16-byte loads over the aligned part, four in flight per thread
+        // 16-byte loads over the aligned part, TK_DEPTH in flight per thread: one workgroup sweeps a
+        // whole row, so its rate is (bytes in flight) / (memory latency) until the CU's load path fills
         int i = tid;
-        for (; i + 3 * TK_THREADS < nvec; i += 4 * TK_THREADS) {
-            float4 q[4];
+        for (; i + (TK_DEPTH - 1) * TK_THREADS < nvec; i += TK_DEPTH * TK_THREADS) {
+            float4 q[TK_DEPTH];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) q[u] = reinterpret_cast<const float4 *>(x)[i + u * TK_THREADS];
+            for (int u = 0; u < TK_DEPTH; ++u) q[u] = reinterpret_cast<const float4 *>(x)[i + u * TK_THREADS];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) { tally(q[u].x); tally(q[u].y); tally(q[u].z); tally(q[u].w); }
+            for (int u = 0; u < TK_DEPTH; ++u) { tally(q[u].x); tally(q[u].y); tally(q[u].z); tally(q[u].w); }
         }
         for (; i < nvec; i += TK_THREADS) {
             const float4 q = reinterpret_cast<const float4 *>(x)[i];
@@ -98,22 +100,30 @@ __global__ __launch_bounds__(TK_THREADS) void topk_kernel(const TopkProblem p0, 
         }
         for (int j = nvec * 4 + tid; j < n; j += TK_THREADS) tally(x[j]);
         __syncthreads();
-        if (tid < 256) {                 // fold the 32 copies of bin `tid` (rotated: one bank per thread)
-            unsigned sum = 0;
+        // Threads 0..255 fold the 32 copies of one bin each (rotated: one bank per thread), bin 255 - tid,
+        // so that an inclusive prefix scan over the threads counts the entries in this bin and above;
+        // the bin that takes the running count to `need` is the next digit of the threshold.
+        unsigned cnt = 0, incl = 0;
+        const int b = 255 - tid;
+        if (tid < 256) {
 #pragma unroll
-            for (int c = 0; c < 32; ++c) sum += hist[(tid << 5) + ((c + tid) & 31)];
-            bins[tid] = sum;
+            for (int c = 0; c < 32; ++c) cnt += hist[(b << 5) + ((c + b) & 31)];
+            incl = cnt;
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) {
+                const unsigned up = __shfl_up(incl, d);
+                if (lane >= d) incl += up;
+            }
+            if (lane == 63) bins[wave] = incl;
         }
         __syncthreads();
-        if (tid == 0) {
-            unsigned cum = 0;
-            int b = 255;
-            for (; b > 0; --b) {
-                if (cum + bins[b] >= need) break;
-                cum += bins[b];
+        if (tid < 256) {
+            for (int wv = 0; wv < wave; ++wv) incl += bins[wv];
+            const unsigned excl = incl - cnt;
+            if ((excl < need && need <= incl) || (b == 0 && incl < need)) {
+                sh_prefix = prefix | ((unsigned)b << shift);
+                sh_need = need - excl;
             }
-            sh_prefix = prefix | ((unsigned)b << shift);
-            sh_need = need - cum;
         }
         __syncthreads();
         prefix = sh_prefix;
@@ -129,11 +139,21 @@ __global__ __launch_bounds__(TK_THREADS) void topk_kernel(const TopkProblem p0, 
     int cgt = 0, ceq = 0;
     const bool vec = nvec > 0;                    // slices start at multiples of 64 elements
     const int vend = vec ? begin + ((max(end - begin, 0)) & ~255) : begin;   // whole 256-element groups
-    for (int i = begin + 4 * lane; i < vend; i += 256) {
-        const float4 q = *reinterpret_cast<const float4 *>(x + i);
+    auto count4 = [&](const float4 &q) {
         const unsigned u0 = order_key(q.x), u1 = order_key(q.y), u2 = order_key(q.z), u3 = order_key(q.w);
         cgt += (u0 > T) + (u1 > T) + (u2 > T) + (u3 > T);
         ceq += (u0 == T) + (u1 == T) + (u2 == T) + (u3 == T);
+    };
+    {
+        int i = begin + 4 * lane;
+        for (; i + (TK_DEPTH - 1) * 256 < vend; i += TK_DEPTH * 256) {
+            float4 q[TK_DEPTH];
+#pragma unroll
+            for (int u = 0; u < TK_DEPTH; ++u) q[u] = *reinterpret_cast<const float4 *>(x + i + u * 256);
+#pragma unroll
+            for (int u = 0; u < TK_DEPTH; ++u) count4(q[u]);
+        }
+        for (; i < vend; i += 256) count4(*reinterpret_cast<const float4 *>(x + i));
     }
     for (int i = vend + lane; i < end; i += 64) {
         const unsigned u = order_key(x[i]);
@@ -155,9 +175,25 @@ __global__ __launch_bounds__(TK_THREADS) void topk_kernel(const TopkProblem p0, 
     const uint64_t lt = minf_lanemask_lt();
     // 256 elements per step: lane l holds indices base + 4l .. 4l+3, so the rank of an element is
     // (selected elements of lower lanes, all four components) + (selected lower components of its lane)
-    for (int base = begin; base < vend; base += 256) {
+    constexpr int EMIT_DEPTH = 8;          // loads of this many steps go out before the first is used
+    float4 qn[EMIT_DEPTH];
+#pragma unroll
+    for (int u = 0; u < EMIT_DEPTH; ++u)
+        if (begin + u * 256 < vend) qn[u] = *reinterpret_cast<const float4 *>(x + begin + u * 256 + 4 * lane);
+    for (int base0 = begin; base0 < vend; base0 += EMIT_DEPTH * 256) {
+      float4 qc[EMIT_DEPTH];
+#pragma unroll
+      for (int u = 0; u < EMIT_DEPTH; ++u) qc[u] = qn[u];
+#pragma unroll
+      for (int u = 0; u < EMIT_DEPTH; ++u)
+          if (base0 + (EMIT_DEPTH + u) * 256 < vend)
+              qn[u] = *reinterpret_cast<const float4 *>(x + base0 + (EMIT_DEPTH + u) * 256 + 4 * lane);
+#pragma unroll
+      for (int uu = 0; uu < EMIT_DEPTH; ++uu) {
+        const int base = base0 + uu * 256;
+        if (base >= vend) break;
         const int i0 = base + 4 * lane;
-        const float4 q = *reinterpret_cast<const float4 *>(x + i0);
+        const float4 q = qc[uu];
         const unsigned u[4] = {order_key(q.x), order_key(q.y), order_key(q.z), order_key(q.w)};
         int g_lower = 0, e_lower = 0, g_all = 0, e_all = 0;
         bool gt[4], eq[4];
@@ -185,6 +221,7 @@ __global__ __launch_bounds__(TK_THREADS) void topk_kernel(const TopkProblem p0, 
         }
         gt_before += g_all;
         eq_before += e_all;
+      }
     }
     for (int base = vend; base < end; base += 64) {
         const int i = base + lane;
