@@ -315,7 +315,15 @@ __global__ __launch_bounds__(TKW_WAVES * 64, ITEMS >= 64 ? 3 : (ITEMS >= 40 ? 5 
     const unsigned diff = kmax ^ kmin;
     const int top_bit = diff ? 31 - __builtin_clz(diff) : -1;            // highest bit in which live keys differ
     unsigned T = top_bit >= 0 ? (top_bit == 31 ? 0u : (kmax >> (top_bit + 1)) << (top_bit + 1)) : kmax;
-    for (int bit = top_bit; bit >= 0; --bit) {
+    // Before the pass of `bit`, the keys that can still decide T are those that agree with T above
+    // `bit` (the bucket [T, T + 2^(bit+1))); `above` counts the keys beyond the bucket (exact),
+    // `from_t` the keys >= T (exact once T has been raised, an upper bound before).  When at most
+    // 64 keys are left in the bucket they are gathered into one register (through LDS) and the
+    // remaining passes compare that register only: an early pass costs a compare per held key, and
+    // there are about as many late passes as early ones.
+    int above = 0, from_t = (jmax + GROUP - 1) / GROUP * GROUP * 64;      // (whole register groups are visited)
+    int bit = top_bit;
+    for (; bit >= 0 && from_t - above > 64; --bit) {
         const unsigned cand = T | (1u << bit);
         // every lane counts its own keys (compare + add with carry), the lane counts (< 128) are
         // summed through seven ballots of their bits
@@ -331,8 +339,36 @@ __global__ __launch_bounds__(TKW_WAVES * 64, ITEMS >= 64 ? 3 : (ITEMS >= 40 ? 5 
 #pragma unroll
         for (int b = 0; b < (ITEMS >= 64 ? 7 : (ITEMS >= 32 ? 6 : (ITEMS >= 16 ? 5 : 3))); ++b)
             cnt += __builtin_popcountll(__ballot((c >> b) & 1)) << b;
-        if (cnt >= k) T = cand;
-        if (cnt == k) break;                         // exactly k keys are >= T: nothing left to decide
+        if (cnt >= k) { T = cand; from_t = cnt; } else above = cnt;
+        if (cnt == k) { bit = -1; break; }           // exactly k keys are >= T: nothing left to decide
+    }
+    if (bit >= 0) {
+        __shared__ unsigned bucket[TKW_WAVES][64];
+        const uint64_t lower = minf_lanemask_lt();
+        int filled = 0;
+#pragma unroll
+        for (int jb = 0; jb < ITEMS; jb += GROUP) {
+            if (jb < jmax) {
+#pragma unroll
+                for (int j = jb; j < jb + GROUP; ++j) {
+                    const bool in = ((key[j] ^ T) >> bit) >> 1 == 0u;      // agrees with T above `bit`
+                    const uint64_t m = __ballot(in);
+                    if (in) bucket[wave][filled + __builtin_popcountll(m & lower)] = key[j];
+                    filled += __builtin_popcountll(m);
+                }
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const unsigned mine = lane < filled ? bucket[wave][lane] : 0u;       // 0 lies below every candidate
+        // (`above` stays what it was at the gather: the keys beyond the gathered bucket)
+        for (; bit >= 0; --bit) {
+            const unsigned cand = T | (1u << bit);
+            const int cnt = above + __builtin_popcountll(__ballot(mine >= cand));
+            if (cnt >= k) T = cand;
+            if (cnt == k) break;
+        }
     }
     int cgt = 0;
 #pragma unroll
