@@ -190,7 +190,7 @@ __device__ __forceinline__ int common_kv_head(const EstParams &p, const WgId &w,
         const int h = lds_hkv[v];
         if (h >= 0) { if (common < 0) common = h; else same = same && h == common; }
     }
-    return (p.gw >= 2 && same) ? common : -1;
+    return __builtin_amdgcn_readfirstlane((p.gw >= 2 && same) ? common : -1);      // (uniform: keep it scalar)
 }
 
 // ---------------------------------------------------------------- stats sweep
@@ -198,7 +198,8 @@ template <typename T, int HD>
 __global__ __launch_bounds__(EST_THREADS, 3) void est_stats_kernel(const EstParams p) {
     constexpr int KS = HD / 16;       // k-steps of one 32x32 score block
     __shared__ float lds_m[4][LQ], lds_l[4][LQ];
-    const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = (int)threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);       // wave-uniform: addresses built from it stay scalar
     const WgId w = decode_wg(p, wave, false);
     if (!w.valid) return;
     const int l32 = lane & 31, g = lane >> 5;
@@ -334,7 +335,8 @@ template <typename T, int HD>
 __global__ __launch_bounds__(EST_THREADS, 2) void est_scores_kernel(const EstParams p) {
     constexpr int KS = HD / 16;
     __shared__ float lds_wwin[4][WWIN];
-    const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = (int)threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);       // wave-uniform: addresses built from it stay scalar
     const WgId w = decode_wg(p, wave, true);
     if (!w.valid) return;
     const int l32 = lane & 31, g = lane >> 5;
