@@ -12,7 +12,9 @@
 // Ties are therefore resolved towards the lowest index (torch.topk, which the
 // reference uses at minference/modules/minference_forward.py:607,612, leaves the
 // tie order unspecified), and the output needs no sort before the index
-// builder.  With reverse_base >= 0 the value written is reverse_base - index
+// builder.  Keys are compared by their bit patterns, so -0.0 ranks just below
+// +0.0 instead of tying with it (the score rows of this path hold no
+// negative zeros: they are sums of probabilities).  With reverse_base >= 0 the value written is reverse_base - index
 // (slash: diagonal offset = N-1-j, so ascending j gives descending offsets).
 #include "minf_common.h"
 
