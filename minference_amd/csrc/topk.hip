@@ -17,6 +17,7 @@
 // negative zeros: they are sums of probabilities).  With reverse_base >= 0 the value written is reverse_base - index
 // (slash: diagonal offset = N-1-j, so ascending j gives descending offsets).
 #include "minf_common.h"
+#include <type_traits>
 
 namespace {
 
@@ -173,63 +174,80 @@ __global__ __launch_bounds__(TK_THREADS) void topk_kernel(const TopkProblem p0, 
     for (int wv = 0; wv < wave; ++wv) { gt_before += wave_gt[wv]; eq_before += wave_eq[wv]; }
 
     // ---- 3. ordered emit ---------------------------------------------------
-    const int r = (int)need;
+    int r = (int)need;
     const uint64_t lt = minf_lanemask_lt();
+    // When every entry equal to T is taken (r == their number: always so when T occurs once), "selected"
+    // is simply key >= T: the loop then runs on the threshold T - 1 with no tie bookkeeping, which
+    // halves its ballots.
+    int tot_eq = 0;
+    for (int wv = 0; wv < TK_WAVES; ++wv) tot_eq += wave_eq[wv];
+    const bool all_ties = tot_eq == r && T != 0u;          // (workgroup-uniform)
+    const unsigned Te = all_ties ? T - 1u : T;
+    if (all_ties) { gt_before += eq_before; eq_before = 0; r = 0; }
     // 256 elements per step: lane l holds indices base + 4l .. 4l+3, so the rank of an element is
     // (selected elements of lower lanes, all four components) + (selected lower components of its lane)
+    auto emit4 = [&](const float4 &q, int i0, auto ties_c) {
+        constexpr bool TIES = decltype(ties_c)::value;
+        const unsigned u[4] = {order_key(q.x), order_key(q.y), order_key(q.z), order_key(q.w)};
+        int g_lower = 0, e_lower = 0, g_all = 0, e_all = 0;
+        bool gt[4], eq[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            gt[c] = u[c] > Te;
+            const uint64_t mg = __ballot(gt[c]);
+            g_lower += __builtin_popcountll(mg & lt);
+            g_all += __builtin_popcountll(mg);
+            eq[c] = false;
+            if constexpr (TIES) {
+                eq[c] = u[c] == Te;
+                const uint64_t me = __ballot(eq[c]);
+                e_lower += __builtin_popcountll(me & lt);
+                e_all += __builtin_popcountll(me);
+            }
+        }
+        if (TIES || g_all) {                               // (wave-uniform)
+            int g_here = gt_before + g_lower, e_here = eq_before + e_lower;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                if (gt[c] || (eq[c] && e_here < r)) {
+                    const int i = i0 + c;
+                    const int pos = g_here + min(e_here, r), val = reverse_base >= 0 ? reverse_base - i : i;
+                    o[pos] = val;
+                    if (pos == k - 1) sh_last = val;
+                }
+                g_here += gt[c];
+                e_here += eq[c];
+            }
+        }
+        gt_before += g_all;
+        eq_before += e_all;
+    };
     constexpr int EMIT_DEPTH = 8;          // loads of this many steps go out before the first is used
     float4 qn[EMIT_DEPTH];
 #pragma unroll
     for (int u = 0; u < EMIT_DEPTH; ++u)
         if (begin + u * 256 < vend) qn[u] = *reinterpret_cast<const float4 *>(x + begin + u * 256 + 4 * lane);
     for (int base0 = begin; base0 < vend; base0 += EMIT_DEPTH * 256) {
-      float4 qc[EMIT_DEPTH];
+        float4 qc[EMIT_DEPTH];
 #pragma unroll
-      for (int u = 0; u < EMIT_DEPTH; ++u) qc[u] = qn[u];
+        for (int u = 0; u < EMIT_DEPTH; ++u) qc[u] = qn[u];
 #pragma unroll
-      for (int u = 0; u < EMIT_DEPTH; ++u)
-          if (base0 + (EMIT_DEPTH + u) * 256 < vend)
-              qn[u] = *reinterpret_cast<const float4 *>(x + base0 + (EMIT_DEPTH + u) * 256 + 4 * lane);
+        for (int u = 0; u < EMIT_DEPTH; ++u)
+            if (base0 + (EMIT_DEPTH + u) * 256 < vend)
+                qn[u] = *reinterpret_cast<const float4 *>(x + base0 + (EMIT_DEPTH + u) * 256 + 4 * lane);
 #pragma unroll
-      for (int uu = 0; uu < EMIT_DEPTH; ++uu) {
-        const int base = base0 + uu * 256;
-        if (base >= vend) break;
-        const int i0 = base + 4 * lane;
-        const float4 q = qc[uu];
-        const unsigned u[4] = {order_key(q.x), order_key(q.y), order_key(q.z), order_key(q.w)};
-        int g_lower = 0, e_lower = 0, g_all = 0, e_all = 0;
-        bool gt[4], eq[4];
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            gt[c] = u[c] > T;
-            eq[c] = u[c] == T;
-            const uint64_t mg = __ballot(gt[c]), me = __ballot(eq[c]);
-            g_lower += __builtin_popcountll(mg & lt);
-            e_lower += __builtin_popcountll(me & lt);
-            g_all += __builtin_popcountll(mg);
-            e_all += __builtin_popcountll(me);
+        for (int uu = 0; uu < EMIT_DEPTH; ++uu) {
+            const int base = base0 + uu * 256;
+            if (base >= vend) break;
+            if (all_ties) emit4(qc[uu], base + 4 * lane, std::false_type{});
+            else emit4(qc[uu], base + 4 * lane, std::true_type{});
         }
-        int g_here = gt_before + g_lower, e_here = eq_before + e_lower;
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            if (gt[c] || (eq[c] && e_here < r)) {
-                const int i = i0 + c;
-                const int pos = g_here + min(e_here, r), val = reverse_base >= 0 ? reverse_base - i : i;
-                o[pos] = val;
-                if (pos == k - 1) sh_last = val;
-            }
-            g_here += gt[c];
-            e_here += eq[c];
-        }
-        gt_before += g_all;
-        eq_before += e_all;
-      }
     }
     for (int base = vend; base < end; base += 64) {
         const int i = base + lane;
         unsigned u = 0;
         bool gt = false, eq = false;
-        if (i < end) { u = order_key(x[i]); gt = u > T; eq = u == T; }
+        if (i < end) { u = order_key(x[i]); gt = u > Te; eq = !all_ties && u == Te; }
         const uint64_t mg = __ballot(gt), me = __ballot(eq);
         const int g_here = gt_before + __builtin_popcountll(mg & lt);
         const int e_here = eq_before + __builtin_popcountll(me & lt);
