@@ -83,25 +83,37 @@ __global__ __launch_bounds__(TK_THREADS) void topk_kernel(const TopkProblem p0, 
     for (int shift = 24; shift >= 0; shift -= 8) {
         for (int i = tid; i < 256 * 32; i += TK_THREADS) hist[i] = 0;
         __syncthreads();
-        auto tally = [&](float xv) {
-            const unsigned u = order_key(xv);
-            if ((u & mask) == prefix) atomicAdd(&hist[(((u >> shift) & 255u) << 5) + (lane & 31)], 1u);
+        // After the first pass the keys that still matter form one bucket [prefix, prefix + width) that
+        // lies wholly among the positive or wholly among the negative floats (the sign is part of the
+        // first digit), i.e. one range of raw bit patterns: membership is a subtract and an unsigned
+        // compare on the raw bits, and only members (few) are turned into keys.
+        const unsigned width = shift < 24 ? 1u << (shift + 8) : 0u;
+        const unsigned raw_base = (prefix & 0x80000000u) ? (prefix ^ 0x80000000u) : ~(prefix + width - 1u);
+        auto sweep = [&](auto first_c) {
+            constexpr bool FIRST = decltype(first_c)::value;        // first pass: every entry counts
+            auto tally = [&](float xv) {
+                if (FIRST || __float_as_uint(xv) - raw_base < width) {
+                    const unsigned u = order_key(xv);
+                    atomicAdd(&hist[(((u >> shift) & 255u) << 5) + (lane & 31)], 1u);
+                }
+            };
+            // 16-byte loads over the aligned part, TK_DEPTH in flight per thread: one workgroup sweeps a
+            // whole row, so its rate is (bytes in flight) / (memory latency) until the CU's load path fills
+            int i = tid;
+            for (; i + (TK_DEPTH - 1) * TK_THREADS < nvec; i += TK_DEPTH * TK_THREADS) {
+                float4 q[TK_DEPTH];
+#pragma unroll
+                for (int u = 0; u < TK_DEPTH; ++u) q[u] = reinterpret_cast<const float4 *>(x)[i + u * TK_THREADS];
+#pragma unroll
+                for (int u = 0; u < TK_DEPTH; ++u) { tally(q[u].x); tally(q[u].y); tally(q[u].z); tally(q[u].w); }
+            }
+            for (; i < nvec; i += TK_THREADS) {
+                const float4 q = reinterpret_cast<const float4 *>(x)[i];
+                tally(q.x); tally(q.y); tally(q.z); tally(q.w);
+            }
+            for (int j = nvec * 4 + tid; j < n; j += TK_THREADS) tally(x[j]);
         };
-        // 16-byte loads over the aligned part, TK_DEPTH in flight per thread: one workgroup sweeps a
-        // whole row, so its rate is (bytes in flight) / (memory latency) until the CU's load path fills
-        int i = tid;
-        for (; i + (TK_DEPTH - 1) * TK_THREADS < nvec; i += TK_DEPTH * TK_THREADS) {
-            float4 q[TK_DEPTH];
-#pragma unroll
-            for (int u = 0; u < TK_DEPTH; ++u) q[u] = reinterpret_cast<const float4 *>(x)[i + u * TK_THREADS];
-#pragma unroll
-            for (int u = 0; u < TK_DEPTH; ++u) { tally(q[u].x); tally(q[u].y); tally(q[u].z); tally(q[u].w); }
-        }
-        for (; i < nvec; i += TK_THREADS) {
-            const float4 q = reinterpret_cast<const float4 *>(x)[i];
-            tally(q.x); tally(q.y); tally(q.z); tally(q.w);
-        }
-        for (int j = nvec * 4 + tid; j < n; j += TK_THREADS) tally(x[j]);
+        if (shift == 24) sweep(std::true_type{}); else sweep(std::false_type{});
         __syncthreads();
         // Threads 0..255 fold the 32 copies of one bin each (rotated: one bank per thread), bin 255 - tid,
         // so that an inclusive prefix scan over the threads counts the entries in this bin and above;
