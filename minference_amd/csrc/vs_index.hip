@@ -72,13 +72,15 @@ __device__ __forceinline__ void copy_shifted(int32_t *dst, const int32_t *src, i
 // one in lane order with scalar arithmetic.  Returns this lane's range start; `starts` gets the
 // mask of lanes that start a range.
 __device__ __forceinline__ int chunk_ranges(int t, int lane, int cur_a, int carried_e, int carried_t,
-                                            uint64_t &starts) {
+                                            uint64_t &starts, uint64_t *gaps = nullptr) {
     int tprev = __shfl_up(t, 1);
     if (lane == 0) tprev = carried_t;
     const bool sure = lane == 0 ? (t > carried_e + 64) : (t > tprev + 127);
     const bool maybe = lane != 0 && !sure && (t > tprev + 64);
     uint64_t sm = __ballot(sure);
     uint64_t mm = __ballot(maybe);
+    // entries more than 64 above their predecessor (lane 0: above the last entry of the previous chunk)
+    if (gaps) *gaps = ((sm | mm) & ~1ull) | (minf_readlane(t, 0) > carried_t + 64 ? 1ull : 0ull);
     const uint64_t le = minf_lanemask_lt() | (1ull << lane);
     const uint64_t below = sm & le;
     const int j0 = below ? 63 - __builtin_clzll(below) : 0;
@@ -235,6 +237,10 @@ __global__ __launch_bounds__(IDX_WAVES *MINF_WAVE) void vs_index_kernel(
 //   cpre[i]   index of the first block of the range that starts at entry i, else -1
 //   crun[i]   ordinal of that range, else -1
 //   run_a[r], run_e[r]   [start, end) of range r
+//   cgaps[i]  the number of entries j <= i with t_j > t_{j-1} + 64 ("gap entries": the only entries
+//             at which a range can start, for any row block -- skipping and clipping only shrink gaps)
+//   glist[j]  the gap entries, ascending, j < ngaps (compacted from cgaps by the bitmap pass): the
+//             first gap entry at or after entry x is glist[cgaps[x - 1]]
 // all in the virtual row's coordinates (real position = virtual + end_m - V).
 // vs_index_fast_kernel then handles a row block as follows: entries from the first valid one are
 // processed exactly like vs_index_kernel until a range starts at an entry that also starts a range
@@ -243,12 +249,17 @@ __global__ __launch_bounds__(IDX_WAVES *MINF_WAVE) void vs_index_kernel(
 // are copied from cpos with a shift (coalesced), and each remaining vertical x is emitted iff it is
 // not inside one of the remaining tabulated ranges, is not below the end of the last range of the
 // explicit part, and is below the last entry's t - the reference's merge rule restated per element.
-#define IDX_TAB_HDR 4
-// per head: header, five tables of nnz_s ints, then a coverage bitmap of the virtual row (one bit
+// Inside the explicit part, a chunk of 64 entries without any gap above 64 means a dense run of
+// diagonals: the entries up to the next entry of glist cannot start a range, so they only extend
+// the current one, to a + 64 ceil((t_last - a) / 64), and their blocks are an arithmetic progression
+// written at once -- lists whose slashes cluster (the usual case near the diagonal) would otherwise
+// walk thousands of entries, 64 at a time, before they meet a tabulated range start.
+#define IDX_TAB_HDR 8
+// per head: header, seven tables of nnz_s ints, then a coverage bitmap of the virtual row (one bit
 // per key position, set inside the tabulated ranges) of bm_words 32-bit words
 __host__ __device__ __forceinline__ long long idx_bm_words(int rows) { return ((long long)rows * 64 + 64 + 31) / 32 + 1; }
 __host__ __device__ __forceinline__ long long idx_tab_ints(int nnz_s, int rows) {
-    return IDX_TAB_HDR + 5ll * nnz_s + idx_bm_words(rows);
+    return IDX_TAB_HDR + 7ll * nnz_s + idx_bm_words(rows);
 }
 
 __global__ __launch_bounds__(MINF_WAVE) void vs_index_prep_kernel(const int32_t *__restrict__ slash,
@@ -258,10 +269,10 @@ __global__ __launch_bounds__(MINF_WAVE) void vs_index_prep_kernel(const int32_t 
     const int32_t *sl = slash + bh * (long long)nnz_s;
     int32_t *hdr = tables + bh * idx_tab_ints(nnz_s, rows);
     int32_t *cpos = hdr + IDX_TAB_HDR, *cpre = cpos + nnz_s, *crun = cpre + nnz_s;
-    int32_t *run_a = crun + nnz_s, *run_e = run_a + nnz_s;
+    int32_t *run_a = crun + nnz_s, *run_e = run_a + nnz_s, *cgaps = run_e + nnz_s;
     const int V = sl[0] + 64;
 
-    int nb = 0, nr = 0;
+    int nb = 0, nr = 0, ng = 0;
     int carried_e = 0, carried_t = 0, cur_a = 0;
     const int nchunks = (nnz_s + MINF_WAVE - 1) / MINF_WAVE;
     // the walk is one chain of chunks; the list entries of the next two chunks are fetched ahead so
@@ -283,8 +294,10 @@ __global__ __launch_bounds__(MINF_WAVE) void vs_index_prep_kernel(const int32_t 
             carried_e = t0 - 64;
             carried_t = t0;
         }
-        uint64_t starts;
-        const int a = chunk_ranges(t, lane, cur_a, carried_e, carried_t, starts);
+        uint64_t starts, gm;
+        const int a = chunk_ranges(t, lane, cur_a, carried_e, carried_t, starts, &gm);
+        if (valid) cgaps[base + lane] = ng + __builtin_popcountll(gm & (minf_lanemask_lt() | (1ull << lane)));
+        ng += __builtin_popcountll(gm);             // (padding lanes repeat the last entry: never a gap)
         const bool is_start = valid && (((starts >> lane) & 1ull) || (c == 0 && lane == 0));
         const int e = a + ((((t - a) + 63) >> 6) << 6);
         int eprev = __shfl_up(e, 1);
@@ -317,6 +330,7 @@ __global__ __launch_bounds__(MINF_WAVE) void vs_index_prep_kernel(const int32_t 
         // the bitmap covers positions [0, 32 * bm_words); a list whose largest offset lies far
         // outside the context does not fit and the row blocks fall back to searching the ranges
         hdr[3] = (long long)V <= 32 * (idx_bm_words(rows) - 1) ? 1 : 0;
+        hdr[4] = ng;
     }
 }
 
@@ -327,11 +341,16 @@ __global__ __launch_bounds__(MINF_WAVE) void vs_index_prep_kernel(const int32_t 
 __global__ __launch_bounds__(256) void vs_index_bitmap_kernel(int32_t *__restrict__ tables, int nnz_s, int rows) {
     const long long bh = blockIdx.y;
     int32_t *hdr = tables + bh * idx_tab_ints(nnz_s, rows);
-    if (!hdr[3]) return;
     const int32_t *run_a = hdr + IDX_TAB_HDR + 3ll * nnz_s, *run_e = run_a + nnz_s;
-    uint32_t *bm = reinterpret_cast<uint32_t *>(hdr + IDX_TAB_HDR + 5ll * nnz_s);
+    uint32_t *bm = reinterpret_cast<uint32_t *>(hdr + IDX_TAB_HDR + 7ll * nnz_s);
     const long long w = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (w >= idx_bm_words(rows)) return;
+    if (w < nnz_s) {                           // (thread w also serves list entry w: the gap list)
+        const int32_t *cgaps = hdr + IDX_TAB_HDR + 5ll * nnz_s;
+        int32_t *glist = hdr + IDX_TAB_HDR + 6ll * nnz_s;
+        const int c = cgaps[w], cprev = w ? cgaps[w - 1] : 0;
+        if (c != cprev) glist[c - 1] = (int)w;
+    }
+    if (w >= idx_bm_words(rows) || !hdr[3]) return;
     const int nr = hdr[1];
     const long long p0 = 32 * w, p1 = p0 + 32;
     int lo = 0, hi = nr;                       // first range with run_e > p0
@@ -349,12 +368,17 @@ __global__ __launch_bounds__(256) void vs_index_bitmap_kernel(int32_t *__restric
     bm[w] = bits;
 }
 
-__global__ __launch_bounds__(IDX_WAVES *MINF_WAVE) void vs_index_fast_kernel(
+// (Two instantiations: the zero-filled form is bound by its stores and measures 3 % faster at 512K
+// tokens when the compiler is held to 64 registers; the payload-only form is bound by its chains of
+// dependent loads and loses more to the few spills that limit costs than it gains.)
+template <bool ZERO_FILL>
+__global__ __launch_bounds__(IDX_WAVES *MINF_WAVE, ZERO_FILL ? 8 : 1) void vs_index_fast_kernel(
     const int32_t *__restrict__ seqlens, const int32_t *__restrict__ vertical,
     const int32_t *__restrict__ slash, const int32_t *__restrict__ tables,
     int32_t *__restrict__ block_count, int32_t *__restrict__ block_offset,
     int32_t *__restrict__ column_count, int32_t *__restrict__ column_index, int heads, int rows,
-    int nnz_v, int nnz_s, int zero_fill, int32_t *error_flag, long long total_rows) {
+    int nnz_v, int nnz_s, int32_t *error_flag, long long total_rows) {
+    constexpr int zero_fill = ZERO_FILL ? 1 : 0;
     __shared__ int lds_t[IDX_WAVES][MINF_WAVE];
     __shared__ int lds_a[IDX_WAVES][MINF_WAVE];
     __shared__ int lds_e[IDX_WAVES][MINF_WAVE];
@@ -373,8 +397,8 @@ __global__ __launch_bounds__(IDX_WAVES *MINF_WAVE) void vs_index_fast_kernel(
     const int32_t *sl = slash + bh * (long long)nnz_s;
     const int32_t *hdr = tables + bh * idx_tab_ints(nnz_s, rows);
     const int32_t *cpos = hdr + IDX_TAB_HDR, *cpre = cpos + nnz_s, *crun = cpre + nnz_s;
-    const int32_t *run_a = crun + nnz_s, *run_e = run_a + nnz_s;
-    const uint32_t *bm = reinterpret_cast<const uint32_t *>(run_e + nnz_s);
+    const int32_t *run_a = crun + nnz_s, *run_e = run_a + nnz_s, *cgaps = run_e + nnz_s, *glist = cgaps + nnz_s;
+    const uint32_t *bm = reinterpret_cast<const uint32_t *>(glist + nnz_s);
 
     const int seqlen = seqlens[b];
     const int start_m = m * 64;
@@ -387,7 +411,7 @@ __global__ __launch_bounds__(IDX_WAVES *MINF_WAVE) void vs_index_fast_kernel(
     // loads that do not depend on each other, issued together (the kernel is bound by chains of
     // dependent loads, not by bandwidth)
     const int o_first = sl[0], o_last = sl[nnz_s - 1];
-    const int tab_blocks = hdr[0], tab_runs = hdr[1], tab_v = hdr[2], bm_ok = hdr[3];
+    const int tab_blocks = hdr[0], tab_runs = hdr[1], tab_v = hdr[2], bm_ok = hdr[3], ngaps = hdr[4];
     const bool whole_list = o_first <= end_m - 64;      // nothing skipped, nothing clipped
 
     int s0 = nnz_s;
@@ -425,25 +449,26 @@ __global__ __launch_bounds__(IDX_WAVES *MINF_WAVE) void vs_index_fast_kernel(
         if (whole_list) {
             g = 0;
         } else {
-            const int n = nnz_s - s0;
-            const int nchunks = (n + MINF_WAVE - 1) / MINF_WAVE;
             int carried_e = 0, carried_t = 0, cur_a = 0;
             int ep0 = INT_MIN;
-            for (int c = 0; c < nchunks; ++c) {
-                const int base = s0 + c * MINF_WAVE;
+            bool first = true;
+            for (int base = s0; base < nnz_s; base += MINF_WAVE) {
                 int cnt = min(MINF_WAVE, nnz_s - base);
+                const bool full = cnt == MINF_WAVE;
                 bool valid = lane < cnt;
                 int t = valid ? max(end_m - sl[base + lane], 64) : 0;
                 int tlast = minf_readlane(t, cnt - 1);
                 if (!valid) t = tlast;
-                if (c == 0) {
+                if (first) {
                     const int t0 = minf_readlane(t, 0);
                     cur_a = t0 - 64;
                     carried_e = t0 - 64;
                     carried_t = t0;
+                    first = false;
                 }
-                uint64_t starts;
-                int a = chunk_ranges(t, lane, cur_a, carried_e, carried_t, starts);
+                uint64_t starts, gm;         // gm: entries of this chunk more than 64 above their predecessor
+                int a = chunk_ranges(t, lane, cur_a, carried_e, carried_t, starts, &gm);
+                const bool any_gap = gm != 0;
                 // the first range start of this chunk that is also a tabulated range start
                 const bool tab = ((starts >> lane) & 1ull) && cpre[base + lane] >= 0;
                 const uint64_t tm = __ballot(tab);
@@ -505,6 +530,32 @@ __global__ __launch_bounds__(IDX_WAVES *MINF_WAVE) void vs_index_fast_kernel(
                     g = base + cut;
                     e_lim = carried_e;
                     break;
+                }
+                // A whole chunk without a gap: a dense run.  No range can start before the next entry of
+                // the gap list, so the entries up to there only extend the current range; their blocks
+                // are written at once and the walk resumes at that entry.
+                const int lo = base + MINF_WAVE;             // first entry not looked at yet
+                if (full && !any_gap && lo < nnz_s) {
+                    const int pos = __builtin_amdgcn_readfirstlane(cgaps[lo - 1]);   // gap entries below lo
+                    const int X = pos < ngaps ? __builtin_amdgcn_readfirstlane(glist[pos]) : nnz_s;      // first one >= lo
+                    if (X > lo) {
+                        const int t_end = max(end_m - __builtin_amdgcn_readfirstlane(sl[X - 1]), 64);
+                        const int e_end = cur_a + ((((t_end - cur_a) + 63) >> 6) << 6);
+                        const int nnew = (e_end - carried_e) >> 6;
+                        for (int j = lane; j < nnew; j += MINF_WAVE) bo_row[nb + j] = carried_e + 64 * j;
+                        nb += nnew;
+                        // the verticals below t_end lie inside the current range: none is emitted
+                        while (vp < nnz_v) {
+                            const int x = (vp + lane < nnz_v) ? vert[vp + lane] : INT_MAX;
+                            const int k = __builtin_popcountll(__ballot(x < t_end));
+                            vp += k;
+                            if (k < MINF_WAVE) break;
+                        }
+                        carried_e = e_end;
+                        carried_t = t_end;
+                        ep0 = e_end;
+                        base = X - MINF_WAVE;                // (the loop's increment makes it X)
+                    }
                 }
             }
         }
@@ -607,7 +658,8 @@ static int index_build_tables(const int32_t *seqlens, const int32_t *vertical_id
                        stream, slash_idx, workspace, nnz_s, rows);
     int status = minf_launch_status();
     if (status != MINF_OK) return status;
-    hipLaunchKernelGGL(vs_index_bitmap_kernel, dim3((unsigned)((idx_bm_words(rows) + 255) / 256), (unsigned)(batch * heads)),
+    const long long bm_threads = idx_bm_words(rows) > nnz_s ? idx_bm_words(rows) : (long long)nnz_s;   // words and list entries
+    hipLaunchKernelGGL(vs_index_bitmap_kernel, dim3((unsigned)((bm_threads + 255) / 256), (unsigned)(batch * heads)),
                        dim3(256), 0, stream, workspace, nnz_s, rows);
     status = minf_launch_status();
     if (status != MINF_OK) return status;
@@ -616,10 +668,16 @@ static int index_build_tables(const int32_t *seqlens, const int32_t *vertical_id
     // payload-only form is bound by its chains of dependent loads and wants every wave it can get.
     // Unused dynamic LDS is the occupancy limiter: 3 KB static + 24000 B -> 6 workgroups per CU.
     const unsigned occupancy_lds = zero_fill ? 24000u : 0u;
-    hipLaunchKernelGGL(vs_index_fast_kernel, dim3((unsigned)nblk), dim3(IDX_WAVES * MINF_WAVE), occupancy_lds,
-                       stream, seqlens, vertical_idx, slash_idx, (const int32_t *)workspace,
-                       block_count, block_offset, column_count, column_index, heads, rows, nnz_v, nnz_s,
-                       zero_fill, error_flag, total);
+    if (zero_fill)
+        hipLaunchKernelGGL(vs_index_fast_kernel<true>, dim3((unsigned)nblk), dim3(IDX_WAVES * MINF_WAVE), occupancy_lds,
+                           stream, seqlens, vertical_idx, slash_idx, (const int32_t *)workspace,
+                           block_count, block_offset, column_count, column_index, heads, rows, nnz_v, nnz_s,
+                           error_flag, total);
+    else
+        hipLaunchKernelGGL(vs_index_fast_kernel<false>, dim3((unsigned)nblk), dim3(IDX_WAVES * MINF_WAVE), occupancy_lds,
+                           stream, seqlens, vertical_idx, slash_idx, (const int32_t *)workspace,
+                           block_count, block_offset, column_count, column_index, heads, rows, nnz_v, nnz_s,
+                           error_flag, total);
     return minf_launch_status();
 }
 

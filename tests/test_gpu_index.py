@@ -60,11 +60,13 @@ def test_offsets_beyond_the_context(gpu, n, smax, ns, nv):
         assert_same(run_gpu([n], v, s, n, gpu), ref)
 
 
-@pytest.mark.parametrize("mode", [0, 1, 2, 3])
+@pytest.mark.parametrize("mode", [0, 1, 2, 3, 4])
 def test_structured_lists_all_rows(gpu, mode):
     """Slash lists that stress the table-driven path: clusters with gaps just below / above the
     64-token merge distance, duplicates, offsets up to n-1 (so most rows skip or clip entries and
-    join the tabulated ranges late), dense runs whose 64-phase depends on the first valid entry."""
+    join the tabulated ranges late), dense runs whose 64-phase depends on the first valid entry;
+    mode 4: runs of hundreds to thousands of consecutive or nearly consecutive offsets (what the
+    estimated slashes of a real head look like), which the row blocks cross in one step."""
     rng = np.random.default_rng(100 + mode)
     for trial in range(6):
         n = int(rng.choice([1500, 4096, 9000, 20000]))
@@ -76,6 +78,15 @@ def test_structured_lists_all_rows(gpu, mode):
         elif mode == 2:
             c = rng.integers(0, n, 6)
             sl = np.sort(np.clip(np.concatenate([cc + rng.integers(-150, 150, S // 6 + 1) for cc in c]), 0, n - 1))[::-1]
+        elif mode == 4:
+            parts, pos = [], int(rng.integers(0, 3))
+            while pos < n and sum(len(x) for x in parts) < 3000:
+                run = int(rng.choice([70, 130, 500, 2000]))
+                step = rng.choice([1, 1, 1, 2, 30, 64], size=run, p=[0.5, 0.2, 0.1, 0.1, 0.05, 0.05])
+                seg = pos + np.cumsum(step)
+                parts.append(seg[seg < n])
+                pos = int(seg[-1]) + int(rng.choice([65, 66, 100, 127, 128, 129, 191, 192, 193, 1000]))
+            sl = np.unique(np.concatenate(parts + [np.arange(3)]))[::-1]
         else:
             steps = rng.choice([1, 1, 2, 63, 64, 65, 127, 128, 129, 500], size=S)
             sl = np.cumsum(steps); sl = sl[sl < n][::-1]
@@ -116,10 +127,23 @@ def test_seqlen_shorter_than_context_and_batch(gpu):
     assert_same(run_gpu([3000, 1700], v, s, 3000, gpu), ref)
 
 
-def test_payload_only_mode(gpu):
-    v, s = gen.vs_index_inputs(2, 4096, 64, 256, seed=12)
-    ref = O.vs_index_build([4096], v, s, 4096)
-    bc, bo, cc, ci = run_gpu([4096], v, s, 4096, gpu, zero_fill=False)
+@pytest.mark.parametrize("lists", ["uniform", "dense runs"])
+def test_payload_only_mode(gpu, lists):
+    """The form without zero tails (its row-block kernel is an instantiation of its own): counts and
+    payload prefixes as in the oracle, on uniform lists and on lists made of long runs of
+    consecutive offsets."""
+    n = 4096
+    if lists == "uniform":
+        v, s = gen.vs_index_inputs(2, n, 64, 256, seed=12)
+    else:
+        rng = np.random.default_rng(12)
+        sl = [np.unique(np.concatenate([np.arange(700), 900 + np.arange(0, 400, int(st)), 1500 + np.arange(1200),
+                                        rng.integers(2800, n, 40)]))[::-1] for st in (1, 2)]
+        m = min(len(x) for x in sl)
+        s = np.ascontiguousarray(np.stack([x[-m:] for x in sl])[None].astype(np.int32))
+        v = np.sort(np.stack([rng.choice(n, size=200, replace=False) for _ in range(2)]), axis=-1)[None].astype(np.int32)
+    ref = O.vs_index_build([n], v, s, n)
+    bc, bo, cc, ci = run_gpu([n], v, s, n, gpu, zero_fill=False)
     assert np.array_equal(bc, ref[0]) and np.array_equal(cc, ref[2])
     for h in range(2):
         for m in range(64):
