@@ -90,11 +90,14 @@ template <typename T> __global__ __launch_bounds__(256) void bs_pool_kernel(cons
     }
 }
 
+constexpr int SCORE_CHUNK = 16;
+
 struct ScoreParams {
     const float *qp, *kp;     // pooled [batch*heads_q, rows, 128], [batch*heads_kv, rows, 128]
     float *scores;            // [batch*heads_q, rows, pitch]
     int heads_q, heads_kv, rows, pitch, force;
     int mtiles, ntiles;
+    int nchunks;              // chunks of SCORE_CHUNK key tiles per query tile
     int skip_masked;
     const int *head_list;     // as in PoolParams; qp and scores have index_heads heads
     int index_heads;
@@ -111,7 +114,11 @@ __device__ __forceinline__ void load_operand(const float *base, int row, int row
 __global__ __launch_bounds__(256) void bs_scores_kernel(const ScoreParams p) {
     const int lane = (int)threadIdx.x & 63, wave = (int)threadIdx.x >> 6;
     const int l32 = lane & 31, g = lane >> 5;
-    const int mt = p.mtiles - 1 - (int)blockIdx.x;            // heavy (late) query tiles first
+    // A workgroup takes one chunk of SCORE_CHUNK key tiles of one query tile (four per wave): with all
+    // key tiles of a query tile in one workgroup, the late query tiles (65 key tiles at 131072 tokens)
+    // ran for more than half of the kernel's time and the launch ended on a few such workgroups.
+    const int mt = p.mtiles - 1 - (int)blockIdx.x / p.nchunks;    // heavy (late) query tiles first
+    const int nt_begin = ((int)blockIdx.x % p.nchunks) * SCORE_CHUNK;
     const int bh = blockIdx.y;
     const int b = bh / p.index_heads, slot = bh % p.index_heads;   // (grid: batch x index_heads)
     const int h = p.head_list ? p.head_list[slot] : slot;
@@ -122,9 +129,11 @@ __global__ __launch_bounds__(256) void bs_scores_kernel(const ScoreParams p) {
     float *out = p.scores + bs * p.rows * p.pitch;
     const int m0 = mt * 32;
 
+    const int nt_stop = min(nt_begin + SCORE_CHUNK, p.skip_masked ? min(p.ntiles, (m0 + 31) / 32 + 1) : p.ntiles);
+    if (nt_begin >= nt_stop) return;                          // (chunks past the diagonal of an early query tile)
     f32x4_t aq[16], bk[16];
     load_operand(qbase, m0 + l32, p.rows, g, aq);             // A operand: query blocks -> accumulator rows
-    for (int nt = wave; nt < p.ntiles; nt += 4) {
+    for (int nt = nt_begin + wave; nt < nt_stop; nt += 4) {
         const int n0 = nt * 32;
         // tiles wholly above the diagonal hold only -inf: when the selection that follows knows
         // that (rows of at most 4096 scores), they are neither computed nor stored
@@ -211,8 +220,9 @@ int block_index_impl(const void *q, const void *k, const int64_t *q_stride, cons
 
     const bool causal_topk = rows <= 64 * 64;      // one wave per row: reads only the stored prefix of a row
     ScoreParams sp{qp, kp, scores, heads_q, heads_kv, rows, pitch, force_diag_first ? 1 : 0,
-                   (rows + 31) / 32, (pitch + 31) / 32, causal_topk ? 1 : 0, head_list, index_heads};
-    hipLaunchKernelGGL(bs_scores_kernel, dim3(sp.mtiles, batch * index_heads), dim3(256), 0, st, sp);
+                   (rows + 31) / 32, (pitch + 31) / 32, ((pitch + 31) / 32 + SCORE_CHUNK - 1) / SCORE_CHUNK,
+                   causal_topk ? 1 : 0, head_list, index_heads};
+    hipLaunchKernelGGL(bs_scores_kernel, dim3(sp.mtiles * sp.nchunks, batch * index_heads), dim3(256), 0, st, sp);
     status = minf_launch_status();
     if (status != MINF_OK) return status;
 
