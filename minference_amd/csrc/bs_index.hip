@@ -97,7 +97,8 @@ struct ScoreParams {
     float *scores;            // [batch*heads_q, rows, pitch]
     int heads_q, heads_kv, rows, pitch, force;
     int mtiles, ntiles;
-    int nchunks;              // chunks of SCORE_CHUNK key tiles per query tile
+    int mquads;               // groups of four query tiles (one workgroup each per chunk)
+    int nchunks;              // chunks of SCORE_CHUNK key tiles per group
     int skip_masked;
     const int *head_list;     // as in PoolParams; qp and scores have index_heads heads
     int index_heads;
@@ -111,13 +112,19 @@ __device__ __forceinline__ void load_operand(const float *base, int row, int row
     for (int s = 0; s < 16; ++s) x[s] = *reinterpret_cast<const f32x4_t *>(src + 8 * s);
 }
 
-__global__ __launch_bounds__(256) void bs_scores_kernel(const ScoreParams p) {
-    const int lane = (int)threadIdx.x & 63, wave = (int)threadIdx.x >> 6;
+// One workgroup: four query tiles (one per wave, A operand held in registers) against one chunk of
+// SCORE_CHUNK key tiles.  A key tile (32 pooled rows = 16 KB, contiguous in memory) is loaded once
+// per workgroup with coalesced 16-byte loads, staged in LDS (two buffers, rows padded by 16 bytes so
+// that the operand reads spread over the banks) and read from there by all four waves in MFMA
+// layout: the matrix instructions then wait for LDS, whose latency two reads in flight cover, and
+// not for L2 -- with the operand read straight from global memory the compiler keeps two of the
+// sixteen loads in flight and the matrix pipe was 45 % busy.
+constexpr int SCORE_PITCH = HD + 4;            // floats per staged row
+__global__ __launch_bounds__(256, 3) void bs_scores_kernel(const ScoreParams p) {
+    __shared__ __attribute__((aligned(16))) float lds_b[2][32 * SCORE_PITCH];
+    const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, g = lane >> 5;
-    // A workgroup takes one chunk of SCORE_CHUNK key tiles of one query tile (four per wave): with all
-    // key tiles of a query tile in one workgroup, the late query tiles (65 key tiles at 131072 tokens)
-    // ran for more than half of the kernel's time and the launch ended on a few such workgroups.
-    const int mt = p.mtiles - 1 - (int)blockIdx.x / p.nchunks;    // heavy (late) query tiles first
+    const int mq = p.mquads - 1 - (int)blockIdx.x / p.nchunks;    // heavy (late) query tiles first
     const int nt_begin = ((int)blockIdx.x % p.nchunks) * SCORE_CHUNK;
     const int bh = blockIdx.y;
     const int b = bh / p.index_heads, slot = bh % p.index_heads;   // (grid: batch x index_heads)
@@ -127,40 +134,73 @@ __global__ __launch_bounds__(256) void bs_scores_kernel(const ScoreParams p) {
     const float *qbase = p.qp + bs * p.rows * HD;
     const float *kbase = p.kp + ((long long)b * p.heads_kv + hkv) * p.rows * HD;
     float *out = p.scores + bs * p.rows * p.pitch;
+    const int mt = 4 * mq + wave;                                  // this wave's query tile (may not exist)
     const int m0 = mt * 32;
+    const bool have_q = mt < p.mtiles;
+    // tiles wholly above the diagonal hold only -inf: when the selection that follows knows that
+    // (rows of at most 4096 scores), they are neither computed nor stored; otherwise they are stored
+    // without arithmetic.  The workgroup walks up to the last tile any of its waves needs.
+    const int last_any = min(p.ntiles - 1, (min(4 * mq + 3, p.mtiles - 1) * 32 + 31) / 32);
+    const int nt_stop = min(nt_begin + SCORE_CHUNK, p.skip_masked ? last_any + 1 : p.ntiles);
+    if (nt_begin >= nt_stop) return;                               // (workgroup-uniform)
+    const int last_mine = (m0 + 31) / 32;                          // last tile this wave computes
 
-    const int nt_stop = min(nt_begin + SCORE_CHUNK, p.skip_masked ? min(p.ntiles, (m0 + 31) / 32 + 1) : p.ntiles);
-    if (nt_begin >= nt_stop) return;                          // (chunks past the diagonal of an early query tile)
-    f32x4_t aq[16], bk[16];
-    load_operand(qbase, m0 + l32, p.rows, g, aq);             // A operand: query blocks -> accumulator rows
-    for (int nt = nt_begin + wave; nt < nt_stop; nt += 4) {
-        const int n0 = nt * 32;
-        // tiles wholly above the diagonal hold only -inf: when the selection that follows knows
-        // that (rows of at most 4096 scores), they are neither computed nor stored
-        if (p.skip_masked && n0 > m0 + 31) continue;
-        f32x16_t acc;
+    f32x4_t aq[16];
+    if (have_q) load_operand(qbase, m0 + l32, p.rows, g, aq);      // A operand: query blocks -> accumulator rows
+    // staging: thread t moves the four 16-byte pieces t, t + 256, ... of the 16 KB tile
+    auto fetch = [&](int nt, f32x4_t (&st)[4]) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[r] = 0.f;
-        if (n0 <= m0 + 31) {
-            load_operand(kbase, n0 + l32, p.rows, g, bk);     // B operand: key blocks -> accumulator columns
-#pragma unroll
-            for (int s = 0; s < 16; ++s)
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(aq[s][j], bk[s][j], acc, 0, 0, 0);
+        for (int i = 0; i < 4; ++i) {
+            const int f = i * 256 + tid;                           // piece: row f / 32, floats 4 * (f % 32) ..
+            const int row = min(nt * 32 + (f >> 5), p.rows - 1);
+            st[i] = *reinterpret_cast<const f32x4_t *>(kbase + (long long)row * HD + 4 * (f & 31));
         }
-        // accumulator element r of lane l: query block m0 + 8*(r/4) + 4*g + r%4, key block n0 + l%32,
-        // so every store instruction writes two full 128-byte row segments
-        const int ncol = n0 + l32;
-        if (ncol < p.pitch) {
+    };
+    auto stage = [&](int buf, const f32x4_t (&st)[4]) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int mrow = m0 + 8 * (r >> 2) + 4 * g + (r & 3);
-                float x = ncol <= mrow ? acc[r] : -INFINITY;
-                if (p.force && (ncol == mrow || ncol == 0)) x = INFINITY;
-                if (mrow < p.rows) out[(long long)mrow * p.pitch + ncol] = x;
+        for (int i = 0; i < 4; ++i) {
+            const int f = i * 256 + tid;
+            *reinterpret_cast<f32x4_t *>(&lds_b[buf][(f >> 5) * SCORE_PITCH + 4 * (f & 31)]) = st[i];
+        }
+    };
+    f32x4_t st[4];
+    fetch(nt_begin, st);
+    stage(0, st);
+    for (int nt = nt_begin; nt < nt_stop; ++nt) {
+        const int buf = (nt - nt_begin) & 1;
+        __syncthreads();                       // tile nt is staged; everyone is done with tile nt - 1
+        const bool more = nt + 1 < nt_stop;
+        if (more) fetch(nt + 1, st);           // in flight during this tile's arithmetic
+        const int n0 = nt * 32;
+        if (have_q && !(p.skip_masked && nt > last_mine)) {
+            f32x16_t acc;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+            if (nt <= last_mine) {
+                // B operand: key blocks -> accumulator columns; lane l reads row l%32, floats 8 s + 4 g ..
+                const float *brow = &lds_b[buf][l32 * SCORE_PITCH + 4 * g];
+#pragma unroll
+                for (int s = 0; s < 16; ++s) {
+                    const f32x4_t bk = *reinterpret_cast<const f32x4_t *>(brow + 8 * s);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(aq[s][j], bk[j], acc, 0, 0, 0);
+                }
+            }
+            // accumulator element r of lane l: query block m0 + 8*(r/4) + 4*g + r%4, key block n0 + l%32,
+            // so every store instruction writes two full 128-byte row segments
+            const int ncol = n0 + l32;
+            if (ncol < p.pitch) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int mrow = m0 + 8 * (r >> 2) + 4 * g + (r & 3);
+                    float x = ncol <= mrow ? acc[r] : -INFINITY;
+                    if (p.force && (ncol == mrow || ncol == 0)) x = INFINITY;
+                    if (mrow < p.rows) out[(long long)mrow * p.pitch + ncol] = x;
+                }
             }
         }
+        if (more) stage(buf ^ 1, st);          // (that buffer was last read for tile nt - 1)
     }
 }
 
@@ -220,9 +260,9 @@ int block_index_impl(const void *q, const void *k, const int64_t *q_stride, cons
 
     const bool causal_topk = rows <= 64 * 64;      // one wave per row: reads only the stored prefix of a row
     ScoreParams sp{qp, kp, scores, heads_q, heads_kv, rows, pitch, force_diag_first ? 1 : 0,
-                   (rows + 31) / 32, (pitch + 31) / 32, ((pitch + 31) / 32 + SCORE_CHUNK - 1) / SCORE_CHUNK,
-                   causal_topk ? 1 : 0, head_list, index_heads};
-    hipLaunchKernelGGL(bs_scores_kernel, dim3(sp.mtiles * sp.nchunks, batch * index_heads), dim3(256), 0, st, sp);
+                   (rows + 31) / 32, (pitch + 31) / 32, ((rows + 31) / 32 + 3) / 4,
+                   ((pitch + 31) / 32 + SCORE_CHUNK - 1) / SCORE_CHUNK, causal_topk ? 1 : 0, head_list, index_heads};
+    hipLaunchKernelGGL(bs_scores_kernel, dim3(sp.mquads * sp.nchunks, batch * index_heads), dim3(256), 0, st, sp);
     status = minf_launch_status();
     if (status != MINF_OK) return status;
 
