@@ -306,11 +306,20 @@ __global__ __launch_bounds__(TKW_WAVES * 64, ITEMS >= 64 ? 3 : (ITEMS >= 40 ? 5 
     constexpr unsigned KEY_FLOOR = 0x007fffffu;          // order_key(-inf)
     const int stored = pr.causal_rows > 0 ? min(n, 32 * ((row % pr.causal_rows) / 32 + 1)) : n;
     unsigned key[ITEMS];
+    constexpr int LGROUP = ITEMS >= 8 ? 8 : ITEMS;
 #pragma unroll
-    for (int j = 0; j < ITEMS; ++j) {
-        const int i = j * 64 + lane;
-        // padding sorts below every real score; entries that are not stored are -inf
-        key[j] = i < stored ? order_key(x[i]) : (i < n ? KEY_FLOOR : 0u);
+    for (int jb = 0; jb < ITEMS; jb += LGROUP) {
+        if (jb * 64 < stored) {                        // (wave-uniform: groups past the stored prefix load nothing)
+#pragma unroll
+            for (int j = jb; j < jb + LGROUP; ++j) {
+                const int i = j * 64 + lane;
+                // padding sorts below every real score; entries that are not stored are -inf
+                key[j] = i < stored ? order_key(x[i]) : (i < n ? KEY_FLOOR : 0u);
+            }
+        } else {
+#pragma unroll
+            for (int j = jb; j < jb + LGROUP; ++j) key[j] = j * 64 + lane < n ? KEY_FLOOR : 0u;
+        }
     }
     // Rows with a masked (-inf) tail, e.g. block-causal score rows: when at least k entries are above
     // -inf, the threshold is too, and register groups that hold nothing above -inf can be skipped
