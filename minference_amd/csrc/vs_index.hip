@@ -25,6 +25,13 @@
 
 #define IDX_WAVES 4
 
+// value of the lane below (lane 0 gets 0): one data-parallel-primitive move, where the general
+// shuffle goes through the LDS crossbar -- the table pass is one wave walking a chain of chunks and
+// pays every cycle of it
+__device__ __forceinline__ int lane_above(int x) {
+    return __builtin_amdgcn_update_dpp(0, x, 0x138 /* wave_shr:1 */, 0xf, 0xf, true);
+}
+
 __device__ __forceinline__ void zero_range(int32_t *p, int from, int to, int lane) {
     int n = to - from;
     if (n <= 0) return;
@@ -73,7 +80,7 @@ __device__ __forceinline__ void copy_shifted(int32_t *dst, const int32_t *src, i
 // mask of lanes that start a range.
 __device__ __forceinline__ int chunk_ranges(int t, int lane, int cur_a, int carried_e, int carried_t,
                                             uint64_t &starts, uint64_t *gaps = nullptr) {
-    int tprev = __shfl_up(t, 1);
+    int tprev = lane_above(t);
     if (lane == 0) tprev = carried_t;
     const bool sure = lane == 0 ? (t > carried_e + 64) : (t > tprev + 127);
     const bool maybe = lane != 0 && !sure && (t > tprev + 64);
@@ -84,7 +91,7 @@ __device__ __forceinline__ int chunk_ranges(int t, int lane, int cur_a, int carr
     const uint64_t le = minf_lanemask_lt() | (1ull << lane);
     const uint64_t below = sm & le;
     const int j0 = below ? 63 - __builtin_clzll(below) : 0;
-    const int tj0 = __shfl(t, j0);
+    const int tj0 = sm ? __shfl(t, j0) : 0;        // (wave-uniform: no shuffle for a chunk without sure starts)
     int a = below ? tj0 - 64 : cur_a;
     while (mm) {
         const int j = __builtin_ctzll(mm);
@@ -169,7 +176,7 @@ __global__ __launch_bounds__(IDX_WAVES *MINF_WAVE) void vs_index_kernel(
             uint64_t starts;
             const int a = chunk_ranges(t, lane, cur_a, carried_e, carried_t, starts);
             const int e = a + ((((t - a) + 63) >> 6) << 6);
-            int eprev = __shfl_up(e, 1);
+            int eprev = lane_above(e);
             if (lane == 0) eprev = carried_e;
             const bool changed = valid && (e != eprev);
             const uint64_t cm = __ballot(changed);
@@ -300,7 +307,7 @@ __global__ __launch_bounds__(MINF_WAVE) void vs_index_prep_kernel(const int32_t 
         ng += __builtin_popcountll(gm);             // (padding lanes repeat the last entry: never a gap)
         const bool is_start = valid && (((starts >> lane) & 1ull) || (c == 0 && lane == 0));
         const int e = a + ((((t - a) + 63) >> 6) << 6);
-        int eprev = __shfl_up(e, 1);
+        int eprev = lane_above(e);
         if (lane == 0) eprev = carried_e;
         const bool changed = valid && (e != eprev);
         const uint64_t cm = __ballot(changed), sm = __ballot(is_start);
@@ -486,7 +493,7 @@ __global__ __launch_bounds__(IDX_WAVES *MINF_WAVE, ZERO_FILL ? 8 : 1) void vs_in
                     if (!valid) { t = tlast; a = alast; }
                 }
                 const int e = a + ((((t - a) + 63) >> 6) << 6);
-                int eprev = __shfl_up(e, 1);
+                int eprev = lane_above(e);
                 if (lane == 0) eprev = carried_e;
                 const bool changed = valid && (e != eprev);
                 const uint64_t cm = __ballot(changed);
