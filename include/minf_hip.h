@@ -106,7 +106,10 @@ int minf_vs_index_build_ws(const int32_t *seqlens, const int32_t *vertical_idx,
  * 32 heads x 6096 slashes x 524288 tokens).  All calls on one GPU share the one array: calls that
  * overlap in time on the same GPU (different streams or threads) race and must be serialised by
  * the caller.  The device address of the array is looked up once per device, on the first call
- * made with that device current.
+ * made with that device current (hipGetDevice + hipGetSymbolAddress): that FIRST call on a device
+ * must therefore be made outside stream capture (one warm-up call before capturing is enough; every
+ * later call on that device only enqueues kernels).  The array is chosen by the CURRENT device, not
+ * by `stream`: the caller must have made the stream's device current, as for any HIP launch.
  */
 #define MINF_VS_INDEX_STATIC_BYTES (8u << 20)
 int minf_vs_index_build_static(const int32_t *seqlens, const int32_t *vertical_idx,
