@@ -37,6 +37,13 @@ extern "C" {
 #define MINF_BF16 0
 #define MINF_F16 1
 
+/* Rounding of the two index selectors (pattern estimation, block index).  MINF_ROUND_NONE: fp32
+ * arithmetic on the 16-bit inputs.  MINF_ROUND_INPUT_DTYPE: round every intermediate that the
+ * reference's torch code holds in the input dtype (bf16/fp16) to that dtype, so that the selected
+ * index sets follow the reference's arithmetic and not a more precise one. */
+#define MINF_ROUND_NONE 0
+#define MINF_ROUND_INPUT_DTYPE 1
+
 /* Library version as major*10000 + minor*100 + patch. */
 int minf_version(void);
 
@@ -218,6 +225,10 @@ int minf_dense_attn_fwd(const minf_qkvo *t, void *stream);
  *   (slash[j] is the mass on the diagonal with offset n-1-j);
  *   then vertical[..., :force_vertical] = +inf and slash[..., n-force_slash:] = +inf
  *   (the reference forces 30 and 100; pass 0 to get the raw sums).
+ * rounding = MINF_ROUND_INPUT_DTYPE reproduces the reference's rounding points on bf16/fp16 tensors
+ * (:602: the einsum result is a tensor of the input dtype, and so is its quotient by sqrt(head_dim);
+ * the softmax then runs in fp32, :604): score = round(round(q.k) * sm_scale), both to `dtype`.
+ * MINF_ROUND_NONE keeps fp32 (what the reference computes on fp32 tensors).
  * q [batch, heads_q, n, head_dim], k [batch, heads_kv, n, head_dim] (head_dim 64 or 128) as base
  * pointer + element strides {batch, head, token}; last_q <= 64 (clamped to n).
  * vertical, slash: [batch, heads_q, n] fp32, contiguous.
@@ -227,7 +238,7 @@ size_t minf_vs_estimate_workspace_bytes(int batch, int heads_q, int n);
 int minf_vs_estimate(const void *q, const void *k, const int64_t *q_stride,
                      const int64_t *k_stride, int batch, int heads_q, int heads_kv, int n,
                      int head_dim, int dtype, float sm_scale, int last_q, int force_vertical,
-                     int force_slash, float *vertical, float *slash, void *workspace,
+                     int force_slash, int rounding, float *vertical, float *slash, void *workspace,
                      size_t workspace_bytes, void *stream);
 
 /*
@@ -241,7 +252,7 @@ int minf_vs_estimate(const void *q, const void *k, const int64_t *q_stride,
 int minf_vs_estimate_heads(const void *q, const void *k, const int64_t *q_stride,
                            const int64_t *k_stride, int batch, int heads_q, int heads_kv, int n,
                            int head_dim, int dtype, float sm_scale, int last_q, int force_vertical,
-                           int force_slash, const int32_t *head_list, int index_heads,
+                           int force_slash, int rounding, const int32_t *head_list, int index_heads,
                            float *vertical, float *slash, void *workspace,
                            size_t workspace_bytes, void *stream);
 
@@ -305,19 +316,24 @@ int minf_topk_indices_pair_ragged(const float *scores_a, const int32_t *k_rows_a
  * padded with 64 - n%64 zero rows, i.e. a whole extra block when n%64 == 0), every (query block,
  * key block) pair is scored with the pooled vectors, key blocks above the diagonal get -inf, and
  * the min(top_k, rows) best key blocks of every query block are written in ascending order (ties:
- * lowest block id first; torch.topk leaves the tie order unspecified).  fp32 arithmetic.
- * force_diag_first != 0 additionally keeps the diagonal block and block 0 of every query block.
+ * lowest block id first; torch.topk leaves the tie order unspecified).
+ * flags: bit 0 (MINF_BS_FORCE_DIAG_FIRST) additionally keeps the diagonal block and block 0 of every
+ * query block; bit 1 (MINF_BS_ROUND_INPUT_DTYPE) rounds the pooled means and the pooled dot
+ * products to `dtype`, as the reference's torch code does on bf16/fp16 tensors (:159-163: `mean`
+ * and `einsum` return tensors of the input dtype); without it the arithmetic is fp32 throughout.
  *   rows = minf_bs_block_index_rows(n) = (n + 64 - n%64) / 64
  *   block_index [batch, heads_q, rows, min(top_k, rows)] int32, contiguous
  *   q [batch, heads_q, n, head_dim], k [batch, heads_kv, n, head_dim] (head_dim 64 or 128): base
  *   pointer + element strides
  *   workspace: minf_bs_block_index_workspace_bytes() bytes, 16-byte aligned
  */
+#define MINF_BS_FORCE_DIAG_FIRST 1
+#define MINF_BS_ROUND_INPUT_DTYPE 2
 int minf_bs_block_index_rows(int n);
 size_t minf_bs_block_index_workspace_bytes(int batch, int heads_q, int heads_kv, int n);
 int minf_bs_block_index(const void *q, const void *k, const int64_t *q_stride,
                         const int64_t *k_stride, int batch, int heads_q, int heads_kv, int n,
-                        int head_dim, int dtype, int top_k, int force_diag_first,
+                        int head_dim, int dtype, int top_k, int flags,
                         int32_t *block_index, void *workspace, size_t workspace_bytes,
                         void *stream);
 
@@ -328,7 +344,7 @@ int minf_bs_block_index(const void *q, const void *k, const int64_t *q_stride,
  */
 int minf_bs_block_index_heads(const void *q, const void *k, const int64_t *q_stride,
                               const int64_t *k_stride, int batch, int heads_q, int heads_kv, int n,
-                              int head_dim, int dtype, int top_k, int force_diag_first,
+                              int head_dim, int dtype, int top_k, int flags,
                               const int32_t *head_list, int index_heads,
                               int32_t *block_index, void *workspace, size_t workspace_bytes,
                               void *stream);

@@ -32,9 +32,9 @@ SIGNATURES = {
     "minf_trishape_attn_fwd": (c_int, [c_ptr, c_int, c_int, c_int, c_ptr]),
     "minf_dense_attn_fwd": (c_int, [c_ptr, c_ptr]),
     "minf_vs_estimate_workspace_bytes": (ctypes.c_size_t, [c_int, c_int, c_int]),
-    "minf_vs_estimate": (c_int, [c_ptr, c_ptr, c_ptr, c_ptr] + [c_int] * 6 + [c_f32] + [c_int] * 3
+    "minf_vs_estimate": (c_int, [c_ptr, c_ptr, c_ptr, c_ptr] + [c_int] * 6 + [c_f32] + [c_int] * 4
                          + [c_ptr, c_ptr, c_ptr, ctypes.c_size_t, c_ptr]),
-    "minf_vs_estimate_heads": (c_int, [c_ptr, c_ptr, c_ptr, c_ptr] + [c_int] * 6 + [c_f32] + [c_int] * 3 + [c_ptr, c_int]
+    "minf_vs_estimate_heads": (c_int, [c_ptr, c_ptr, c_ptr, c_ptr] + [c_int] * 6 + [c_f32] + [c_int] * 4 + [c_ptr, c_int]
                                + [c_ptr, c_ptr, c_ptr, ctypes.c_size_t, c_ptr]),
     "minf_topk_indices_pair_ragged": (c_int, [c_ptr, c_ptr, c_int, c_ptr, c_i64, c_int, c_int, c_int] * 2
                                       + [c_int, c_int, c_i64, c_ptr]),
@@ -71,6 +71,8 @@ class QKVO(ctypes.Structure):
 
 
 MINF_BF16, MINF_F16 = 0, 1
+MINF_ROUND_NONE, MINF_ROUND_INPUT_DTYPE = 0, 1
+MINF_BS_FORCE_DIAG_FIRST, MINF_BS_ROUND_INPUT_DTYPE = 1, 2
 
 
 class MinfError(RuntimeError):

@@ -13,8 +13,9 @@
 //                     and, optionally, forces the diagonal block and block 0 (+inf).
 //   top-k             the shared radix-select kernel (ascending index order, ties -> lowest index).
 //
-// Arithmetic is fp32 throughout; the reference pools and multiplies in the input dtype (bf16/fp16
-// rounding after the mean and after the product), which this build does not imitate.
+// Arithmetic is fp32; with MINF_BS_ROUND_INPUT_DTYPE the pooled means and the pooled dot products
+// are rounded to the input dtype, where the reference's torch code rounds them (its `mean` and
+// `einsum` return bf16/fp16 tensors).
 #include "minf_common.h"
 #include <math.h>
 
@@ -43,6 +44,7 @@ struct PoolParams {
     // (without a list: out_heads = heads, same numbering)
     const int *head_list;
     int out_heads;
+    int round_out;            // round the means to the input dtype (stored as fp32 all the same)
 };
 
 template <typename T> __device__ __forceinline__ float to_f32(unsigned short bits);
@@ -86,7 +88,9 @@ template <typename T> __global__ __launch_bounds__(256) void bs_pool_kernel(cons
         float s = 0.f;
 #pragma unroll
         for (int r = 0; r < 16; ++r) s += red[r][tid];
-        p.out[(((long long)b * p.out_heads + slot) * p.rows + blk) * HD + tid] = s / (float)p.blk;
+        float mean = s / (float)p.blk;
+        if (p.round_out) mean = (float)(T)mean;
+        p.out[(((long long)b * p.out_heads + slot) * p.rows + blk) * HD + tid] = mean;
     }
 }
 
@@ -102,6 +106,7 @@ struct ScoreParams {
     int skip_masked;
     const int *head_list;     // as in PoolParams; qp and scores have index_heads heads
     int index_heads;
+    int round_dtype;          // -1: keep fp32 scores; MINF_BF16 / MINF_F16: round every score to that format
 };
 
 // lane l supplies row l%32 and, for MFMA step (s, j), contraction index 8*s + 4*(l/32) + j:
@@ -194,7 +199,10 @@ __global__ __launch_bounds__(256, 3) void bs_scores_kernel(const ScoreParams p) 
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int mrow = m0 + 8 * (r >> 2) + 4 * g + (r & 3);
-                    float x = ncol <= mrow ? acc[r] : -INFINITY;
+                    float v = acc[r];
+                    if (p.round_dtype == MINF_BF16) v = (float)(__bf16)v;
+                    else if (p.round_dtype == MINF_F16) v = (float)(_Float16)v;
+                    float x = ncol <= mrow ? v : -INFINITY;
                     if (p.force && (ncol == mrow || ncol == 0)) x = INFINITY;
                     if (mrow < p.rows) out[(long long)mrow * p.pitch + ncol] = x;
                 }
@@ -220,13 +228,16 @@ namespace {
 
 int block_index_impl(const void *q, const void *k, const int64_t *q_stride, const int64_t *k_stride, int batch,
                      int heads_q, int heads_kv, int n, int head_dim, int dtype, int blk, int rows, int top_k,
-                     int force_diag_first, int32_t *block_index, void *workspace, size_t workspace_bytes,
+                     int flags, int32_t *block_index, void *workspace, size_t workspace_bytes,
                      void *stream, const int32_t *head_list = nullptr, int index_heads = 0) {
     if (!q || !k || !q_stride || !k_stride || !block_index) return MINF_ERR_INVALID_ARG;
     if (head_list && index_heads <= 0) return MINF_ERR_INVALID_ARG;
     if (!head_list) index_heads = heads_q;
     if (batch < 0 || heads_q <= 0 || heads_kv <= 0 || n <= 0 || top_k <= 0) return MINF_ERR_INVALID_ARG;
     if (heads_q % heads_kv != 0) return MINF_ERR_INVALID_ARG;
+    if (flags & ~(MINF_BS_FORCE_DIAG_FIRST | MINF_BS_ROUND_INPUT_DTYPE)) return MINF_ERR_INVALID_ARG;
+    const int force_diag_first = flags & MINF_BS_FORCE_DIAG_FIRST;
+    const int rounded = (flags & MINF_BS_ROUND_INPUT_DTYPE) ? 1 : 0;
     if (head_dim != HD && head_dim != 64) return MINF_ERR_UNSUPPORTED;
     if (dtype != MINF_BF16 && dtype != MINF_F16) return MINF_ERR_UNSUPPORTED;
     if (((uintptr_t)q | (uintptr_t)k) & 15) return MINF_ERR_ALIGNMENT;
@@ -246,8 +257,8 @@ int block_index_impl(const void *q, const void *k, const int64_t *q_stride, cons
     float *scores = (float *)ws;
     hipStream_t st = (hipStream_t)stream;
 
-    PoolParams pq{(const char *)q, {q_stride[0], q_stride[1], q_stride[2]}, head_dim, qp, heads_q, n, rows, blk, head_list, index_heads};
-    PoolParams pk{(const char *)k, {k_stride[0], k_stride[1], k_stride[2]}, head_dim, kp, heads_kv, n, rows, blk, nullptr, heads_kv};
+    PoolParams pq{(const char *)q, {q_stride[0], q_stride[1], q_stride[2]}, head_dim, qp, heads_q, n, rows, blk, head_list, index_heads, rounded};
+    PoolParams pk{(const char *)k, {k_stride[0], k_stride[1], k_stride[2]}, head_dim, kp, heads_kv, n, rows, blk, nullptr, heads_kv, rounded};
     if (dtype == MINF_BF16) {
         hipLaunchKernelGGL(bs_pool_kernel<__bf16>, dim3(rows, batch * index_heads), dim3(256), 0, st, pq);
         hipLaunchKernelGGL(bs_pool_kernel<__bf16>, dim3(rows, batch * heads_kv), dim3(256), 0, st, pk);
@@ -261,7 +272,8 @@ int block_index_impl(const void *q, const void *k, const int64_t *q_stride, cons
     const bool causal_topk = rows <= 64 * 64;      // one wave per row: reads only the stored prefix of a row
     ScoreParams sp{qp, kp, scores, heads_q, heads_kv, rows, pitch, force_diag_first ? 1 : 0,
                    (rows + 31) / 32, (pitch + 31) / 32, ((rows + 31) / 32 + 3) / 4,
-                   ((pitch + 31) / 32 + SCORE_CHUNK - 1) / SCORE_CHUNK, causal_topk ? 1 : 0, head_list, index_heads};
+                   ((pitch + 31) / 32 + SCORE_CHUNK - 1) / SCORE_CHUNK, causal_topk ? 1 : 0, head_list, index_heads,
+                   rounded ? dtype : -1};
     hipLaunchKernelGGL(bs_scores_kernel, dim3(sp.mquads * sp.nchunks, batch * index_heads), dim3(256), 0, st, sp);
     status = minf_launch_status();
     if (status != MINF_OK) return status;
@@ -281,23 +293,23 @@ extern "C" size_t minf_bs_block_index_workspace_bytes(int batch, int heads_q, in
 
 extern "C" int minf_bs_block_index(const void *q, const void *k, const int64_t *q_stride,
                                    const int64_t *k_stride, int batch, int heads_q, int heads_kv,
-                                   int n, int head_dim, int dtype, int top_k, int force_diag_first,
+                                   int n, int head_dim, int dtype, int top_k, int flags,
                                    int32_t *block_index, void *workspace, size_t workspace_bytes,
                                    void *stream) {
     return block_index_impl(q, k, q_stride, k_stride, batch, heads_q, heads_kv, n, head_dim, dtype, BLK,
-                            n > 0 ? padded_rows(n) : 0, top_k, force_diag_first, block_index, workspace,
+                            n > 0 ? padded_rows(n) : 0, top_k, flags, block_index, workspace,
                             workspace_bytes, stream);
 }
 
 extern "C" int minf_bs_block_index_heads(const void *q, const void *k, const int64_t *q_stride,
                                          const int64_t *k_stride, int batch, int heads_q, int heads_kv,
-                                         int n, int head_dim, int dtype, int top_k, int force_diag_first,
+                                         int n, int head_dim, int dtype, int top_k, int flags,
                                          const int32_t *head_list, int index_heads,
                                          int32_t *block_index, void *workspace, size_t workspace_bytes,
                                          void *stream) {
     if (!head_list) return MINF_ERR_INVALID_ARG;
     return block_index_impl(q, k, q_stride, k_stride, batch, heads_q, heads_kv, n, head_dim, dtype, BLK,
-                            n > 0 ? padded_rows(n) : 0, top_k, force_diag_first, block_index, workspace,
+                            n > 0 ? padded_rows(n) : 0, top_k, flags, block_index, workspace,
                             workspace_bytes, stream, head_list, index_heads);
 }
 extern "C" size_t minf_search_block_index_workspace_bytes(int batch, int heads_q, int heads_kv, int n) {

@@ -1,7 +1,7 @@
 // Version and status text of libminf_hip.so.
 #include "minf_common.h"
 
-extern "C" int minf_version(void) { return 200; }   // 0.2.0
+extern "C" int minf_version(void) { return 300; }   // 0.3.0
 
 extern "C" size_t minf_qkvo_size(void) { return sizeof(minf_qkvo); }
 

@@ -28,8 +28,10 @@
 // trip to L2/HBM per kv head instead of one per query head.  The second sweep hands out its
 // workgroups in the reverse order of the first, so that it starts on the K chunks that the first
 // sweep touched last and finds part of K still cached.
-// All arithmetic is fp32 on 16-bit inputs (the reference rounds q.k to bf16
-// before its fp32 softmax).
+// Arithmetic is fp32 on 16-bit inputs.  With `rounding` set (template parameter RR) every score is
+// rounded where the reference's torch code rounds it on 16-bit inputs: the dot product to the input
+// dtype (the einsum's result), then the product with sm_scale to the input dtype again (the division
+// by sqrt(head_dim)), before the fp32 softmax (minference_forward.py:602-604).
 #include "minf_common.h"
 #include <math.h>
 #include <type_traits>
@@ -51,6 +53,7 @@ struct EstParams {
     long long qs[3], ks[3];     // element strides batch, head, token
     int batch, hq, hk, n, last_q;
     float scale_log2;
+    float scale;                // sm_scale itself (the rounded form scales in the natural-log domain)
     int nchunks;
     float *stats;               // [B, Hq, nchunks, LQ, 2]
     float *rowstat;             // [B, Hq, LQ] (part of the workspace layout; no longer used)
@@ -79,6 +82,15 @@ template <> __device__ __forceinline__ f32x16_t mma<__bf16>(const Frag &a, const
 template <> __device__ __forceinline__ f32x16_t mma<_Float16>(const Frag &a, const Frag &b, f32x16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a.h, b.h, c, 0, 0, 0);
 }
+
+// x rounded to the 16-bit input format and back (round to nearest even; fp16 overflows to inf like
+// torch's conversion)
+template <typename T> __device__ __forceinline__ float round_to(float x) { return (float)(T)x; }
+// the score the softmax sees, in the natural-log domain, rounded like the reference's bf16/fp16 torch ops
+template <typename T> __device__ __forceinline__ float ref_logit(float dot, float scale) {
+    return round_to<T>(round_to<T>(dot) * scale);
+}
+constexpr float LOG2E = 1.4426950408889634f;
 
 struct WgId { int b, h, hkv, chunk, slot, kq; bool valid, wave_valid; };
 
@@ -194,7 +206,7 @@ __device__ __forceinline__ int common_kv_head(const EstParams &p, const WgId &w,
 }
 
 // ---------------------------------------------------------------- stats sweep
-template <typename T, int HD>
+template <typename T, int HD, bool RR>
 __global__ __launch_bounds__(EST_THREADS, 3) void est_stats_kernel(const EstParams p) {
     constexpr int KS = HD / 16;       // k-steps of one 32x32 score block
     __shared__ float lds_m[4][LQ], lds_l[4][LQ];
@@ -215,6 +227,9 @@ __global__ __launch_bounds__(EST_THREADS, 3) void est_stats_kernel(const EstPara
     const int key_begin = w.chunk * KC + w.kq * klen;
     const int qpos0 = p.n - p.last_q;          // absolute position of query row 0
     const int nblk = klen / 32;
+    // factor that takes a score to the log2 domain: the raw dot product needs sm_scale * log2(e), a
+    // score that was already scaled and rounded only log2(e)
+    const float sl2 = RR ? LOG2E : p.scale_log2;
     // scores one 32-key block whose K fragments are in kf
     auto score_block = [&](int c0, const Frag (&kf)[KS]) {
         f32x16_t st[2];
@@ -226,6 +241,12 @@ __global__ __launch_bounds__(EST_THREADS, 3) void est_stats_kernel(const EstPara
             for (int ks = 0; ks < KS; ++ks) st[nb] = mma<T>(kf[ks], qf[nb][ks], st[nb]);
         }
         const bool edge = c0 + 31 > qpos0 || c0 + 32 > p.n;
+        if constexpr (RR) {
+#pragma unroll
+            for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) st[nb][r] = ref_logit<T>(st[nb][r], p.scale);
+        }
 #pragma unroll
         for (int nb = 0; nb < 2; ++nb) {
             const int i = 32 * nb + l32;
@@ -243,11 +264,11 @@ __global__ __launch_bounds__(EST_THREADS, 3) void est_stats_kernel(const EstPara
 #pragma unroll
             for (int r = 3; r + 1 < 16; r += 2) mx = fmaxf(fmaxf(mx, st[nb][r]), st[nb][r + 1]);
             mx = fmaxf(mx, st[nb][15]);
-            const float m_new = fmaxf(m_run[nb], mx * p.scale_log2);
+            const float m_new = fmaxf(m_run[nb], mx * sl2);
             const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
             float sum = 0.f;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) sum += __builtin_amdgcn_exp2f(fmaf(st[nb][r], p.scale_log2, -m_use));
+            for (int r = 0; r < 16; ++r) sum += __builtin_amdgcn_exp2f(fmaf(st[nb][r], sl2, -m_use));
             l_run[nb] = l_run[nb] * __builtin_amdgcn_exp2f(m_run[nb] - m_use) + sum;
             m_run[nb] = m_new;
         }
@@ -331,7 +352,7 @@ __device__ __forceinline__ float wave_shr1(float x) {      // lane L <- lane L -
 
 // (min 2 waves per SIMD: caps the kernel at 256 registers; it is latency bound and one resident
 // wave per SIMD ran 1.4x slower)
-template <typename T, int HD>
+template <typename T, int HD, bool RR>
 __global__ __launch_bounds__(EST_THREADS, 2) void est_scores_kernel(const EstParams p) {
     constexpr int KS = HD / 16;
     __shared__ float lds_wwin[4][WWIN];
@@ -416,7 +437,10 @@ __global__ __launch_bounds__(EST_THREADS, 2) void est_scores_kernel(const EstPar
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) sc = mma<T>(qf[mb][ks], kf[ks], sc);
 #pragma unroll
-            for (int r = 0; r < 16; ++r) pr[mb][r] = __builtin_amdgcn_exp2f(fmaf(sc[r], p.scale_log2, -mrow[mb][r]));
+            for (int r = 0; r < 16; ++r) {
+                if constexpr (RR) pr[mb][r] = __builtin_amdgcn_exp2f(fmaf(ref_logit<T>(sc[r], p.scale), LOG2E, -mrow[mb][r]));
+                else pr[mb][r] = __builtin_amdgcn_exp2f(fmaf(sc[r], p.scale_log2, -mrow[mb][r]));
+            }
         }
         if (edge) {      // (a block of its own, kept one by the empty asm: merged into the straight-line code
                          // the 32 compares and selects would run for every block)
@@ -550,6 +574,7 @@ int fill(EstParams &p, const void *q, const void *k, const int64_t *q_stride, co
     p.batch = batch; p.hq = heads_q; p.hk = heads_kv; p.n = n;
     p.last_q = last_q < n ? last_q : n;
     p.scale_log2 = sm_scale * 1.4426950408889634f;
+    p.scale = sm_scale;
     p.nchunks = (n + KC - 1) / KC;
     const long long bh = (long long)batch * index_heads;
     const size_t stats_b = (size_t)bh * p.nchunks * LQ * 2 * sizeof(float);
@@ -585,8 +610,9 @@ static int estimate_launch(const void *q, const void *k, const int64_t *q_stride
                            int batch, int heads_q, int heads_kv, int n, int head_dim, int dtype, float sm_scale,
                            int last_q, int force_vertical, int force_slash, float *vertical, float *slash,
                            void *workspace, size_t workspace_bytes, const int32_t *head_list, int index_heads,
-                           void *stream) {
+                           int rounding, void *stream) {
     EstParams p;
+    if (rounding != MINF_ROUND_NONE && rounding != MINF_ROUND_INPUT_DTYPE) return MINF_ERR_INVALID_ARG;
     if (batch == 0) return MINF_OK;
     int st = fill(p, q, k, q_stride, k_stride, batch, heads_q, heads_kv, n, head_dim, dtype, sm_scale,
                   last_q, force_vertical, force_slash, vertical, slash, workspace, workspace_bytes,
@@ -600,40 +626,47 @@ static int estimate_launch(const void *q, const void *k, const int64_t *q_stride
     const dim3 g((unsigned)grid), b(EST_THREADS);
     // (plain launches: a kernel template whose body holds lambdas is not instantiated for the host
     // when its address is only taken inside a generic lambda)
-#define EST_LAUNCH(kernel)                                                                          \
+#define EST_LAUNCH_RR(kernel, RR)                                                                   \
     do {                                                                                            \
         if (head_dim == 128) {                                                                      \
-            if (bf) hipLaunchKernelGGL((kernel<__bf16, 128>), g, b, 0, s, p);                       \
-            else hipLaunchKernelGGL((kernel<_Float16, 128>), g, b, 0, s, p);                        \
+            if (bf) hipLaunchKernelGGL((kernel<__bf16, 128, RR>), g, b, 0, s, p);                   \
+            else hipLaunchKernelGGL((kernel<_Float16, 128, RR>), g, b, 0, s, p);                    \
         } else {                                                                                    \
-            if (bf) hipLaunchKernelGGL((kernel<__bf16, 64>), g, b, 0, s, p);                        \
-            else hipLaunchKernelGGL((kernel<_Float16, 64>), g, b, 0, s, p);                         \
+            if (bf) hipLaunchKernelGGL((kernel<__bf16, 64, RR>), g, b, 0, s, p);                    \
+            else hipLaunchKernelGGL((kernel<_Float16, 64, RR>), g, b, 0, s, p);                     \
         }                                                                                           \
+    } while (0)
+#define EST_LAUNCH(kernel)                                                                          \
+    do {                                                                                            \
+        if (rounding == MINF_ROUND_INPUT_DTYPE) EST_LAUNCH_RR(kernel, true);                        \
+        else EST_LAUNCH_RR(kernel, false);                                                          \
     } while (0)
     EST_LAUNCH(est_stats_kernel);
     EST_LAUNCH(est_scores_kernel);
     hipLaunchKernelGGL(est_finalize_kernel, dim3((unsigned)((n + 255) / 256), (unsigned)bh), dim3(256), 0, s, p);
 #undef EST_LAUNCH
+#undef EST_LAUNCH_RR
     return minf_launch_status();
 }
 
 extern "C" int minf_vs_estimate(const void *q, const void *k, const int64_t *q_stride,
                                 const int64_t *k_stride, int batch, int heads_q, int heads_kv, int n,
                                 int head_dim, int dtype, float sm_scale, int last_q, int force_vertical,
-                                int force_slash, float *vertical, float *slash, void *workspace,
+                                int force_slash, int rounding, float *vertical, float *slash, void *workspace,
                                 size_t workspace_bytes, void *stream) {
     return estimate_launch(q, k, q_stride, k_stride, batch, heads_q, heads_kv, n, head_dim, dtype, sm_scale, last_q,
-                           force_vertical, force_slash, vertical, slash, workspace, workspace_bytes, nullptr, 0, stream);
+                           force_vertical, force_slash, vertical, slash, workspace, workspace_bytes, nullptr, 0,
+                           rounding, stream);
 }
 
 extern "C" int minf_vs_estimate_heads(const void *q, const void *k, const int64_t *q_stride,
                                       const int64_t *k_stride, int batch, int heads_q, int heads_kv, int n,
                                       int head_dim, int dtype, float sm_scale, int last_q, int force_vertical,
-                                      int force_slash, const int32_t *head_list, int index_heads,
+                                      int force_slash, int rounding, const int32_t *head_list, int index_heads,
                                       float *vertical, float *slash, void *workspace,
                                       size_t workspace_bytes, void *stream) {
     if (!head_list) return MINF_ERR_INVALID_ARG;
     return estimate_launch(q, k, q_stride, k_stride, batch, heads_q, heads_kv, n, head_dim, dtype, sm_scale, last_q,
                            force_vertical, force_slash, vertical, slash, workspace, workspace_bytes, head_list,
-                           index_heads, stream);
+                           index_heads, rounding, stream);
 }

@@ -34,11 +34,25 @@ def _prep16(q, k):
     return _prep(q), _prep(k)
 
 
-def vertical_slash_scores(q, k, last_q=LAST_Q, force_vertical=FORCE_VERTICAL, force_slash=FORCE_SLASH):
+def reference_rounding_for(dtype, reference_rounding=None):
+    """The rounding mode of the two index selectors: by default (None) the reference's own -- its
+    torch code holds the scaled q.k scores and the pooled block means / products in the INPUT dtype
+    (minference_forward.py:602, block_sparse_flash_attention.py:159-163), so bf16/fp16 inputs are
+    rounded at those points and fp32 inputs are not."""
+    if reference_rounding is None:
+        reference_rounding = dtype in (torch.bfloat16, torch.float16)
+    return bool(reference_rounding) and dtype != torch.float32
+
+
+def vertical_slash_scores(q, k, last_q=LAST_Q, force_vertical=FORCE_VERTICAL, force_slash=FORCE_SLASH,
+                          reference_rounding=None):
     """-> (vertical [B,H,N], slash [B,H,N]) fp32 score vectors.  ``slash[..., j]`` is the
     probability mass on the diagonal with offset ``N-1-j`` (same indexing as the reference's
-    ``sum_all_diagonal_matrix(qk)[..., :-last_q+1]``).  Forced entries are +inf."""
+    ``sum_all_diagonal_matrix(qk)[..., :-last_q+1]``).  Forced entries are +inf.
+    ``reference_rounding``: None = like the reference (bf16/fp16 inputs: scores rounded to the input
+    dtype after the dot product and after the scaling; fp32 inputs: not), False = fp32 arithmetic."""
     _check_qkv(q, k, k)
+    rounding = _lib.MINF_ROUND_INPUT_DTYPE if reference_rounding_for(q.dtype, reference_rounding) else _lib.MINF_ROUND_NONE
     head_dim = q.shape[-1]
     q16, k16 = _prep16(q, k)
     B, H, N, _ = q16.shape
@@ -54,7 +68,7 @@ def vertical_slash_scores(q, k, last_q=LAST_Q, force_vertical=FORCE_VERTICAL, fo
         st = lib.minf_vs_estimate(
             q16.data_ptr(), k16.data_ptr(), i64x3(*q16.stride()[:3]), i64x3(*k16.stride()[:3]),
             B, H, Hk, N, q16.shape[-1], _lib.MINF_BF16 if q16.dtype == torch.bfloat16 else _lib.MINF_F16,
-            float(head_dim) ** -0.5, int(last_q), int(force_vertical), int(force_slash),
+            float(head_dim) ** -0.5, int(last_q), int(force_vertical), int(force_slash), rounding,
             vertical.data_ptr(), slash.data_ptr(), ws.data_ptr(), ws_bytes, _lib.stream_ptr(dev))
     _lib.check(st, "minf_vs_estimate")
     return vertical, slash
@@ -79,14 +93,14 @@ def topk_indices(scores, k, reverse_base=-1):
 
 
 def estimate_vertical_slash(q, k, vertical_size, slash_size, last_q=LAST_Q,
-                            force_vertical=FORCE_VERTICAL, force_slash=FORCE_SLASH):
+                            force_vertical=FORCE_VERTICAL, force_slash=FORCE_SLASH, reference_rounding=None):
     """-> (v_idx [B,H,v] int32 ascending key positions, s_idx [B,H,s] int32 descending diagonal
     offsets), already in the order the index builder wants.  Sizes are clamped like the
     reference (:600): v = min(N, max(vertical_size, 30)), s = min(N, max(slash_size, 50))."""
     N = q.shape[2]
     v = min(N, max(int(vertical_size), 30))
     s = min(N, max(int(slash_size), 50))
-    vertical, slash = vertical_slash_scores(q, k, last_q, force_vertical, force_slash)
+    vertical, slash = vertical_slash_scores(q, k, last_q, force_vertical, force_slash, reference_rounding)
     return topk_vertical_slash(vertical, slash, v, s)
 
 

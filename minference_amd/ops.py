@@ -35,19 +35,23 @@ def _prep(t: torch.Tensor) -> torch.Tensor:
 
 
 _F16_SAFE_ABS = 32768.0
+_F16_TINY_ABS = 2.0 ** -10
 
 
 def _narrow_fp32(*tensors):
-    """16-bit operands for fp32 inputs.  The reference computes at the input element type
-    (pit_sparse_flash_attention_v2.py:96-99, :123 cast q and p to Q's dtype), which for fp32
-    means tl.dot's default TF32 products: 10 explicit mantissa bits.  fp16 operands have the same 10
-    bits, so fp32 tensors are narrowed to fp16 whenever every |value| is at most 32768 (one
-    max-abs reduction and a host read per call -- the fp32 path is the reference's CPU-checkable
-    case, not the serving path); otherwise to bf16 (8 bits, fp32's range).  Accumulation,
-    softmax statistics and the scale stay fp32 either way."""
+    """16-bit operands for fp32 inputs.  The reference picks fp16 operands for every input that is
+    not bf16 (pit_sparse_flash_attention_v2.py:175: ``tl.float16``; :99 and :123 cast q and p to
+    it), with fp32 accumulation.  Here fp32 tensors are narrowed to fp16 as well, unless the values
+    do not fit that format: when some |value| exceeds 32768 (fp16 would overflow) or the largest
+    |value| is below 2^-10 (fp16 would flush most of the tensor to zero or to subnormals) they are
+    narrowed to bf16 instead, which has fp32's exponent range and 8 mantissa bits.  The decision
+    costs one max-abs reduction and ONE HOST READ (a stream synchronisation) per call: the fp32 path
+    is the reference's CPU-checkable case, not the serving path.  Accumulation, softmax statistics
+    and the scale stay fp32 either way."""
     amax = torch.stack([torch.linalg.vector_norm(t.reshape(-1).float(), float("inf")) if t.numel() else
-                        torch.zeros((), device=t.device) for t in tensors]).max().item()
-    dt = torch.float16 if amax <= _F16_SAFE_ABS else torch.bfloat16     # (NaN / inf -> bf16)
+                        torch.ones((), device=t.device) for t in tensors]).max().item()
+    fits = _F16_TINY_ABS <= amax <= _F16_SAFE_ABS                        # (NaN / inf -> bf16)
+    dt = torch.float16 if fits else torch.bfloat16
     return tuple(t.to(dt) for t in tensors)
 
 
@@ -186,14 +190,20 @@ def block_sparse_attention_from_index(query, key, value, block_index):
     return c.result()
 
 
-def _build_block_index(query, key, top_k, block_size_M=64, block_size_N=64, force_diag_first=False):
+def _build_block_index(query, key, top_k, block_size_M=64, block_size_N=64, force_diag_first=False,
+                       reference_rounding=None):
     """Top-k key blocks per query block from mean-pooled Q/K
     (block_sparse_flash_attention.py:151-166, including the zero padding its caller applies at
     :178-180).  Pooling, block scores (fp32 matrix cores) and the top-k all run in libminf_hip.so;
     K may have fewer heads than Q.  Returns int32 [batch, heads_q, rows, min(top_k, rows)] with
-    rows = (n + 64 - n % 64) / 64, every row ascending."""
+    rows = (n + 64 - n % 64) / 64, every row ascending.  ``reference_rounding``: None = like the
+    reference (bf16/fp16 inputs: pooled means and pooled products rounded to the input dtype, the
+    dtype its ``mean`` and ``einsum`` return; fp32 inputs: not), False = fp32 arithmetic."""
     if block_size_M != 64 or block_size_N != 64:
         raise ValueError("only 64x64 blocks are supported")
+    from .estimate import reference_rounding_for
+    flags = (_lib.MINF_BS_FORCE_DIAG_FIRST if force_diag_first else 0) | \
+            (_lib.MINF_BS_ROUND_INPUT_DTYPE if reference_rounding_for(query.dtype, reference_rounding) else 0)
     c = _Call(query, key, key, need_out=False)
     lib = _lib.load()
     rows = lib.minf_bs_block_index_rows(c.N)
@@ -207,7 +217,7 @@ def _build_block_index(query, key, top_k, block_size_M=64, block_size_N=64, forc
     ks = (ctypes.c_int64 * 3)(*c.k.stride()[:3])
     with torch.cuda.device(c.q.device):
         st = lib.minf_bs_block_index(c.q.data_ptr(), c.k.data_ptr(), qs, ks, c.B, c.H, c.Hk, c.N,
-                                     c.kernel_dim, c.struct.dtype, int(top_k), int(bool(force_diag_first)),
+                                     c.kernel_dim, c.struct.dtype, int(top_k), flags,
                                      out.data_ptr(), ws.data_ptr(), ws_bytes, _lib.stream_ptr(c.q.device))
     _lib.check(st, "minf_bs_block_index")
     return out

@@ -14,6 +14,7 @@ from __future__ import annotations
 
 import json
 import os
+from collections import OrderedDict
 
 import torch
 
@@ -58,15 +59,91 @@ def _head_plan(config, layer_idx, num_heads):
 VERTICAL_PAD = 0x3FFFFFFF      # a vertical index no range ever reaches: never emitted by the index builder
 
 
+class _LayerPlan:
+    """What a layer's pattern table fixes once and for all: the parsed plan and, per (batch, tokens,
+    device), the small device tensors its launch chains read (head lists, per-head top-k sizes).
+    The reference parses the table and copies ``[context_size]`` to the device on every call of
+    every head (minference_forward.py:621-625, pit_sparse_flash_attention_v2.py:220); here a layer's
+    second call issues no host-to-device copy at all."""
+
+    def __init__(self, config, layer_idx, num_heads):
+        self.pattern = config.get("best_pattern")          # pins the object whose id() is the cache key
+        self.plan = _head_plan(config, layer_idx, num_heads)
+        self.num_heads = num_heads
+        ok = ("vertical_and_slash", "block_sparse", "stream_llm")
+        for (ty, _, _) in self.plan:
+            if ty not in ok:
+                raise KeyError(ty)
+        self.vs = sorted((h, v, s) for (ty, v, s), hs in self.plan.items() if ty == "vertical_and_slash" for h in hs)
+        self.bs = sorted(h for (ty, _, _), hs in self.plan.items() if ty == "block_sparse" for h in hs)
+        self.stream = {}
+        for (ty, v, s), hs in self.plan.items():
+            if ty == "stream_llm":
+                self.stream.setdefault((v, s), []).extend(hs)
+        covered = len(self.vs) + len(self.bs) + sum(len(hs) for hs in self.stream.values())
+        if covered != num_heads:
+            # the shared output buffer is torch.empty: a head without a launch would return garbage
+            raise ValueError(f"pattern table covers {covered} of {num_heads} heads")
+        self._dev = {}
+
+    def device_tensors(self, B, N, dev):
+        """-> dict of int32 device tensors for this (batch, tokens, device), built on first use."""
+        key = (B, N, str(dev))
+        d = self._dev.get(key)
+        if d is None:
+            d = {}
+            if self.vs:
+                # sizes clamped like the reference (:600)
+                kv = [min(N, max(int(v), 30)) for _, v, _ in self.vs]
+                ksl = [min(N, max(int(s), 50)) for _, _, s in self.vs]
+                d["vs_heads"] = _head_list([h for h, _, _ in self.vs], dev)
+                d["vs_kv"] = torch.tensor(kv * B, dtype=torch.int32).to(dev)
+                d["vs_ks"] = torch.tensor(ksl * B, dtype=torch.int32).to(dev)
+                d["vs_max"] = (max(kv), max(ksl))
+            if self.bs:
+                d["bs_heads"] = _head_list(self.bs, dev)
+            d["stream_heads"] = {key2: _head_list(hs, dev) for key2, hs in self.stream.items()}
+            if len(self._dev) >= 8:                        # a few prompt lengths per layer at most
+                self._dev.pop(next(iter(self._dev)))
+            self._dev[key] = d
+        return d
+
+
+_PLAN_CACHE = OrderedDict()
+_PLAN_CACHE_MAX = 512          # layers x tables held; the least recently used entry goes first
+
+
+def _layer_plan(config, layer_idx, num_heads):
+    """The cached _LayerPlan of (pattern table object, layer, head count, ratio)."""
+    best = config.get("best_pattern")
+    key = (id(best), layer_idx, num_heads, config.get("minference_ratio") if "minference_ratio" in config else None)
+    lp = _PLAN_CACHE.get(key)
+    if lp is not None and lp.pattern is best:
+        _PLAN_CACHE.move_to_end(key)
+        return lp
+    lp = _LayerPlan(config, layer_idx, num_heads)
+    _PLAN_CACHE[key] = lp
+    while len(_PLAN_CACHE) > _PLAN_CACHE_MAX:
+        _PLAN_CACHE.popitem(last=False)
+    return lp
+
+
+def clear_plan_cache():
+    """Forget every cached layer plan.  A pattern table is treated as immutable once a layer has
+    used it; call this after editing a ``best_pattern`` list in place."""
+    _PLAN_CACHE.clear()
+
+
 def _head_list(heads, device):
     """int32 device tensor of the (ascending) query head numbers of one pattern group."""
     return torch.tensor(sorted(heads), dtype=torch.int32).to(device)
 
 
-def _mixed_layer(query_states, key_states, value_states, plan):
-    """All heads of a layer whose pattern table mixes types and sizes: q/k/v are prepared once, the
-    output is one shared buffer, and every pattern type is ONE launch chain over the original
-    tensors with a head selection -- no gathered copies of Q, no scattered writes of O:
+def _mixed_layer(query_states, key_states, value_states, lp):
+    """All heads of a layer whose pattern table mixes types and sizes (``lp``: its _LayerPlan): q/k/v
+    are prepared once, the output is one shared buffer, and every pattern type is ONE launch chain
+    over the original tensors with a head selection -- no gathered copies of Q, no scattered writes
+    of O:
 
     * vertical_and_slash heads with any mix of (vertical_size, slash_size): one estimation over those
       heads, one ragged top-k (every head keeps its own sizes; shorter lists are padded with entries
@@ -76,10 +153,10 @@ def _mixed_layer(query_states, key_states, value_states, plan):
 
     The reference runs one operator call per head here (minference_forward.py:657-667)."""
     from . import _lib
-    from .estimate import FORCE_SLASH, FORCE_VERTICAL, LAST_Q
+    from .estimate import FORCE_SLASH, FORCE_VERTICAL, LAST_Q, reference_rounding_for
     from .ops import _Call
-    import ctypes
     B, H, N, D = query_states.shape
+    rounded = reference_rounding_for(query_states.dtype)     # the reference's rounding points on 16-bit inputs
     dev = query_states.device
     c = _Call(query_states, key_states, value_states)
     lib = _lib.load()
@@ -88,76 +165,64 @@ def _mixed_layer(query_states, key_states, value_states, plan):
     qs, ks = i64x3(*c.q.stride()[:3]), i64x3(*c.k.stride()[:3])
     rows = (N + 63) // 64
     keep = []                                             # tensors the enqueued kernels still read
+    dt = lp.device_tensors(B, N, dev)
 
-    vs = [(h, v, s) for (ty, v, s), hs in plan.items() if ty == "vertical_and_slash" for h in hs]
-    bs = sorted(h for (ty, _, _), hs in plan.items() if ty == "block_sparse" for h in hs)
-    st_groups = {}
-    for (ty, v, s), hs in plan.items():
-        if ty == "stream_llm":
-            st_groups.setdefault((v, s), []).extend(hs)
-        elif ty not in ("vertical_and_slash", "block_sparse"):
-            raise KeyError(ty)
-
-    with torch.cuda.device(dev):
-        if vs:
-            vs.sort()
-            heads = [h for h, _, _ in vs]
-            nh = len(heads)
-            # sizes clamped like the reference (:600)
-            kv = [min(N, max(int(v), 30)) for _, v, _ in vs]
-            ksl = [min(N, max(int(s), 50)) for _, _, s in vs]
-            vmax, smax = max(kv), max(ksl)
-            slot = _head_list(heads, dev)
-            vertical = torch.empty((B, nh, N), dtype=torch.float32, device=dev)
-            slash = torch.empty((B, nh, N), dtype=torch.float32, device=dev)
-            ws_bytes = lib.minf_vs_estimate_workspace_bytes(B, nh, N)
-            ws = torch.empty((ws_bytes + 15) // 16 * 16, dtype=torch.uint8, device=dev)
-            st = lib.minf_vs_estimate_heads(c.q.data_ptr(), c.k.data_ptr(), qs, ks, B, H, c.Hk, N, c.kernel_dim,
-                                            c.struct.dtype, float(D) ** -0.5, LAST_Q, FORCE_VERTICAL, FORCE_SLASH,
-                                            slot.data_ptr(), nh, vertical.data_ptr(), slash.data_ptr(),
-                                            ws.data_ptr(), ws_bytes, stream)
-            _lib.check(st, "minf_vs_estimate_heads")
-            kv_t = torch.tensor(kv * B, dtype=torch.int32).to(dev)
-            ks_t = torch.tensor(ksl * B, dtype=torch.int32).to(dev)
-            v_idx = torch.empty((B, nh, vmax), dtype=torch.int32, device=dev)
-            s_idx = torch.empty((B, nh, smax), dtype=torch.int32, device=dev)
-            st = lib.minf_topk_indices_pair_ragged(vertical.data_ptr(), kv_t.data_ptr(), vmax, v_idx.data_ptr(), vmax, -1, 1, VERTICAL_PAD,
-                                                   slash.data_ptr(), ks_t.data_ptr(), smax, s_idx.data_ptr(), smax, N - 1, 2, 0,
-                                                   B * nh, N, N, stream)
-            _lib.check(st, "minf_topk_indices_pair_ragged")
-            seqlens = torch.full((B,), N, dtype=torch.int32, device=dev)
-            bc, bo, cc, ci = convert_vertical_slash_indexes(seqlens, v_idx, s_idx, N, 64, 64, zero_fill=False)
-            c.struct.seqlens = seqlens.data_ptr()
-            c.select_heads(slot)
-            st = lib.minf_vs_attn_fwd(c.ref, bc.data_ptr(), bo.data_ptr(), cc.data_ptr(), ci.data_ptr(), rows,
-                                      smax, vmax, stream)
-            _lib.check(st, "minf_vs_attn_fwd")
-            c.struct.seqlens = None
-            keep += [slot, vertical, slash, ws, kv_t, ks_t, v_idx, s_idx, seqlens, bc, bo, cc, ci]
-        if bs:
-            nh = len(bs)
-            slot = _head_list(bs, dev)
-            brows = lib.minf_bs_block_index_rows(N)
-            kk = min(100, brows)                          # top_k fixed at 100 (:616-618)
-            ws_bytes = lib.minf_bs_block_index_workspace_bytes(B, nh, c.Hk, N)
-            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
-            bi = torch.empty((B, nh, brows, kk), dtype=torch.int32, device=dev)
-            st = lib.minf_bs_block_index_heads(c.q.data_ptr(), c.k.data_ptr(), qs, ks, B, H, c.Hk, N, c.kernel_dim,
-                                               c.struct.dtype, 100, 0, slot.data_ptr(), nh, bi.data_ptr(),
-                                               ws.data_ptr(), ws_bytes, stream)
-            _lib.check(st, "minf_bs_block_index_heads")
-            c.select_heads(slot)
-            st = lib.minf_bs_attn_fwd(c.ref, bi.data_ptr(), brows, kk, stream)
-            _lib.check(st, "minf_bs_attn_fwd")
-            keep += [slot, ws, bi]
-        for (n_init, n_local), hs in st_groups.items():
-            slot = _head_list(hs, dev)
-            c.select_heads(slot)
-            if N > 0:
-                st = lib.minf_ashape_attn_fwd(c.ref, int(n_init), int(n_local), stream)
-                _lib.check(st, "minf_ashape_attn_fwd")
-            keep.append(slot)
-    c.select_heads(None)
+    try:
+        with torch.cuda.device(dev):
+            if lp.vs:
+                nh = len(lp.vs)
+                vmax, smax = dt["vs_max"]
+                slot, kv_t, ks_t = dt["vs_heads"], dt["vs_kv"], dt["vs_ks"]
+                vertical = torch.empty((B, nh, N), dtype=torch.float32, device=dev)
+                slash = torch.empty((B, nh, N), dtype=torch.float32, device=dev)
+                ws_bytes = lib.minf_vs_estimate_workspace_bytes(B, nh, N)
+                ws = torch.empty((ws_bytes + 15) // 16 * 16, dtype=torch.uint8, device=dev)
+                st = lib.minf_vs_estimate_heads(c.q.data_ptr(), c.k.data_ptr(), qs, ks, B, H, c.Hk, N, c.kernel_dim,
+                                                c.struct.dtype, float(D) ** -0.5, LAST_Q, FORCE_VERTICAL, FORCE_SLASH,
+                                                _lib.MINF_ROUND_INPUT_DTYPE if rounded else _lib.MINF_ROUND_NONE,
+                                                slot.data_ptr(), nh, vertical.data_ptr(), slash.data_ptr(),
+                                                ws.data_ptr(), ws_bytes, stream)
+                _lib.check(st, "minf_vs_estimate_heads")
+                v_idx = torch.empty((B, nh, vmax), dtype=torch.int32, device=dev)
+                s_idx = torch.empty((B, nh, smax), dtype=torch.int32, device=dev)
+                st = lib.minf_topk_indices_pair_ragged(vertical.data_ptr(), kv_t.data_ptr(), vmax, v_idx.data_ptr(), vmax, -1, 1, VERTICAL_PAD,
+                                                       slash.data_ptr(), ks_t.data_ptr(), smax, s_idx.data_ptr(), smax, N - 1, 2, 0,
+                                                       B * nh, N, N, stream)
+                _lib.check(st, "minf_topk_indices_pair_ragged")
+                seqlens = torch.full((B,), N, dtype=torch.int32, device=dev)
+                bc, bo, cc, ci = convert_vertical_slash_indexes(seqlens, v_idx, s_idx, N, 64, 64, zero_fill=False)
+                c.struct.seqlens = seqlens.data_ptr()
+                c.select_heads(slot)
+                st = lib.minf_vs_attn_fwd(c.ref, bc.data_ptr(), bo.data_ptr(), cc.data_ptr(), ci.data_ptr(), rows,
+                                          smax, vmax, stream)
+                c.struct.seqlens = None
+                _lib.check(st, "minf_vs_attn_fwd")
+                keep += [vertical, slash, ws, v_idx, s_idx, seqlens, bc, bo, cc, ci]
+            if lp.bs:
+                nh = len(lp.bs)
+                slot = dt["bs_heads"]
+                brows = lib.minf_bs_block_index_rows(N)
+                kk = min(100, brows)                          # top_k fixed at 100 (:616-618)
+                ws_bytes = lib.minf_bs_block_index_workspace_bytes(B, nh, c.Hk, N)
+                ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+                bi = torch.empty((B, nh, brows, kk), dtype=torch.int32, device=dev)
+                st = lib.minf_bs_block_index_heads(c.q.data_ptr(), c.k.data_ptr(), qs, ks, B, H, c.Hk, N, c.kernel_dim,
+                                                   c.struct.dtype, 100, _lib.MINF_BS_ROUND_INPUT_DTYPE if rounded else 0,
+                                                   slot.data_ptr(), nh, bi.data_ptr(),
+                                                   ws.data_ptr(), ws_bytes, stream)
+                _lib.check(st, "minf_bs_block_index_heads")
+                c.select_heads(slot)
+                st = lib.minf_bs_attn_fwd(c.ref, bi.data_ptr(), brows, kk, stream)
+                _lib.check(st, "minf_bs_attn_fwd")
+                keep += [ws, bi]
+            for (n_init, n_local), slot in dt["stream_heads"].items():
+                c.select_heads(slot)
+                if N > 0:
+                    st = lib.minf_ashape_attn_fwd(c.ref, int(n_init), int(n_local), stream)
+                    _lib.check(st, "minf_ashape_attn_fwd")
+    finally:
+        c.struct.seqlens = None
+        c.select_heads(None)
     out = c.result()
     # torch's caching allocator hands a freed block only to work enqueued later on the same stream, so
     # dropping `keep` here is safe for kernels that are still running
@@ -213,11 +278,11 @@ def minference_prefill_forward(query_states, key_states, value_states, prefill_k
         return _search_layer(query_states, key_states, value_states, prefill_kwargs)
     if layer_idx < starting_layer:
         return dense_causal_attention(query_states, key_states, value_states)
-    plan = _head_plan(config, layer_idx, H)
-    if len(plan) == 1:
-        (ty, vs, ss), _ = next(iter(plan.items()))
+    lp = _layer_plan(config, layer_idx, H)
+    if len(lp.plan) == 1:
+        (ty, vs, ss), _ = next(iter(lp.plan.items()))
         return minference_prefill_kernel(query_states, key_states, value_states, ty, vs, ss)
-    return _mixed_layer(query_states, key_states, value_states, plan)
+    return _mixed_layer(query_states, key_states, value_states, lp)
 
 
 def a_shape_kernel(query_states, key_states, value_states, prefill_kwargs):

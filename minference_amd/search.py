@@ -93,7 +93,7 @@ def pattern_recall(q, k, candidates=CANDIDATES, row_begin=ROW_BEGIN):
                            "minf_flags_set_range")
             elif ty == "vertical_and_slash":
                 if scores is None:
-                    scores = vertical_slash_scores(q, k, 64, SEARCH_FORCE, SEARCH_FORCE)
+                    scores = vertical_slash_scores(q, k, 64, SEARCH_FORCE, SEARCH_FORCE, reference_rounding=False)
                 v_idx = topk_indices(scores[0], min(a, N))
                 s_idx = topk_indices(scores[1], min(b, N), reverse_base=N - 1)
                 for idx, flags in ((v_idx, col), (s_idx, diag)):

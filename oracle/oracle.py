@@ -15,8 +15,11 @@ Every function cites the reference lines it restates.  Parity status:
 * ``ashape_mask``         pinned (closed form vs per-element loop, n_local>=N -> causal SDPA)
 * ``search_candidate_mask`` / ``search_pattern_scores``  pinned (Q=0 closed forms counted by
   explicit loops, all-kept candidates -> 1, brute force on tiny inputs)
-* ``torch.topk`` tie order and Triton's bf16 rounding points are implementation
-  defined in the reference (not in its source): "parity unpinned" for those;
+* ``estimate_scores(reference_rounding=True)`` / ``bs_block_scores(reference_rounding=True)``: the
+  rounding points of the reference's torch code on 16-bit inputs; pinned by per-element loops that
+  round with ``.to(dtype)`` at exactly those points (tests/test_oracle_rounding.py)
+* ``torch.topk`` tie order and Triton's bf16 rounding points inside the attention kernels are
+  implementation defined in the reference (not in its source): "parity unpinned" for those;
   tests compare top-k *sets* away from ties and outputs within tolerance.
 """
 from __future__ import annotations
@@ -141,15 +144,24 @@ def sum_all_diagonal(p: torch.Tensor) -> torch.Tensor:
     return strided.sum(0)[1:]
 
 
-def estimate_scores(q: torch.Tensor, k: torch.Tensor, last_q: int = 64):
+def estimate_scores(q: torch.Tensor, k: torch.Tensor, last_q: int = 64, reference_rounding: bool = False):
     """Score vectors before forcing.  q,k [B,H,N,D] (same H) on CPU.
     Returns (vertical [B,H,N], slash [B,H,N]) fp32 where slash[..., j] is the
     probability mass on the diagonal with offset N-1-j
-    (minference_forward.py:601-609; arithmetic done in fp32 throughout)."""
+    (minference_forward.py:601-609).
+
+    Default: fp32 arithmetic throughout.  ``reference_rounding=True`` rounds where the reference's
+    torch code rounds for 16-bit inputs: the einsum result (fp32 accumulation, one rounding to the
+    input dtype, :602), then the division by sqrt(D) in the input dtype (:602); the softmax and
+    both sums run in fp32 (``dtype=torch.float32``, :604).  For fp32 inputs the two modes agree."""
     B, H, N, D = q.shape
     lq = min(last_q, N)
     qf, kf = q.float(), k.float()
-    qk = torch.einsum("bhmk,bhnk->bhmn", qf[:, :, -lq:, :], kf) / math.sqrt(D)
+    qk = torch.einsum("bhmk,bhnk->bhmn", qf[:, :, -lq:, :], kf)
+    if reference_rounding and q.dtype != torch.float32:
+        qk = (qk.to(q.dtype) / math.sqrt(D)).float()       # tensor / python scalar: fp32 quotient, rounded to q.dtype
+    else:
+        qk = qk / math.sqrt(D)
     ar = torch.arange(lq)
     corner = ar[:, None] >= ar[None, :]
     qk[:, :, :, -lq:] = torch.where(corner, qk[:, :, :, -lq:], torch.tensor(-torch.inf))
@@ -172,14 +184,15 @@ def topk_lowest_index(x: torch.Tensor, k: int) -> torch.Tensor:
     return order.sort(dim=-1).values
 
 
-def estimate_vs(q, k, vertical_size, slash_size, last_q=64, force_vertical=30, force_slash=100):
+def estimate_vs(q, k, vertical_size, slash_size, last_q=64, force_vertical=30, force_slash=100,
+                reference_rounding=False):
     """minference_forward.py:599-612: returns (v_idx [B,H,v] ascending key
     positions, s_idx [B,H,s] descending diagonal offsets, vertical scores,
     slash scores) -- scores after forcing (+inf)."""
     N = q.shape[2]
     v = min(N, max(vertical_size, 30))
     s = min(N, max(slash_size, 50))
-    vertical, slash = estimate_scores(q, k, last_q)
+    vertical, slash = estimate_scores(q, k, last_q, reference_rounding)
     vertical = vertical.clone(); slash = slash.clone()
     vertical[..., :force_vertical] = torch.inf
     slash[..., -force_slash:] = torch.inf
@@ -234,18 +247,36 @@ def vs_mask_rows(block_count_m, block_offset_m, column_count_m, column_index_m, 
     return mask
 
 
-def bs_block_index(q: torch.Tensor, k: torch.Tensor, top_k: int, force_diag_first: bool = False):
-    """block_sparse_flash_attention.py:151-166 on tensors already padded to a
-    multiple of 64 (the caller pads, :178-180).  fp32 arithmetic; ties -> lowest
-    block id.  force_diag_first adds the benchmark rule "always keep the
-    diagonal block and block 0" before the sort."""
+def bs_block_scores(q: torch.Tensor, k: torch.Tensor, reference_rounding: bool = False):
+    """Pooled block scores [B,H,R,R] (fp32 values) of block_sparse_flash_attention.py:159-164 on
+    tensors already padded to a multiple of 64; non-causal pairs are -inf.  Default: fp32
+    arithmetic.  ``reference_rounding=True`` rounds where the reference's torch code rounds for
+    16-bit inputs: each 64-token mean (fp32 accumulation, rounded to the input dtype, :159-160)
+    and each pooled dot product (fp32 accumulation, rounded to the input dtype, :163)."""
     B, H, N, D = q.shape
     qp = q.float().reshape(B, H, -1, 64, D).mean(-2)
     kp = k.float().reshape(B, H, -1, 64, D).mean(-2)
+    rr = reference_rounding and q.dtype != torch.float32
+    if rr:
+        qp, kp = qp.to(q.dtype).float(), kp.to(q.dtype).float()
     R = qp.shape[2]
     p = torch.einsum("bhmk,bhnk->bhmn", qp, kp)
+    if rr:
+        p = p.to(q.dtype).float()
     ar = torch.arange(R)
-    p = torch.where(ar[:, None] >= ar[None, :], p, torch.tensor(-torch.inf))
+    return torch.where(ar[:, None] >= ar[None, :], p, torch.tensor(-torch.inf))
+
+
+def bs_block_index(q: torch.Tensor, k: torch.Tensor, top_k: int, force_diag_first: bool = False,
+                   reference_rounding: bool = False):
+    """block_sparse_flash_attention.py:151-166 on tensors already padded to a
+    multiple of 64 (the caller pads, :178-180).  fp32 arithmetic unless
+    ``reference_rounding`` (see bs_block_scores); ties -> lowest
+    block id.  force_diag_first adds the benchmark rule "always keep the
+    diagonal block and block 0" before the sort."""
+    p = bs_block_scores(q, k, reference_rounding)
+    R = p.shape[-1]
+    ar = torch.arange(R)
     if force_diag_first:
         p[..., ar, ar] = torch.inf
         p[..., :, 0] = torch.inf

@@ -200,7 +200,7 @@ int main() {
     const size_t est_bytes = minf_vs_estimate_workspace_bytes(B, HQ, N);
     void *dest;
     CHECK_HIP(hipMalloc(&dest, est_bytes));
-    CHECK_MINF(minf_vs_estimate(dq, dk, qs, ks, B, HQ, HK, N, D, MINF_BF16, t.sm_scale, 64, 30, 100, dvert, dslash, dest, est_bytes, stream));
+    CHECK_MINF(minf_vs_estimate(dq, dk, qs, ks, B, HQ, HK, N, D, MINF_BF16, t.sm_scale, 64, 30, 100, MINF_ROUND_INPUT_DTYPE, dvert, dslash, dest, est_bytes, stream));
     CHECK_MINF(minf_topk_indices(dvert, HQ, N, N, 40, dtop, 40, -1, stream));
     CHECK_HIP(hipStreamSynchronize(stream));
     std::vector<int32_t> top((size_t)HQ * 40);

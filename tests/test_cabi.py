@@ -75,10 +75,12 @@ def test_argument_validation_of_the_index_estimate_and_search_entry_points(lib):
     bad = (_lib.c_i64 * 3)(128 * 64 * 4, 128 * 64, 100)
     P = 4096                                                     # any 16-byte aligned non-null address; never dereferenced
     # estimate: workspace too small / misaligned strides / last_q out of range
-    assert lib.minf_vs_estimate(P, P, i3, i3, 1, 4, 4, 64, 128, 0, 0.1, 64, 30, 100, P, P, P, 16, None) == -4
-    assert lib.minf_vs_estimate(P, P, bad, i3, 1, 4, 4, 64, 128, 0, 0.1, 64, 30, 100, P, P, P, 1 << 30, None) == -3
-    assert lib.minf_vs_estimate(P, P, i3, i3, 1, 4, 4, 64, 128, 0, 0.1, 65, 30, 100, P, P, P, 1 << 30, None) == -1
-    assert lib.minf_vs_estimate(P, P, i3, i3, 1, 4, 4, 64, 96, 0, 0.1, 64, 30, 100, P, P, P, 1 << 30, None) == -2
+    assert lib.minf_vs_estimate(P, P, i3, i3, 1, 4, 4, 64, 128, 0, 0.1, 64, 30, 100, 0, P, P, P, 16, None) == -4
+    assert lib.minf_vs_estimate(P, P, bad, i3, 1, 4, 4, 64, 128, 0, 0.1, 64, 30, 100, 0, P, P, P, 1 << 30, None) == -3
+    assert lib.minf_vs_estimate(P, P, i3, i3, 1, 4, 4, 64, 128, 0, 0.1, 65, 30, 100, 0, P, P, P, 1 << 30, None) == -1
+    assert lib.minf_vs_estimate(P, P, i3, i3, 1, 4, 4, 64, 96, 0, 0.1, 64, 30, 100, 1, P, P, P, 1 << 30, None) == -2
+    assert lib.minf_vs_estimate(P, P, i3, i3, 1, 4, 4, 64, 128, 0, 0.1, 64, 30, 100, 7, P, P, P, 1 << 30, None) == -1   # no such rounding mode
+    assert lib.minf_bs_block_index(P, P, i3, i3, 1, 4, 4, 64, 128, 0, 10, 4, P, P, 1 << 30, None) == -1      # unknown flag bit
     # block index: head counts, head_dim, workspace
     assert lib.minf_bs_block_index(P, P, i3, i3, 1, 4, 3, 64, 128, 0, 10, 0, P, P, 1 << 30, None) == -1
     assert lib.minf_bs_block_index(P, P, i3, i3, 1, 4, 4, 64, 256, 0, 10, 0, P, P, 1 << 30, None) == -2

@@ -342,7 +342,7 @@ def test_golden_fixtures(gpu):
     check(M.block_sparse_attention(q, k, v, 2), torch.from_numpy(z["bs_out"]), "golden-bs")
 
 
-def _check_block_index(bi_gpu, p, top_k):
+def _check_block_index(bi_gpu, p, top_k, rel_tol=1e-5, min_exact=0.98):
     """bi_gpu [H, R, K] against oracle block scores p [H, R, R] (fp32): ascending unique rows, and
     the same selection as the oracle's rule up to near-ties of the fp32 scores (the GPU sums in a
     different order): everything clearly above the k-th score is selected, nothing clearly below."""
@@ -360,14 +360,14 @@ def _check_block_index(bi_gpu, p, top_k):
                 exact += 1
                 continue
             kth = p[h, m, order[h, m, K - 1]]
-            tol = 1e-5 * max(1.0, abs(kth)) if np.isfinite(kth) else 0.0
+            tol = rel_tol * max(1.0, abs(kth)) if np.isfinite(kth) else 0.0
             sel = np.zeros(R, bool); sel[row] = True
             if np.isfinite(kth):
                 assert sel[p[h, m] > kth + tol].all(), (h, m)
                 assert (p[h, m][sel] >= kth - tol).all(), (h, m)
             else:                                   # fewer finite scores than k: all finite ones are in
                 assert sel[np.isfinite(p[h, m]) | (p[h, m] == np.inf)].all(), (h, m)
-    assert exact >= 0.98 * H * R, f"only {exact}/{H * R} rows identical to the oracle"
+    assert exact >= min_exact * H * R, f"only {exact}/{H * R} rows identical to the oracle"
 
 
 def _oracle_block_scores(q, k, hq, force):
@@ -404,11 +404,25 @@ def test_block_index_kernel_vs_oracle(gpu, n, top_k, hq, hk, force, dtype, d):
     from minference_amd.ops import _build_block_index
     print(f"case block-index n={n} top_k={top_k} hq={hq} hk={hk} force={force} d={d}", flush=True)
     q, k, _ = make(1, hq, hk, n, 40, dtype, d=d)
-    bi = _build_block_index(q.to(gpu), k.to(gpu), top_k, force_diag_first=force)
+    bi = _build_block_index(q.to(gpu), k.to(gpu), top_k, force_diag_first=force, reference_rounding=False)
     R = (n + 64 - (n & 63)) // 64
     assert tuple(bi.shape) == (1, hq, R, min(top_k, R)) and bi.dtype == torch.int32
     p = _oracle_block_scores(q, k, hq, force)
     _check_block_index(bi[0].cpu().numpy(), p, top_k)
+    # the default mode for 16-bit inputs rounds the pooled means and products to the input dtype like
+    # the reference's torch code (block_sparse_flash_attention.py:159-163); against the oracle's rounded
+    # scores.  A product within an fp32 rounding error of a 16-bit boundary may round the other way
+    # (the matrix cores add in another order), so near the k-th score one unit of the format is allowed.
+    bi_r = _build_block_index(q.to(gpu), k.to(gpu), top_k, force_diag_first=force)
+    pad_r = 64 - (n & 63)
+    pr = O.bs_block_scores(torch.nn.functional.pad(q, [0, 0, 0, pad_r]),
+                           torch.nn.functional.pad(expand(k, hq), [0, 0, 0, pad_r]), reference_rounding=True)[0].double().numpy()
+    if force:
+        ar = np.arange(R)
+        pr[:, ar, ar] = np.inf
+        pr[:, :, 0] = np.inf
+    _check_block_index(bi_r[0].cpu().numpy(), pr, top_k, rel_tol=2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10,
+                       min_exact=0.9)
     # and the oracle's own index builder agrees with the score matrix used above
     pad = 64 - (n & 63)
     ob = O.bs_block_index(torch.nn.functional.pad(q, [0, 0, 0, pad]),

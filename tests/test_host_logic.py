@@ -143,3 +143,23 @@ def test_reference_patch_function_names():
     assert patch_hf(sentinel, "hf", {"n_init": 1}, n_local=2) is sentinel
     with pytest.raises(NotImplementedError):
         patch_hf(sentinel, "inf_llm")
+
+
+def test_layer_plan_is_cached_per_table_object_and_checks_head_coverage():
+    """The dispatcher parses a layer's table once (minference_forward.py:621-625 does it per call)."""
+    layer = {"0": ["vertical_and_slash", 100, 200, 0.9], "1": ["block_sparse", 100, 6096, 0.9],
+             "2": ["stream_llm", 128, 512, 0.9]}
+    config = cfg([layer])
+    prefill.clear_plan_cache()
+    a = prefill._layer_plan(config, 0, 3)
+    assert prefill._layer_plan(config, 0, 3) is a
+    assert [h for h, _, _ in a.vs] == [0] and a.bs == [1] and a.stream == {(128, 512): [2]}
+    # an equal table in another object is another entry; a ratio is part of the key
+    assert prefill._layer_plan(cfg([dict(layer)]), 0, 3) is not a
+    assert prefill._layer_plan(dict(config, minference_ratio=0.5), 0, 3) is not a
+    # heads without an entry take the default pattern, so 5 heads are covered as well
+    assert len(prefill._layer_plan(config, 0, 5).vs) == 3
+    with pytest.raises(KeyError):
+        prefill._layer_plan(cfg([{"0": ["no_such_pattern", 1, 1, 0.5]}]), 0, 1)
+    prefill.clear_plan_cache()
+    assert prefill._layer_plan(config, 0, 3) is not a
