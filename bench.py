@@ -94,66 +94,110 @@ def _time_steps(torch, f, steps, warmup):
     return a.elapsed_time(b) / steps
 
 
-def bench_index_c3(args, torch, gen, M, dev):
+def measure_index_c3(torch, gen, M, dev, steps, warmup, lengths=(262144, 524288)):
     """BASELINE config 3: the vertical_slash_index builder alone, 32 heads, 1000 verticals, 6096
-    slashes drawn uniformly, full zero-filled tensors (the reference's output contract)."""
+    slashes drawn uniformly, full zero-filled tensors (the reference's output contract).
+    -> {n: {"ms", "bytes", "gbs", "frac_of_hbm_peak"}}; bytes = every element of the four outputs."""
     import numpy as np
     out = {}
-    for n in (262144, 524288):
+    for n in lengths:
         vi, si = gen.vs_index_inputs(32, n, 1000, 6096, seed=300)
         seqlens = torch.tensor([n], dtype=torch.int32, device=dev)
         vi_t, si_t = torch.from_numpy(vi).to(dev), torch.from_numpy(np.ascontiguousarray(si)).to(dev)
-        ms = _time_steps(torch, lambda: M.convert_vertical_slash_indexes(seqlens, vi_t, si_t, n), args.steps, args.warmup)
+        ms = _time_steps(torch, lambda: M.convert_vertical_slash_indexes(seqlens, vi_t, si_t, n), steps, warmup)
         rows = n // 64
         full = 4 * 32 * rows * (6096 + 1000 + 2)
-        out[n] = (ms, full)
+        gbs = full / (ms * 1e-3) / 1e9
+        out[n] = {"ms": round(ms, 3), "bytes": full, "gbs": round(gbs, 1), "frac_of_hbm_peak": round(gbs / PEAK_HBM_GBS, 4)}
         torch.cuda.empty_cache()
-    ms, full = out[524288]
-    gbs = full / (ms * 1e-3) / 1e9
+    return out
+
+
+def bench_index_c3(args, torch, gen, M, dev):
+    out = measure_index_c3(torch, gen, M, dev, args.steps, args.warmup)
+    r = out[524288]
     print(json.dumps({
-        "metric": "vertical_slash_index build, ms (BASELINE config 3, seq 524288)", "value": round(ms, 3),
-        "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 3),
+        "metric": "vertical_slash_index build, ms (BASELINE config 3, seq 524288)", "value": r["ms"],
+        "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": r["ms"],
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "int32", "data": "synthetic",
         "config": {"workload": "BASELINE config 3: index builder alone, 32 heads, 1000 verticals, 6096 slashes, "
                                "full zero-filled outputs", "seq_len": 524288},
-        "ms_at_262144": round(out[262144][0], 3),
+        "ms_at_262144": out[262144]["ms"],
         "roofline": {"kernel": "vs_index_prep_kernel + vs_index_fast_kernel", "bound": "hbm",
-                     "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None, "bytes_per_launch": full}}))
+                     "achieved": r["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": r["frac_of_hbm_peak"], "traffic": None, "bytes_per_launch": r["bytes"]}}))
+
+
+def measure_block_sparse_c4(torch, M, q, k, v, steps, warmup):
+    """BASELINE config 4: top-100 block-sparse attention (diagonal and block 0 always kept) on
+    resident q/k/v [1, 32, n, 128] / [1, 8, n, 128]."""
+    from minference_amd.ops import _build_block_index, block_sparse_attention_from_index
+    n = q.shape[2]
+    ms_idx = _time_steps(torch, lambda: _build_block_index(q, k, 100, force_diag_first=True), steps, warmup)
+    bi = _build_block_index(q, k, 100, force_diag_first=True)
+    ms_att = _time_steps(torch, lambda: block_sparse_attention_from_index(q, k, v, bi), steps, warmup)
+    tiles = q.shape[1] * sum(min(m + 1, 100) for m in range((n + 63) // 64))
+    tf = tiles * TILE_FLOP / (ms_att * 1e-3) / 1e12
+    return {"block_index_ms": round(ms_idx, 3), "attention_ms": round(ms_att, 3), "computed_tiles": tiles,
+            "tflops": round(tf, 1), "frac_of_bf16_peak": round(tf / PEAK_BF16_TFLOPS, 4)}
 
 
 def bench_block_sparse_c4(args, torch, gen, M, dev):
-    """BASELINE config 4: top-100 block-sparse attention (diagonal and block 0 always kept) on the
-    config 2 inputs, 131072 tokens, 32 q / 8 kv heads."""
-    from minference_amd.ops import _build_block_index, block_sparse_attention_from_index
     n = args.seq
     q, k, v, _ = gen.planted_layer(n, 32, 8, seed=100, dtype=torch.bfloat16)
     q, k, v = q.to(dev), k.to(dev), v.to(dev)
-    ms_idx = _time_steps(torch, lambda: _build_block_index(q, k, 100, force_diag_first=True), args.steps, args.warmup)
-    bi = _build_block_index(q, k, 100, force_diag_first=True)
-    ms_att = _time_steps(torch, lambda: block_sparse_attention_from_index(q, k, v, bi), args.steps, args.warmup)
-    tiles = 32 * sum(min(m + 1, 100) for m in range((n + 63) // 64))
-    tf = tiles * TILE_FLOP / (ms_att * 1e-3) / 1e12
+    r = measure_block_sparse_c4(torch, M, q, k, v, args.steps, args.warmup)
+    total = r["block_index_ms"] + r["attention_ms"]
     print(json.dumps({
-        "metric": "block-sparse prefill attn ms/layer @128K (BASELINE config 4)", "value": round(ms_idx + ms_att, 3),
+        "metric": "block-sparse prefill attn ms/layer @128K (BASELINE config 4)", "value": round(total, 3),
         "unit": "ms/layer", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_idx + ms_att, 3), "higher_is_better": False, "scaling": "weak",
+        "ms_per_step": round(total, 3), "higher_is_better": False, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "BASELINE config 4: block-sparse top-100 (diagonal and first block kept), "
                                "32 q / 8 kv heads, planted inputs of config 2", "seq_len": n},
-        "stage_ms": {"block_index": round(ms_idx, 3), "attention": round(ms_att, 3)}, "computed_tiles": tiles,
-        "roofline": {"kernel": "attn_fwd_kernel<bf16, block-sparse>", "bound": "mfma", "achieved": round(tf, 1),
-                     "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / PEAK_BF16_TFLOPS, 4),
-                     "traffic": None, "launch_ms": round(ms_att, 3), "flop_per_launch": tiles * TILE_FLOP}}))
+        "stage_ms": {"block_index": r["block_index_ms"], "attention": r["attention_ms"]}, "computed_tiles": r["computed_tiles"],
+        "roofline": {"kernel": "attn_fwd_kernel<bf16, block-sparse>", "bound": "mfma", "achieved": r["tflops"],
+                     "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": r["frac_of_bf16_peak"],
+                     "traffic": None, "launch_ms": r["attention_ms"], "flop_per_launch": r["computed_tiles"] * TILE_FLOP}}))
 
 
-def bench_llama_c5(args, torch, dev):
+def ashape_tiles(n, n_init, n_local):
+    """64 x 64 tiles one head visits: per row block the window tiles plus the sink tiles left of them."""
+    sink = (n_init + 63) // 64
+    t = 0
+    for m in range((n + 63) // 64):
+        lo = m * 64 - n_local + 1
+        t_lo = lo // 64 if lo > 0 else 0
+        t += (m - t_lo + 1) + min(sink, t_lo)
+    return t
+
+
+def measure_ashape_c5(torch, M, q, k, v, steps, warmup, n_init=128, n_local=4096):
+    """BASELINE config 5's A-shape heads: sink 128 + window 4096 on resident q/k/v."""
+    ms = _time_steps(torch, lambda: M.streaming_forward(q, k, v, n_init, n_local), steps, warmup)
+    tiles = q.shape[1] * ashape_tiles(q.shape[2], n_init, n_local)
+    tf = tiles * TILE_FLOP / (ms * 1e-3) / 1e12
+    return {"ms": round(ms, 3), "heads": q.shape[1], "computed_tiles": tiles, "tflops": round(tf, 1),
+            "frac_of_bf16_peak": round(tf / PEAK_BF16_TFLOPS, 4)}
+
+
+def measure_c5_layer_slice(torch, M, q, k, v, steps, warmup):
+    """BASELINE config 5's attention-layer slice: one layer of the seeded 70/20/10 per-head pattern
+    table (layer 0 of seed 501) through the per-head dispatcher on resident q/k/v."""
+    from minference_amd.llama import seeded_pattern_mix
+    table = seeded_pattern_mix(1, q.shape[1], seed=501)
+    kwargs = {"layer_idx": 0, "attn_forward_config": {"best_pattern": table}}
+    kinds = [e[0] for e in table[0].values()]
+    ms = _time_steps(torch, lambda: M.minference_prefill_forward(q, k, v, kwargs), steps, warmup)
+    return {"ms": round(ms, 3), "heads": {kind: kinds.count(kind) for kind in sorted(set(kinds))}}
+
+
+def measure_llama_c5(torch, dev, n, layers, steps, warmup):
     """BASELINE config 5: random-init Llama-3-8B (32 layers, hidden 4096, 32 q / 8 kv heads, RoPE
-    theta 500000, SwiGLU 14336, vocab 128256), one 262144-token prefill, per-head patterns drawn
+    theta 500000, SwiGLU 14336, vocab 128256), one n-token prefill, per-head patterns drawn
     with seed 501 (70 % vertical_slash 1000/6096, 20 % block_sparse top-100, 10 % A-shape 128+4096)."""
     from minference_amd.llama import LlamaConfig, LlamaPrefill, seeded_pattern_mix
-    n = args.seq if args.seq != 131072 else 262144
-    cfg = LlamaConfig(num_layers=args.layers)
+    cfg = LlamaConfig(num_layers=layers)
     model = LlamaPrefill(cfg, device=dev, seed=0)
     ids = torch.randint(0, cfg.vocab_size, (n,), generator=torch.Generator().manual_seed(500))
     afc = {"best_pattern": seeded_pattern_mix(cfg.num_layers, cfg.num_heads, seed=501)}
@@ -161,25 +205,81 @@ def bench_llama_c5(args, torch, dev):
     def run():
         logits, _ = model.prefill(ids, afc)
         return logits
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         run()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         logits = run()
     torch.cuda.synchronize()
-    sec = (time.perf_counter() - t0) / args.steps
+    sec = (time.perf_counter() - t0) / steps
     assert torch.isfinite(logits).all()
+    out = {"s_per_prefill": round(sec, 3), "tokens": n, "layers": cfg.num_layers, "repetitions": steps, "warmup": warmup,
+           "tokens_per_s": round(n / sec, 1),
+           "linear_tflops_if_attention_were_free": round(model.flops_linear(n) / sec / 1e12, 1)}
+    del model
+    torch.cuda.empty_cache()
+    return out
+
+
+def bench_llama_c5(args, torch, dev):
+    n = args.seq if args.seq != 131072 else 262144
+    r = measure_llama_c5(torch, dev, n, args.layers, args.steps, args.warmup)
     print(json.dumps({
-        "metric": "Llama-3-8B prefill seconds @262144 tokens (BASELINE config 5)", "value": round(sec, 3),
+        "metric": "Llama-3-8B prefill seconds @262144 tokens (BASELINE config 5)", "value": r["s_per_prefill"],
         "unit": "s/prefill", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(sec * 1e3, 1), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": round(r["s_per_prefill"] * 1e3, 1), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "BASELINE config 5: random-init Llama-3-8B architecture, random token ids, "
                                "seeded 70/20/10 per-head mix of vertical_slash / block_sparse / A-shape",
-                   "seq_len": n, "layers": cfg.num_layers},
-        "tokens_per_s": round(n / sec, 1),
-        "linear_tflops_if_attention_were_free": round(model.flops_linear(n) / sec / 1e12, 1)}))
+                   "seq_len": n, "layers": r["layers"]},
+        "tokens_per_s": r["tokens_per_s"],
+        "linear_tflops_if_attention_were_free": r["linear_tflops_if_attention_were_free"]}))
+
+
+def gemm_ceiling(torch, dev):
+    """What the vendor GEMM (torch bf16 matmul -> hipBLASLt) reaches on this GPU in this process, on
+    N(0,1) operands and on all-zero operands: the matrix pipe's practical ceiling on live data (the
+    chip lowers its clock with the switching activity of the operands) next to the nominal peak."""
+    out = {}
+    for size in (8192, 16384):
+        for name in ("randn", "zeros"):
+            if name == "randn":
+                g = torch.Generator(device=dev).manual_seed(size)
+                a = torch.randn((size, size), device=dev, dtype=torch.float32, generator=g).to(torch.bfloat16)
+                b = torch.randn((size, size), device=dev, dtype=torch.float32, generator=g).to(torch.bfloat16)
+            else:
+                a = torch.zeros((size, size), device=dev, dtype=torch.bfloat16)
+                b = torch.zeros((size, size), device=dev, dtype=torch.bfloat16)
+            c = torch.empty((size, size), device=dev, dtype=torch.bfloat16)
+            ms = _time_steps(torch, lambda: torch.matmul(a, b, out=c), 10, 3)
+            out[f"{size}_{name}"] = {"ms": round(ms, 3), "tflops": round(2 * size ** 3 / ms / 1e9, 1)}
+            del a, b, c
+    torch.cuda.empty_cache()
+    out["best_live_tflops"] = max(out[f"{size}_randn"]["tflops"] for size in (8192, 16384))
+    out["best_zero_tflops"] = max(out[f"{size}_zeros"]["tflops"] for size in (8192, 16384))
+    out["what"] = "torch.matmul of two square bf16 matrices (hipBLASLt), event-timed, 10 repetitions after 3"
+    return out
+
+
+def secondary_configs(args, torch, gen, M, dev):
+    """BASELINE's other configs, timed in the same process as the headline (NOT part of `value`;
+    config 4 is measured by the caller on the headline's resident inputs): config 3 (index builder
+    alone), config 5's A-shape heads, config 5's mixed attention layer, and -- unless --no-llama --
+    one whole config-5 prefill."""
+    sec = {}
+    sec["index_c3"] = {str(n): r for n, r in measure_index_c3(torch, gen, M, dev, 5, 2).items()}
+    n5 = 262144
+    q5, k5, v5, _ = gen.planted_layer(n5, 32, 8, seed=100, dtype=torch.bfloat16)
+    q5, k5, v5 = q5.to(dev), k5.to(dev), v5.to(dev)
+    sec["ashape_c5"] = dict(measure_ashape_c5(torch, M, q5, k5, v5, 5, 2), seq_len=n5, n_init=128, n_local=4096)
+    sec["c5_layer_slice"] = dict(measure_c5_layer_slice(torch, M, q5, k5, v5, 3, 2), seq_len=n5,
+                                 inputs="planted layer of config 2 at 262144 tokens")
+    del q5, k5, v5
+    torch.cuda.empty_cache()
+    if not args.no_llama:
+        sec["llama_c5"] = measure_llama_c5(torch, dev, n5, 32, 1, 0)
+    return sec
 
 
 def sensitivity_lines(args, torch, gen, M, dev, n, hq, hk):
@@ -248,6 +348,10 @@ def main():
     ap.add_argument("--layers", type=int, default=32, help="llama_c5: number of decoder layers")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-dense", action="store_true")
+    ap.add_argument("--no-secondary", action="store_true",
+                    help="skip BASELINE's other configs (index builder alone, block-sparse, A-shape, the config-5 "
+                         "attention layer and one config-5 prefill), which the default line reports under `secondary`")
+    ap.add_argument("--no-llama", action="store_true", help="secondary: skip the whole config-5 prefill (about 30 s)")
     ap.add_argument("--no-sensitivity", action="store_true",
                     help="skip the extra timings off the headline workload (literal config 2 text, scattered lists, zero operands)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -376,6 +480,19 @@ def main():
         extra["sensitivity"]["zero_operands"] = {
             "attention_ms": round(zero_ms, 3), "tflops_on_computed_tiles": round(tiles * TILE_FLOP / zero_ms / 1e9, 1),
             "frac_of_peak": round(tiles * TILE_FLOP / zero_ms / 1e9 / PEAK_BF16_TFLOPS, 4)}
+        extra["sensitivity"]["gemm_ceiling"] = gemm_ceiling(torch, dev)
+    if not args.no_secondary:
+        try:
+            del out
+        except NameError:
+            pass
+        del bc, bo, cc, ci
+        torch.cuda.empty_cache()
+        extra["secondary"] = {"block_sparse_c4": dict(measure_block_sparse_c4(torch, M, q, k, v, 5, 2), seq_len=n)}
+        del q, k, v
+        torch.cuda.empty_cache()
+        extra["secondary"].update(secondary_configs(args, torch, gen, M, dev))
+    gemm = extra.get("sensitivity", {}).get("gemm_ceiling")
     result = {
         "metric": "sparse prefill attn ms/layer @128K (Llama-3-8B shape); effective TFLOP/s",
         "value": round(ms_per_step, 3), "unit": "ms/layer", "n_gpus": 1, "steps": args.steps,
@@ -385,7 +502,8 @@ def main():
                                f"seq {n}, 32 q / 8 kv heads, head_dim 128, vertical 1000, slash 6096, "
                                "planted sink/heavy-column/local-decay structure (tests/gen.py planted_layer); "
                                "the timed index stage writes counts and payload only (zero_fill=0); the reference's "
-                               "zero-filled full tensors are timed beside it as stage_ms.index_zero_filled_full",
+                               "zero-filled full tensors are timed beside it as stage_ms.index_zero_filled_full; "
+                               "`secondary` holds BASELINE's other configs timed in the same process, not part of `value`",
                    "seq_len": n, "batch": 1},
         "effective_tflops": round(eff_tflops, 1),
         "computed_tiles": tiles, "coverage": round(tiles / causal_tiles, 4),
@@ -401,6 +519,8 @@ def main():
         "roofline": {"kernel": "attn_fwd_kernel<bf16, vertical-slash>", "bound": "mfma",
                      "achieved": round(eff_tflops, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(eff_tflops / PEAK_BF16_TFLOPS, 4),
+                     # the same rate against the vendor GEMM's on live (N(0,1)) operands in this process
+                     "frac_of_gemm_ceiling": round(eff_tflops / gemm["best_live_tflops"], 4) if gemm else None,
                      "traffic": traffic["attention_bytes"] if traffic else None,
                      "traffic_source": traffic["source"] if traffic else None,
                      "launch_ms": round(attn_ms, 3), "flop_per_launch": tiles * TILE_FLOP},
