@@ -137,7 +137,9 @@ int minf_vs_index_build_static(const int32_t *seqlens, const int32_t *vertical_i
  *   needed; the reference always expands K/V first,
  *   minference/modules/forward.py:128-132).  head_dim must be 64 or 128 (the
  *   reference's kernels accept 16/32/64/128, pit_sparse_flash_attention_v2.py:172;
- *   smaller head dims are zero-padded to 64 by the caller).
+ *   smaller head dims are zero-padded to 64 by the caller); the A-shape, tri-shape and dense
+ *   entry points also take 256, as the reference's streaming kernel does
+ *   (minference/ops/streaming_kernel.py:429).
  *   seqlens [batch] int32 may be NULL (= n for every batch).  Rows >= seqlen
  *   are written as zeros (the reference leaves its zeros_like buffer untouched).
  *   sm_scale multiplies q.k before the softmax (reference: head_dim^-0.5).
@@ -204,8 +206,12 @@ int minf_ashape_attn_fwd(const minf_qkvo *t, int n_init, int n_local, void *stre
  * minference/ops/streaming_kernel.py:820-833 and minference/modules/minference_forward.py:444-455),
  * which runs the A-shape op on the truncated sequence, a dense einsum/softmax for the last rows
  * and a torch.cat.  The caller clamps n_last to n - 1 like the reference.
+ * sm_scale_last scales q.k of the last n_last rows (0 = t->sm_scale): the reference scales those by
+ * head_dim^-0.5 (:826) but the A-shape rows by the power-of-two PADDED head_dim^-0.5 (:575 after
+ * :793-797), which differ when head_dim is not a power of two.
  */
-int minf_trishape_attn_fwd(const minf_qkvo *t, int n_init, int n_local, int n_last, void *stream);
+int minf_trishape_attn_fwd(const minf_qkvo *t, int n_init, int n_local, int n_last,
+                           float sm_scale_last, void *stream);
 
 /*
  * Dense causal forward on the same tile engine (the in-house comparator for

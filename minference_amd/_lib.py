@@ -29,7 +29,7 @@ SIGNATURES = {
     "minf_vs_attn_fwd": (c_int, [c_ptr] * 5 + [c_int] * 3 + [c_ptr]),
     "minf_bs_attn_fwd": (c_int, [c_ptr, c_ptr, c_int, c_int, c_ptr]),
     "minf_ashape_attn_fwd": (c_int, [c_ptr, c_int, c_int, c_ptr]),
-    "minf_trishape_attn_fwd": (c_int, [c_ptr, c_int, c_int, c_int, c_ptr]),
+    "minf_trishape_attn_fwd": (c_int, [c_ptr, c_int, c_int, c_int, c_f32, c_ptr]),
     "minf_dense_attn_fwd": (c_int, [c_ptr, c_ptr]),
     "minf_vs_estimate_workspace_bytes": (ctypes.c_size_t, [c_int, c_int, c_int]),
     "minf_vs_estimate": (c_int, [c_ptr, c_ptr, c_ptr, c_ptr] + [c_int] * 6 + [c_f32] + [c_int] * 4

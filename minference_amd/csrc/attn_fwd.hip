@@ -76,7 +76,7 @@ enum { MODE_VS = 0, MODE_BS = 1, MODE_ASHAPE = 2, MODE_DENSE = 3 };
 
 constexpr int BM = 64;        // query rows per workgroup
 constexpr int BN = 64;        // keys per tile
-constexpr int HD_MAX = 128;   // head_dim: 128 or 64 (template parameter HD of the kernel)
+constexpr int HD_MAX = 256;   // head_dim: 64, 128 or (dense / A-shape / tri-shape only) 256: template parameter HD of the kernel
 constexpr int NTHREADS = 128; // 2 wavefronts per 64-row block, two row blocks per workgroup
 // Scheduling constants (measured on MI355X): K fragments are read QK_AHEAD k-steps ahead of their
 // MFMAs; VALU_PER_MFMA softmax instructions are placed behind each of the first twelve PV MFMAs.
@@ -97,6 +97,7 @@ struct AttnParams {
     int batch, hq, hk, n;
     const int *seqlens;
     float scale_log2;
+    float scale_log2_dense;  // tri-shape: scale of the rows >= dense_from (the reference scales them by the unpadded head_dim)
     int rows;
     // vertical-slash
     const int *bc, *bo, *cc, *ci;
@@ -233,7 +234,8 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
                                           char (&lds_v)[AttnLds<MODE, HD>::NK],
                                           int (&vs_only)[AttnLds<MODE, HD>::NONLY], int (&vs_wsum)[4], int &vs_bad,
                                           int &lds_redo) {
-    static_assert(HD == 128 || HD == 64, "head_dim 128 or 64");
+    static_assert(HD == 256 || HD == 128 || HD == 64, "head_dim 64, 128 or 256");
+    static_assert(HD <= 128 || !(MODE == MODE_VS || MODE == MODE_BS), "the list walks are built for head_dim <= 128");
     constexpr int ROW_BYTES = HD * 2;                       // one token row of K / V / Q / O
     constexpr int KS = HD / 16;                             // k-steps of S^T = K.Q^T
     constexpr int NDB = HD / 32;                            // 32-row blocks of O^T
@@ -242,8 +244,8 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
     // LDS chunk permutations (conflict-free ds_read_b128 of 32 K rows / transpose reads of 4 V rows):
     // 256-byte rows: K chunk ^ row%16, V chunk ^ 4*(row%4); 128-byte rows (two rows per bank sweep):
     // K chunk ^ (row/2)%8, V chunk ^ 4*((row/2)%2)
-    auto swz_k = [](int row) { return HD == 128 ? (row & 15) : ((row >> 1) & 7); };
-    auto swz_v = [](int row) { return HD == 128 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); };
+    auto swz_k = [](int row) { return HD >= 128 ? (row & 15) : ((row >> 1) & 7); };
+    auto swz_v = [](int row) { return HD >= 128 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); };
     constexpr int NT = 2 * NTHREADS;                        // threads per workgroup
     constexpr int CROWS = 16;                               // tile rows copied by one wave (shared tile)
     // VSP: the paired walk of two block lists -- the vertical-slash block lists, or the block-sparse
@@ -328,6 +330,11 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
     const long long ridx = ((long long)b * p.index_heads + hs) * p.rows + min(m, p.rows - 1);
 
     constexpr bool every_max = EVERY_MAX;
+    // log2-domain scale of this lane's query row: one value per launch, except for the dense rows of a
+    // tri-shape launch (the reference scales its A-shape rows by the padded head_dim and its last
+    // rows by the unpadded one, streaming_kernel.py:575 against :826)
+    float sc_l2 = p.scale_log2;
+    if constexpr (MODE == MODE_ASHAPE) sc_l2 = qrow >= p.dense_from ? p.scale_log2_dense : p.scale_log2;
     // ---- Q fragments (B operand of S^T): row qrow, d = 16*ks + 8*g + 0..7 ----
     Frag qf[KS];
     {
@@ -505,10 +512,14 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
     const int cp_c = lane % NCH;                 // LDS chunk
     // gathered tiles: lane l holds the token id of tile row l (one load per lane, issued an
     // iteration ahead); the copy fetches the ids of its own rows with wave shuffles
-    int k_lane[4], v_lane;
+    // (per-lane offsets of the buffer-form copies: the K permutation repeats every 16 rows, i.e. every
+    // KL copy instructions, the V permutation every 4 rows: every VL instructions)
+    constexpr int KL = RPI >= 4 ? 4 : 16 / RPI, VL = RPI >= 4 ? 1 : 4 / RPI;
+    int k_lane[KL], v_lane[VL];
 #pragma unroll
-    for (int jj = 0; jj < 4; ++jj) k_lane[jj] = cp_r * (int)k_row + ((cp_c ^ swz_k(RPI * jj + cp_r)) << 4);
-    v_lane = cp_r * (int)v_row + ((cp_c ^ swz_v(cp_r)) << 4);
+    for (int jj = 0; jj < KL; ++jj) k_lane[jj] = cp_r * (int)k_row + ((cp_c ^ swz_k(RPI * jj + cp_r)) << 4);
+#pragma unroll
+    for (int jj = 0; jj < VL; ++jj) v_lane[jj] = cp_r * (int)v_row + ((cp_c ^ swz_v(RPI * jj + cp_r)) << 4);
     auto gather_ids = [&](const Tile &t) -> int {
         if (MODE == MODE_VS && t.gathered) return p.ci[ridx * p.nnz_v + t.start + min(lane, max(t.nvalid, 1) - 1)];
         return 0;
@@ -533,7 +544,7 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
             if constexpr (VSP) asm volatile("" : "+s"(soff0), "+s"(sstep), "+s"(lds0));
 #pragma unroll
             for (int j = 0; j < CROWS / RPI; ++j) {
-                const int voff = is_v ? v_lane : k_lane[j & 3];     // (the K permutation repeats every 16 rows)
+                const int voff = is_v ? v_lane[j & (VL - 1)] : k_lane[j & (KL - 1)];
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(srd, (__attribute__((address_space(3))) void *)(unsigned long long)(unsigned)(lds0 + RPI * j * ROW_BYTES),
                                                          16, voff, soff0 + j * sstep, 0, 0);
             }
@@ -631,7 +642,10 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
 
     // ---- mask, V^T fragment reads, online softmax, O^T += V^T . P^T
     auto sm_pv_block = [&](const Tile &cur, const char *vbuf, f32x16_t &s0, f32x16_t &s1) {
-        Frag vf[4][NDB];
+        // (head_dim 256: the 64 registers of a whole tile's V^T fragments do not fit next to O^T and Q;
+        // that form reads the fragments of one key group at a time, right before their MFMAs)
+        constexpr bool VF_AHEAD = HD <= 128;
+        Frag vf[VF_AHEAD ? 4 : 1][NDB];
         // element (blk, r) of this lane is tile-local key tk = tkc + 4*g with the compile-time
         // part tkc = 32*blk + 8*(r/4) + r%4.  keep <=> tk <= hi && (tk > wlo || tk < slim).
         bool need_mask;
@@ -679,6 +693,7 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
         // chain: the PV block below is bound by its vector instructions, so every LDS read moved out
         // of it shortens it (+3 % for the 24 reads that used to sit between its MFMAs), and the reads
         // fill the dependency gaps of the max chain (+0.7 % over reading them before the K copy).
+        if constexpr (VF_AHEAD) {
 #pragma unroll
         for (int s = 0; s < 4; ++s)
 #pragma unroll
@@ -687,6 +702,7 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
             for (int jj = 0; jj < 2; ++jj)
                 vf[s][db].s4[jj] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
                     (__attribute__((address_space(3))) short4_t *)(vbuf + v_rd_off[db] + (16 * s + 8 * jj) * ROW_BYTES));
+        }
         }
         // ---- online softmax (exp2 domain) -------------------------------------
         // The reference maximum m_i of a row only has to keep exp2 inside the range of fp32 (bf16 has the
@@ -710,7 +726,7 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
             mx = fmaxf(fmaxf(fmaxf(m4[0], m4[1]), m4[2]), m4[3]);
         }
         { const unsigned u = __float_as_uint(mx); auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false); mx = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1])); }
-        const float cand = mx * p.scale_log2;
+        const float cand = mx * sc_l2;
         // lazy: raised only when a tile exceeds it by more than LAZY_MAX powers of two (probabilities of
         // f16 operands must stay inside the f16 range: 2^8 leaves room for the row sums)
         constexpr float LAZY_MAX = std::is_same<T, __bf16>::value ? LAZY_MAX_BF16 : 8.0f;
@@ -727,7 +743,7 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
             const f32x16_t &sx = q < 2 ? s0 : s1;
             float pv[8];
 #pragma unroll
-            for (int r = 0; r < 8; ++r) pv[r] = __builtin_amdgcn_exp2f(fmaf(sx[8 * (q & 1) + r], p.scale_log2, -m_use));
+            for (int r = 0; r < 8; ++r) pv[r] = __builtin_amdgcn_exp2f(fmaf(sx[8 * (q & 1) + r], sc_l2, -m_use));
             cvt8<T>(&pv[0], pfr[q]);
             psum = pair_sum<T>(pfr[q], psum);
         };
@@ -746,6 +762,7 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
             probs(2);
             probs(3);
             l_i = l_i * alpha + psum;
+            if constexpr (VF_AHEAD) {
 #pragma unroll
             for (int s = 0; s < 4; ++s)
 #pragma unroll
@@ -756,6 +773,20 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
             for (int i = 0; i < 4 * NDB; ++i) {
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
                 if (i < 3 * NDB) __builtin_amdgcn_sched_group_barrier(VALU_MASK, VALU_PER_MFMA * 4 / NDB, 0);
+            }
+            } else {
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+#pragma unroll
+                for (int db = 0; db < NDB; ++db)
+#pragma unroll
+                    for (int jj = 0; jj < 2; ++jj)
+                        vf[0][db].s4[jj] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                            (__attribute__((address_space(3))) short4_t *)(vbuf + v_rd_off[db] + (16 * s + 8 * jj) * ROW_BYTES));
+#pragma unroll
+                for (int db = 0; db < NDB; ++db)
+                    oacc[db] = Mma<T>::mfma(frag_as<T>(vf[0][db]), frag_as<T>(pfr[s]), oacc[db]);
+            }
             }
         }
         __builtin_amdgcn_s_setprio(0);
@@ -916,8 +947,10 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
     return !every_max && lds_redo != 0;                   // (workgroup-uniform)
 }
 
+// (head_dim 256: O^T, Q and the V^T fragments of a wave need more than 256 registers, so that form
+// runs one wave per SIMD with the accumulators in the second half of the register file)
 template <typename T, int MODE, int HD>
-__global__ __launch_bounds__(2 * NTHREADS, 2) void attn_fwd_kernel(const AttnParams p) {
+__global__ __launch_bounds__(2 * NTHREADS, HD > 128 ? 1 : 2) void attn_fwd_kernel(const AttnParams p) {
     typedef AttnLds<MODE, HD> L;
     __shared__ __attribute__((aligned(16))) char lds_k[L::NK];
     __shared__ __attribute__((aligned(16))) char lds_v[L::NK];
@@ -937,7 +970,7 @@ __global__ __launch_bounds__(2 * NTHREADS, 2) void attn_fwd_kernel(const AttnPar
     }
 }
 
-int check_tensors(const minf_qkvo *t) {
+int check_tensors(const minf_qkvo *t, bool allow_256 = false) {
     if (!t) return MINF_ERR_INVALID_ARG;
     if (t->batch < 0 || t->heads_q <= 0 || t->heads_kv <= 0 || t->n < 0) return MINF_ERR_INVALID_ARG;
     // empty problems (no batch or no tokens) have no storage: nothing to check, nothing is launched
@@ -945,7 +978,7 @@ int check_tensors(const minf_qkvo *t) {
     if (!empty && (!t->q || !t->k || !t->v || !t->o)) return MINF_ERR_INVALID_ARG;
     if (t->heads_q % t->heads_kv != 0) return MINF_ERR_INVALID_ARG;
     if (t->head_list && t->index_heads <= 0) return MINF_ERR_INVALID_ARG;
-    if (t->head_dim != 128 && t->head_dim != 64) return MINF_ERR_UNSUPPORTED;
+    if (t->head_dim != 128 && t->head_dim != 64 && !(allow_256 && t->head_dim == 256)) return MINF_ERR_UNSUPPORTED;
     if (t->dtype != MINF_BF16 && t->dtype != MINF_F16) return MINF_ERR_UNSUPPORTED;
     const void *ptrs[4] = {t->q, t->k, t->v, t->o};
     const int64_t *strides[4] = {t->q_stride, t->k_stride, t->v_stride, t->o_stride};
@@ -971,6 +1004,7 @@ void fill_params(AttnParams &p, const minf_qkvo *t) {
     p.batch = t->batch; p.hq = t->heads_q; p.hk = t->heads_kv; p.n = t->n;
     p.seqlens = t->seqlens;
     p.scale_log2 = t->sm_scale * 1.4426950408889634f;
+    p.scale_log2_dense = p.scale_log2;
     p.rows = (t->n + BM - 1) / BM;
     p.bc = p.bo = p.cc = p.ci = nullptr; p.nnz_s = p.nnz_v = 0;
     p.bidx = nullptr; p.max_blocks = 0; p.bidx_rows = 0;
@@ -999,6 +1033,9 @@ template <int MODE, int HD> int launch_hd(AttnParams p, int dtype, void *stream)
 }
 
 template <int MODE> int launch(const AttnParams &p, const minf_qkvo *t, void *stream) {
+    if constexpr (MODE == MODE_ASHAPE || MODE == MODE_DENSE)
+        if (t->head_dim == 256) return launch_hd<MODE, 256>(p, t->dtype, stream);
+    if (t->head_dim == 256) return MINF_ERR_UNSUPPORTED;
     return t->head_dim == 64 ? launch_hd<MODE, 64>(p, t->dtype, stream) : launch_hd<MODE, 128>(p, t->dtype, stream);
 }
 
@@ -1034,7 +1071,7 @@ extern "C" int minf_bs_attn_fwd(const minf_qkvo *t, const int32_t *block_index, 
 }
 
 extern "C" int minf_ashape_attn_fwd(const minf_qkvo *t, int n_init, int n_local, void *stream) {
-    int st = check_tensors(t);
+    int st = check_tensors(t, true);
     if (st) return st;
     if (n_init < 0 || n_local < 1) return MINF_ERR_INVALID_ARG;
     AttnParams p;
@@ -1043,19 +1080,21 @@ extern "C" int minf_ashape_attn_fwd(const minf_qkvo *t, int n_init, int n_local,
     return launch<MODE_ASHAPE>(p, t, stream);
 }
 
-extern "C" int minf_trishape_attn_fwd(const minf_qkvo *t, int n_init, int n_local, int n_last, void *stream) {
-    int st = check_tensors(t);
+extern "C" int minf_trishape_attn_fwd(const minf_qkvo *t, int n_init, int n_local, int n_last,
+                                      float sm_scale_last, void *stream) {
+    int st = check_tensors(t, true);
     if (st) return st;
-    if (n_init < 0 || n_local < 1 || n_last < 0) return MINF_ERR_INVALID_ARG;
+    if (n_init < 0 || n_local < 1 || n_last < 0 || !(sm_scale_last >= 0.f)) return MINF_ERR_INVALID_ARG;
     AttnParams p;
     fill_params(p, t);
+    if (sm_scale_last > 0.f) p.scale_log2_dense = sm_scale_last * 1.4426950408889634f;
     p.n_init = n_init; p.n_local = n_local;
     p.dense_from = n_last < t->n ? t->n - n_last : 0;
     return launch<MODE_ASHAPE>(p, t, stream);
 }
 
 extern "C" int minf_dense_attn_fwd(const minf_qkvo *t, void *stream) {
-    int st = check_tensors(t);
+    int st = check_tensors(t, true);
     if (st) return st;
     AttnParams p;
     fill_params(p, t);

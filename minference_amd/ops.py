@@ -23,8 +23,8 @@ import torch
 from . import _lib
 from .index import convert_vertical_slash_indexes
 
-_SUPPORTED_D = 128            # largest head_dim
-_NATIVE_D = (64, 128)         # head_dims the tile engine is instantiated for; others are zero-padded up
+_NATIVE_D = (64, 128)         # head_dims every kernel is instantiated for; others are zero-padded up
+_NATIVE_D_STREAMING = (64, 128, 256)   # ... and the A-shape / tri-shape / dense kernels also for 256
 
 
 def _prep(t: torch.Tensor) -> torch.Tensor:
@@ -72,7 +72,7 @@ class _Call:
     """Holds the (possibly cast/padded) tensors of one operator call and the
     filled ``minf_qkvo`` struct."""
 
-    def __init__(self, q, k, v, seqlens=None, need_out=True):
+    def __init__(self, q, k, v, seqlens=None, need_out=True, native_dims=_NATIVE_D, sm_scale=None):
         _check_qkv(q, k, v)
         self.out_dtype = q.dtype
         self.head_dim = q.shape[-1]
@@ -82,11 +82,14 @@ class _Call:
         elif q.dtype not in (torch.bfloat16, torch.float16):
             raise ValueError(f"unsupported dtype {q.dtype}")
         D = q.shape[-1]
-        if D > _SUPPORTED_D:
-            raise ValueError(f"head_dim {D} > {_SUPPORTED_D} is not supported")
+        if D > max(native_dims):
+            # the reference's vertical-slash and block-sparse kernels assert head_dim <= 128
+            # (pit_sparse_flash_attention_v2.py:172, block_sparse_flash_attention.py:128), its streaming
+            # kernel head_dim <= 256 (streaming_kernel.py:429)
+            raise ValueError(f"head_dim {D} > {max(native_dims)} is not supported by this operator")
         # the reference runs head_dim 16, 32, 64, 128 (pit_sparse_flash_attention_v2.py:172); here 64 and
-        # 128 are native, anything else is zero-padded to the next of the two
-        Dk = min(d for d in _NATIVE_D if d >= D)
+        # 128 (and 256 for the streaming operators) are native, anything else is zero-padded to the next
+        Dk = min(d for d in native_dims if d >= D)
         if D < Dk:
             # zero columns change neither q.k nor the first D output columns
             pad = Dk - D
@@ -108,7 +111,7 @@ class _Call:
         s.dtype = _lib.MINF_BF16 if self.q.dtype == torch.bfloat16 else _lib.MINF_F16
         self.seqlens = seqlens
         s.seqlens = seqlens.data_ptr() if seqlens is not None else None
-        s.sm_scale = float(self.head_dim) ** -0.5
+        s.sm_scale = float(self.head_dim) ** -0.5 if sm_scale is None else float(sm_scale)
         self.struct = s
 
     @property
@@ -232,10 +235,21 @@ def block_sparse_attention(query, key, value, top_k: int, block_size_M: int = 64
     return block_sparse_attention_from_index(query, key, value, block_index)
 
 
+def _streaming_scale(head_dim: int) -> float:
+    """Softmax scale of the reference's streaming operator: it zero-pads a head_dim outside
+    {16, 32, 64, 128, 256} to the next power of two FIRST (streaming_kernel.py:621-626, :793-797) and
+    then scales by 1/sqrt of the padded size (:575) -- e.g. head_dim 96 is scaled by 128^-0.5."""
+    d = int(head_dim)
+    if d not in (16, 32, 64, 128, 256):
+        d = 1 << (d - 1).bit_length()
+    return float(d) ** -0.5
+
+
 def streaming_forward(q, k, v, n_init: int, n_local: int):
     """A-shape attention: n_init sink tokens + a sliding window of n_local
-    (streaming_kernel.py:611-646), in one pass."""
-    c = _Call(q, k, v)
+    (streaming_kernel.py:611-646), in one pass.  head_dim up to 256 like the reference (:429); the
+    scale follows the reference's padded head_dim (see _streaming_scale)."""
+    c = _Call(q, k, v, native_dims=_NATIVE_D_STREAMING, sm_scale=_streaming_scale(q.shape[-1]))
     lib = _lib.load()
     with torch.cuda.device(c.q.device):
         st = lib.minf_ashape_attn_fwd(c.ref, int(n_init), int(n_local), _lib.stream_ptr(c.q.device))
@@ -246,20 +260,21 @@ def streaming_forward(q, k, v, n_init: int, n_local: int):
 def tri_shape_forward(q, k, v, n_init: int, n_local: int, n_last: int = 100):
     """Tri-shape attention: A-shape (n_init sink tokens + window of n_local) for all but the last
     n_last query rows, dense causal attention for those (streaming_kernel.py:820-833,
-    minference_forward.py:444-455), in one launch."""
-    c = _Call(q, k, v)
+    minference_forward.py:444-455), in one launch.  Like the reference, the A-shape rows are scaled
+    by the padded head_dim (see _streaming_scale) and the last rows by head_dim^-0.5 (:826)."""
+    c = _Call(q, k, v, native_dims=_NATIVE_D_STREAMING, sm_scale=_streaming_scale(q.shape[-1]))
     n_last = min(int(n_last), c.N - 1)                   # reference: min(n_last, q.size(2) - 1)
     lib = _lib.load()
     with torch.cuda.device(c.q.device):
         st = lib.minf_trishape_attn_fwd(c.ref, int(n_init), int(n_local), max(n_last, 0),
-                                        _lib.stream_ptr(c.q.device))
+                                        float(c.head_dim) ** -0.5, _lib.stream_ptr(c.q.device))
     _lib.check(st, "minf_trishape_attn_fwd")
     return c.result()
 
 
 def dense_causal_attention(q, k, v):
     """Dense causal attention on the same tile engine (comparator for speed-up figures)."""
-    c = _Call(q, k, v)
+    c = _Call(q, k, v, native_dims=_NATIVE_D_STREAMING)
     lib = _lib.load()
     with torch.cuda.device(c.q.device):
         st = lib.minf_dense_attn_fwd(c.ref, _lib.stream_ptr(c.q.device))

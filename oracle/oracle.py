@@ -371,15 +371,44 @@ def block_sparse_attention(q, k, v, top_k):
     return out
 
 
+def streaming_scale(head_dim):
+    """The softmax scale of the reference's streaming operator: head dims outside {16, 32, 64, 128,
+    256} are zero-padded to the next power of two first (streaming_kernel.py:621-626; a_shape_kernel
+    :793-797) and ``append`` then takes 1/sqrt of the PADDED size (:575)."""
+    d = head_dim
+    if d not in (16, 32, 64, 128, 256):
+        d = 2 ** math.ceil(math.log2(d))
+    return 1.0 / math.sqrt(d)
+
+
 def streaming_forward(q, k, v, n_init, n_local):
-    """streaming_kernel.py:611-646 on CPU in fp32."""
+    """streaming_kernel.py:611-646 on CPU in fp32 (scale: see streaming_scale)."""
     B, H, N, D = q.shape
     m = ashape_mask(N, n_init, n_local)
     out = torch.empty(B, H, N, D, dtype=torch.float32)
     for b in range(B):
         for h in range(H):
-            out[b, h] = masked_attention(q[b, h], k[b, h], v[b, h], m)
+            out[b, h] = masked_attention(q[b, h], k[b, h], v[b, h], m, scale=streaming_scale(D))
     return out
+
+
+def tri_shape_forward(q, k, v, n_init, n_local, n_last):
+    """tri_shape_kernel (streaming_kernel.py:820-833, minference_forward.py:444-455) on CPU in fp32:
+    the A-shape operator on all but the last n_last tokens (its scale: streaming_scale), dense causal
+    rows scaled by 1/sqrt(head_dim) (:826) for the last n_last queries."""
+    B, H, N, D = q.shape
+    n_last = min(n_last, N - 1)
+    if n_last <= 0:
+        return streaming_forward(q, k, v, n_init, n_local)
+    y1 = streaming_forward(q[:, :, :-n_last], k[:, :, :-n_last], v[:, :, :-n_last], n_init, n_local)
+    dense = torch.ones(N, N, dtype=torch.bool).tril()[-n_last:]
+    y2 = torch.empty(B, H, n_last, D, dtype=torch.float32)
+    for b in range(B):
+        for h in range(H):
+            s = (q[b, h, -n_last:].float() @ k[b, h].float().T) / math.sqrt(D)
+            s = torch.where(dense, s, torch.tensor(-torch.inf))
+            y2[b, h] = torch.softmax(s, dim=-1) @ v[b, h].float()
+    return torch.cat([y1, y2], dim=2)
 
 
 # --------------------------------------------------------------------------

@@ -98,7 +98,7 @@ def test_argument_validation_of_the_index_estimate_and_search_entry_points(lib):
     assert lib.minf_vs_attn_fwd(ctypes.byref(t), None, P, P, P, 3, 8, 8, None) == -1
     assert lib.minf_bs_attn_fwd(ctypes.byref(t), P, 2, 4, None) == -1                     # too few rows
     assert lib.minf_ashape_attn_fwd(ctypes.byref(t), 4, 0, None) == -1                    # n_local < 1
-    assert lib.minf_trishape_attn_fwd(ctypes.byref(t), 4, 8, -1, None) == -1
+    assert lib.minf_trishape_attn_fwd(ctypes.byref(t), 4, 8, -1, 0.0, None) == -1
     # pattern search: flag pitch rules, candidate bit range, workspace
     assert lib.minf_pattern_recall(P, P, i3, i3, 1, 4, 4, 130, 128, 0, 0.1, P, P, 128, None, 0, 0, P, P, 1 << 20, None) == -1   # pitch < 192
     assert lib.minf_pattern_recall(P, P, i3, i3, 1, 4, 4, 130, 128, 0, 0.1, P, P, 192, None, 0, 0, P, P, 8, None) == -4

@@ -506,6 +506,47 @@ def test_tri_shape_vs_oracle(gpu, n, n_init, n_local, n_last):
     check(out, ref, "trishape")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("d,n,hq,hk,n_init,n_local", [
+    (256, 700, 2, 1, 16, 100), (192, 1000, 4, 2, 128, 256), (256, 2049, 2, 2, 0, 640), (256, 63, 1, 1, 4, 1000),
+    (96, 900, 2, 1, 8, 200), (160, 333, 2, 2, 70, 50)])
+def test_streaming_head_dims_up_to_256(gpu, monkeypatch, dtype, d, n, hq, hk, n_init, n_local):
+    """The streaming operator takes head_dim up to 256 (streaming_kernel.py:429) and zero-pads other
+    sizes to the next power of two, taking its scale from the PADDED size (:621-626, :575): 192 runs
+    as 256 with scale 1/16, 96 as 128 with scale 128^-0.5, 160 as 256.  Dense causal attention at the
+    same head dims against torch's SDPA (scale 1/sqrt(head_dim))."""
+    import minference_amd as M
+    print(f"case streaming head_dim={d} n={n} hq={hq} hk={hk} {dtype}", flush=True)
+    q, k, v = make(1, hq, hk, n, 300 + d, dtype, d=d)
+    qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
+    if d == 256:                                   # native: no zero-padded copies
+        def no_pad(*a, **kw):
+            raise AssertionError("head_dim 256 must not be padded")
+        monkeypatch.setattr(torch.nn.functional, "pad", no_pad)
+    out = M.streaming_forward(qg, kg, vg, n_init, n_local)
+    dense = M.dense_causal_attention(qg, kg, vg)
+    monkeypatch.undo()
+    assert out.shape == q.shape and out.dtype == dtype
+    ke, ve = expand(k, hq), expand(v, hq)
+    check(out, O.streaming_forward(q, ke, ve, n_init, n_local), f"a-shape d{d}")
+    check(dense, sdpa_causal(q, ke, ve), f"dense d{d}")
+    n_last = min(n - 1, 100)
+    tri = M.tri_shape_forward(qg, kg, vg, n_init, n_local, n_last)
+    check(tri, O.tri_shape_forward(q, ke, ve, n_init, n_local, n_last), f"tri-shape d{d}")
+
+
+def test_vertical_slash_and_block_sparse_refuse_head_dim_above_128(gpu):
+    """The reference's kernels assert head_dim <= 128 there (pit_sparse_flash_attention_v2.py:172,
+    block_sparse_flash_attention.py:128)."""
+    import minference_amd as M
+    q = torch.zeros((1, 1, 128, 256), dtype=torch.bfloat16, device=gpu)
+    idx = torch.zeros((1, 1, 1), dtype=torch.int32, device=gpu)
+    with pytest.raises(ValueError):
+        M.vertical_slash_sparse_attention(q, q, q, idx, idx)
+    with pytest.raises(ValueError):
+        M.block_sparse_attention(q, q, q, 4)
+
+
 @pytest.mark.parametrize("seed", list(range(8)))
 def test_seeded_random_shapes_all_operators(gpu, seed):
     """Random sequence lengths (any remainder modulo 64), head counts, list sizes and window sizes,

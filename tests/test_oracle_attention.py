@@ -169,3 +169,42 @@ def test_trishape_mask_definition_and_limits():
     # n_last >= n clamps to n - 1: every row but the first is dense, and row 0 only sees key 0 anyway
     assert np.array_equal(O.trishape_mask(50, 2, 5, 1000), np.tril(np.ones((50, 50), bool)))
     assert np.array_equal(O.trishape_mask(50, 2, 5, 0), O.ashape_mask(50, 2, 5))
+
+
+def test_streaming_scale_follows_the_padded_head_dim():
+    """streaming_kernel.py:621-626 zero-pads a head_dim outside {16, ..., 256} to the next power of
+    two and :575 then scales by 1/sqrt(q.shape[-1]) of the PADDED tensor.  Restated literally: pad
+    physically, run the generic masked attention with its default 1/sqrt(last dim), slice."""
+    n, n_init, n_local = 150, 4, 40
+    for d, padded in ((96, 128), (192, 256), (48, 64), (64, 64), (128, 128), (256, 256), (16, 16)):
+        assert abs(O.streaming_scale(d) - padded ** -0.5) < 1e-12
+    g = torch.Generator().manual_seed(3)
+    q, k, v = (torch.randn(1, 2, n, 96, generator=g) for _ in range(3))
+    got = O.streaming_forward(q, k, v, n_init, n_local)
+    pad = lambda t: torch.nn.functional.pad(t, [0, 32])
+    m = O.ashape_mask(n, n_init, n_local)
+    for h in range(2):
+        want = O.masked_attention(pad(q)[0, h], pad(k)[0, h], pad(v)[0, h], m)[:, :96]
+        assert torch.allclose(got[0, h], want, atol=1e-6)
+        plain = O.masked_attention(q[0, h], k[0, h], v[0, h], m)           # 1/sqrt(96): not what the reference does
+        assert (plain - got[0, h]).abs().max() > 1e-3
+
+
+def test_tri_shape_forward_two_scales():
+    """tri_shape_kernel (streaming_kernel.py:820-833): A-shape operator on the first n - n_last tokens,
+    dense rows scaled by 1/sqrt(head_dim) for the rest.  For a power-of-two head_dim both scales agree
+    and the result is the masked attention under trishape_mask; for head_dim 96 the last rows equal
+    torch's causal SDPA rows (scale 1/sqrt(96)) and the first rows the streaming operator's."""
+    n, n_init, n_local, n_last = 130, 3, 20, 17
+    g = torch.Generator().manual_seed(5)
+    q, k, v = (torch.randn(1, 1, n, 64, generator=g) for _ in range(3))
+    got = O.tri_shape_forward(q, k, v, n_init, n_local, n_last)
+    want = O.masked_attention(q[0, 0], k[0, 0], v[0, 0], O.trishape_mask(n, n_init, n_local, n_last))
+    assert torch.allclose(got[0, 0], want, atol=1e-6)
+    q, k, v = (torch.randn(1, 1, n, 96, generator=g) for _ in range(3))
+    got = O.tri_shape_forward(q, k, v, n_init, n_local, n_last)
+    sdpa = torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True)
+    assert torch.allclose(got[:, :, -n_last:], sdpa[:, :, -n_last:], atol=1e-5)
+    first = O.streaming_forward(q[:, :, :-n_last], k[:, :, :-n_last], v[:, :, :-n_last], n_init, n_local)
+    assert torch.equal(got[:, :, :-n_last], first)
+    assert torch.equal(O.tri_shape_forward(q, k, v, n_init, n_local, 0), O.streaming_forward(q, k, v, n_init, n_local))
