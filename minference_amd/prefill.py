@@ -154,7 +154,7 @@ def _mixed_layer(query_states, key_states, value_states, lp):
     The reference runs one operator call per head here (minference_forward.py:657-667)."""
     from . import _lib
     from .estimate import FORCE_SLASH, FORCE_VERTICAL, LAST_Q, reference_rounding_for
-    from .ops import _Call
+    from .ops import _Call, _streaming_scale
     B, H, N, D = query_states.shape
     rounded = reference_rounding_for(query_states.dtype)     # the reference's rounding points on 16-bit inputs
     dev = query_states.device
@@ -215,6 +215,8 @@ def _mixed_layer(query_states, key_states, value_states, lp):
                 st = lib.minf_bs_attn_fwd(c.ref, bi.data_ptr(), brows, kk, stream)
                 _lib.check(st, "minf_bs_attn_fwd")
                 keep += [ws, bi]
+            # (the reference's streaming operator scales by the power-of-two padded head_dim)
+            c.struct.sm_scale = _streaming_scale(D)
             for (n_init, n_local), slot in dt["stream_heads"].items():
                 c.select_heads(slot)
                 if N > 0:
@@ -222,6 +224,7 @@ def _mixed_layer(query_states, key_states, value_states, lp):
                     _lib.check(st, "minf_ashape_attn_fwd")
     finally:
         c.struct.seqlens = None
+        c.struct.sm_scale = float(D) ** -0.5
         c.select_heads(None)
     out = c.result()
     # torch's caching allocator hands a freed block only to work enqueued later on the same stream, so

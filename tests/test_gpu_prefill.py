@@ -36,6 +36,30 @@ def test_mixed_patterns_route_to_the_right_kernels(gpu):
     assert (out[:, 3:5] - ref_def).abs().max() <= 2e-2
 
 
+def test_mixed_patterns_at_head_dim_96(gpu):
+    """A Phi-3-shaped head_dim (96, zero-padded to 128 by the operators): every head of a mixed layer
+    equals its own operator call bit for bit -- in particular the stream_llm heads, which the
+    reference scales by the PADDED head_dim (streaming_kernel.py:575), the others by head_dim^-0.5
+    (pit_sparse_flash_attention_v2.py:221)."""
+    import minference_amd as M
+    n, hq, hk, d = 1500, 4, 2, 96
+    q, k, v = gen.qkv(1, hq, hk, n, d, seed=5, scale=1.0)
+    q, k, v = q.bfloat16().to(gpu), k.bfloat16().to(gpu), v.bfloat16().to(gpu)
+    layer = {"0": ["stream_llm", 16, 200, 1.0], "1": ["vertical_and_slash", 100, 300, 1.0],
+             "2": ["block_sparse", 100, 0, 1.0], "3": ["stream_llm", 16, 200, 1.0]}
+    out = M.minference_prefill_forward(q, k, v, {"layer_idx": 0, "attn_forward_config": {"best_pattern": [layer]}})
+    assert out.shape == q.shape
+    for h in range(hq):
+        qh, kh, vh = q[:, h:h + 1], k[:, h // 2:h // 2 + 1], v[:, h // 2:h // 2 + 1]
+        ty = layer[str(h)][0]
+        ref = (M.streaming_forward(qh, kh, vh, 16, 200) if ty == "stream_llm" else
+               M.vertical_slash_prefill(qh, kh, vh, 100, 300) if ty == "vertical_and_slash" else
+               M.block_sparse_attention(qh, kh, vh, 100))
+        assert torch.equal(out[:, h:h + 1], ref), (h, ty)
+    want = O.streaming_forward(q[:, :1].cpu(), k[:, :1].cpu(), v[:, :1].cpu(), 16, 200)
+    assert (out[:, :1].float().cpu() - want).abs().max() <= 2e-2
+
+
 def _ragged_table(hq):
     """Per-head patterns in the shape of the shipped Llama-3-8B table: vertical_and_slash heads with
     five distinct (vertical, slash) sizes, block_sparse heads, stream_llm heads with two settings."""
