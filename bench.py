@@ -321,17 +321,52 @@ def sensitivity_lines(args, torch, gen, M, dev, n, hq, hk):
     out["literal_c2"] = {"coverage": round(tiles / causal_tiles, 4), "attention_ms": round(ms, 3),
                          "layer_ms": round(ms_layer, 3), "tflops_on_computed_tiles": round(tiles * TILE_FLOP / ms / 1e9, 1)}
     del bc, bo, cc, ci
+    out["scattered"] = measure_scattered(torch, gen, M, dev, q, k, v, 3)
+    return out
+
+
+def measure_scattered(torch, gen, M, dev, q, k, v, reps):
+    """The index lists of BASELINE config 3's generator at q's length with 600 slashes (0..63 forced,
+    the rest uniform) and 1000 uniform verticals, on resident q/k/v: one attention launch, timed."""
+    import numpy as np
+    n, hq = q.shape[2], q.shape[1]
+    rows = (n + 63) // 64
+    causal_tiles = hq * rows * (rows + 1) // 2
+    seqlens = torch.full((1,), n, dtype=torch.int32, device=dev)
     vi, si = gen.vs_index_inputs(hq, n, 1000, 600, seed=300)
     vi_t, si_t = torch.from_numpy(vi).to(dev), torch.from_numpy(np.ascontiguousarray(si)).to(dev)
     bc, bo, cc, ci = M.convert_vertical_slash_indexes(seqlens, vi_t, si_t, n, 64, 64, zero_fill=False)
     tiles = int(bc.sum().item() + ((cc + 63) // 64).sum().item())
     gathered = int(((cc + 63) // 64).sum().item())
-    ms = timed(lambda: M.vertical_slash_attention_from_index(q, k, v, bc, bo, cc, ci, seqlens), 3)
-    out["scattered"] = {"coverage": round(tiles / causal_tiles, 4), "attention_ms": round(ms, 3),
-                        "gathered_tile_share": round(gathered / tiles, 4),
-                        "tflops_on_computed_tiles": round(tiles * TILE_FLOP / ms / 1e9, 1),
-                        "kv_tile_fetch_tbs": round(tiles * 2 * 64 * 128 * 2 / ms / 1e9, 2), "bound": "hbm"}
-    return out
+    ms = _time_steps(torch, lambda: M.vertical_slash_attention_from_index(q, k, v, bc, bo, cc, ci, seqlens), reps, 1)
+    return {"coverage": round(tiles / causal_tiles, 4), "attention_ms": round(ms, 3), "computed_tiles": tiles,
+            "gathered_tile_share": round(gathered / tiles, 4),
+            "tflops_on_computed_tiles": round(tiles * TILE_FLOP / ms / 1e9, 1),
+            "kv_tile_bytes": tiles * 2 * 64 * 128 * 2,
+            "kv_tile_fetch_tbs": round(tiles * 2 * 64 * 128 * 2 / ms / 1e9, 2), "bound": "hbm"}
+
+
+def bench_scattered(args, torch, gen, M, dev):
+    """The scattered-list launch alone (used for the committed counter summary of that case)."""
+    n = args.seq
+    q, k, v, _ = gen.planted_layer(n, 32, 8, seed=100, dtype=torch.bfloat16, sink_logit=3.0, heavy_logit=2.0,
+                                   decay_per_token=0.0)
+    q, k, v = q.to(dev), k.to(dev), v.to(dev)
+    r = measure_scattered(torch, gen, M, dev, q, k, v, args.steps)
+    extra = {}
+    if args.calibrate_copy:
+        src = torch.ones(1 << 28, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        torch.mul(src, 2.0, out=dst)                   # one elementwise kernel: reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        extra["calibrate_copy_bytes_each_way"] = src.numel() * 4
+    print(json.dumps({
+        "metric": "vertical-slash attention ms on scattered lists @128K (config 3's list generator, 600 slashes)",
+        "value": r["attention_ms"], "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": 1,
+        "ms_per_step": r["attention_ms"], "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "scattered lists: 1000 uniform verticals + 600 slashes (0..63 forced, the rest uniform) "
+                               "per head, 32 q / 8 kv heads", "seq_len": n}, **r, **extra}))
 
 
 def main():
@@ -340,11 +375,12 @@ def main():
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--seq", type=int, default=131072)
-    ap.add_argument("--workload", default="vs_c2", choices=["vs_c2", "index_c3", "block_sparse_c4", "llama_c5"],
+    ap.add_argument("--workload", default="vs_c2", choices=["vs_c2", "index_c3", "block_sparse_c4", "llama_c5", "scattered"],
                     help="vs_c2 (default): the headline layer, BASELINE config 2; index_c3: the index "
                          "builder alone on config 3; block_sparse_c4: config 4 (secondary lines, used "
                          "for the committed rocprofv3 summaries); llama_c5: random-init Llama-3-8B "
-                         "prefill of 262144 tokens with config 5's seeded per-head pattern mix")
+                         "prefill of 262144 tokens with config 5's seeded per-head pattern mix; scattered: the "
+                         "attention launch on config 3's scattered lists alone (for its counter summary)")
     ap.add_argument("--layers", type=int, default=32, help="llama_c5: number of decoder layers")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-dense", action="store_true")
@@ -376,6 +412,8 @@ def main():
         return bench_block_sparse_c4(args, torch, gen, M, dev)
     if args.workload == "llama_c5":
         return bench_llama_c5(args, torch, dev)
+    if args.workload == "scattered":
+        return bench_scattered(args, torch, gen, M, dev)
     n, hq, hk = args.seq, 32, 8
     vertical_size, slash_size = 1000, 6096
 

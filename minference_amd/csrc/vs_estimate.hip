@@ -83,12 +83,29 @@ template <> __device__ __forceinline__ f32x16_t mma<_Float16>(const Frag &a, con
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a.h, b.h, c, 0, 0, 0);
 }
 
-// x rounded to the 16-bit input format and back (round to nearest even; fp16 overflows to inf like
-// torch's conversion)
-template <typename T> __device__ __forceinline__ float round_to(float x) { return (float)(T)x; }
-// the score the softmax sees, in the natural-log domain, rounded like the reference's bf16/fp16 torch ops
-template <typename T> __device__ __forceinline__ float ref_logit(float dot, float scale) {
-    return round_to<T>(round_to<T>(dot) * scale);
+// Two values rounded to the 16-bit input format and back (round to nearest even; fp16 overflows to inf
+// like torch's conversion): one packed conversion for the pair, then the two halves are widened again
+// (bf16: a shift and a mask).
+template <typename T> __device__ __forceinline__ void round_pair(float &a, float &b);
+template <> __device__ __forceinline__ void round_pair<__bf16>(float &a, float &b) {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    const bf16x2 p = __builtin_convertvector(f32x2{a, b}, bf16x2);
+    const unsigned u = __builtin_bit_cast(unsigned, p);
+    a = __uint_as_float(u << 16);
+    b = __uint_as_float(u & 0xffff0000u);
+}
+template <> __device__ __forceinline__ void round_pair<_Float16>(float &a, float &b) {
+    a = (float)(_Float16)a;
+    b = (float)(_Float16)b;
+}
+// the scores the softmax sees, in the natural-log domain, rounded like the reference's bf16/fp16 torch
+// ops: round(round(q.k) * sm_scale)
+template <typename T> __device__ __forceinline__ void ref_logit_pair(float &a, float &b, float scale) {
+    round_pair<T>(a, b);
+    a *= scale;
+    b *= scale;
+    round_pair<T>(a, b);
 }
 constexpr float LOG2E = 1.4426950408889634f;
 
@@ -245,7 +262,11 @@ __global__ __launch_bounds__(EST_THREADS, 3) void est_stats_kernel(const EstPara
 #pragma unroll
             for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) st[nb][r] = ref_logit<T>(st[nb][r], p.scale);
+                for (int r = 0; r < 16; r += 2) {
+                    float a = st[nb][r], b = st[nb][r + 1];
+                    ref_logit_pair<T>(a, b, p.scale);
+                    st[nb][r] = a; st[nb][r + 1] = b;
+                }
         }
 #pragma unroll
         for (int nb = 0; nb < 2; ++nb) {
@@ -436,11 +457,17 @@ __global__ __launch_bounds__(EST_THREADS, 2) void est_scores_kernel(const EstPar
             for (int r = 0; r < 16; ++r) sc[r] = 0.f;
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) sc = mma<T>(qf[mb][ks], kf[ks], sc);
+            if constexpr (RR) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                if constexpr (RR) pr[mb][r] = __builtin_amdgcn_exp2f(fmaf(ref_logit<T>(sc[r], p.scale), LOG2E, -mrow[mb][r]));
-                else pr[mb][r] = __builtin_amdgcn_exp2f(fmaf(sc[r], p.scale_log2, -mrow[mb][r]));
+                for (int r = 0; r < 16; r += 2) {
+                    float a = sc[r], b = sc[r + 1];
+                    ref_logit_pair<T>(a, b, p.scale);
+                    sc[r] = a; sc[r + 1] = b;
+                }
             }
+            const float sl2 = RR ? LOG2E : p.scale_log2;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) pr[mb][r] = __builtin_amdgcn_exp2f(fmaf(sc[r], sl2, -mrow[mb][r]));
         }
         if (edge) {      // (a block of its own, kept one by the empty asm: merged into the straight-line code
                          // the 32 compares and selects would run for every block)
