@@ -269,29 +269,27 @@ __host__ __device__ __forceinline__ long long idx_tab_ints(int nnz_s, int rows) 
     return IDX_TAB_HDR + 7ll * nnz_s + idx_bm_words(rows);
 }
 
-__global__ __launch_bounds__(MINF_WAVE) void vs_index_prep_kernel(const int32_t *__restrict__ slash,
-                                                                  int32_t *__restrict__ tables, int nnz_s, int rows) {
+// The walk of chunks [c_begin, c_end) of one head's list by one wavefront, starting from the state
+// (cur_a, carried_e, carried_t) that the entries before chunk c_begin leave behind and from the
+// counts (nb, nr, ng) of blocks, ranges and gap entries before it.  WRITE = false only counts.
+struct PrepState { int cur_a, carried_e, carried_t; };
+template <bool WRITE>
+__device__ __forceinline__ void prep_walk(const int32_t *__restrict__ sl, int32_t *__restrict__ hdr, int nnz_s, int V,
+                                          int c_begin, int c_end, PrepState &st, int &nb, int &nr, int &ng) {
     const int lane = minf_lane();
-    const long long bh = blockIdx.x;
-    const int32_t *sl = slash + bh * (long long)nnz_s;
-    int32_t *hdr = tables + bh * idx_tab_ints(nnz_s, rows);
     int32_t *cpos = hdr + IDX_TAB_HDR, *cpre = cpos + nnz_s, *crun = cpre + nnz_s;
     int32_t *run_a = crun + nnz_s, *run_e = run_a + nnz_s, *cgaps = run_e + nnz_s;
-    const int V = sl[0] + 64;
-
-    int nb = 0, nr = 0, ng = 0;
-    int carried_e = 0, carried_t = 0, cur_a = 0;
-    const int nchunks = (nnz_s + MINF_WAVE - 1) / MINF_WAVE;
+    int carried_e = st.carried_e, carried_t = st.carried_t, cur_a = st.cur_a;
     // the walk is one chain of chunks; the list entries of the next two chunks are fetched ahead so
     // that no chunk waits for a load
-    int o_next = sl[min(lane, nnz_s - 1)], o_next2 = sl[min(MINF_WAVE + lane, nnz_s - 1)];
-    for (int c = 0; c < nchunks; ++c) {
+    int o_next = sl[min(c_begin * MINF_WAVE + lane, nnz_s - 1)], o_next2 = sl[min((c_begin + 1) * MINF_WAVE + lane, nnz_s - 1)];
+    for (int c = c_begin; c < c_end; ++c) {
         const int base = c * MINF_WAVE;
         const int cnt = min(MINF_WAVE, nnz_s - base);
         const bool valid = lane < cnt;
         const int o_cur = o_next;
         o_next = o_next2;
-        o_next2 = sl[min(base + 3 * MINF_WAVE + lane - MINF_WAVE, nnz_s - 1)];
+        o_next2 = sl[min(base + 2 * MINF_WAVE + lane, nnz_s - 1)];
         int t = valid ? max(V - o_cur, 64) : 0;
         const int tlast = minf_readlane(t, cnt - 1);
         if (!valid) t = tlast;
@@ -303,7 +301,7 @@ __global__ __launch_bounds__(MINF_WAVE) void vs_index_prep_kernel(const int32_t 
         }
         uint64_t starts, gm;
         const int a = chunk_ranges(t, lane, cur_a, carried_e, carried_t, starts, &gm);
-        if (valid) cgaps[base + lane] = ng + __builtin_popcountll(gm & (minf_lanemask_lt() | (1ull << lane)));
+        if (WRITE && valid) cgaps[base + lane] = ng + __builtin_popcountll(gm & (minf_lanemask_lt() | (1ull << lane)));
         ng += __builtin_popcountll(gm);             // (padding lanes repeat the last entry: never a gap)
         const bool is_start = valid && (((starts >> lane) & 1ull) || (c == 0 && lane == 0));
         const int e = a + ((((t - a) + 63) >> 6) << 6);
@@ -311,16 +309,18 @@ __global__ __launch_bounds__(MINF_WAVE) void vs_index_prep_kernel(const int32_t 
         if (lane == 0) eprev = carried_e;
         const bool changed = valid && (e != eprev);
         const uint64_t cm = __ballot(changed), sm = __ballot(is_start);
-        const uint64_t lt = minf_lanemask_lt();
-        const int kpos = nb + __builtin_popcountll(cm & lt);
-        if (changed) cpos[kpos] = e - 64;
-        if (valid) {
-            const int r = nr + __builtin_popcountll(sm & lt);
-            cpre[base + lane] = is_start ? kpos : -1;
-            crun[base + lane] = is_start ? r : -1;
-            if (is_start) {
-                run_a[r] = a;
-                if (r > 0) run_e[r - 1] = eprev;
+        if (WRITE) {
+            const uint64_t lt = minf_lanemask_lt();
+            const int kpos = nb + __builtin_popcountll(cm & lt);
+            if (changed) cpos[kpos] = e - 64;
+            if (valid) {
+                const int r = nr + __builtin_popcountll(sm & lt);
+                cpre[base + lane] = is_start ? kpos : -1;
+                crun[base + lane] = is_start ? r : -1;
+                if (is_start) {
+                    run_a[r] = a;
+                    if (r > 0) run_e[r - 1] = eprev;
+                }
             }
         }
         nb += __builtin_popcountll(cm);
@@ -329,15 +329,112 @@ __global__ __launch_bounds__(MINF_WAVE) void vs_index_prep_kernel(const int32_t 
         carried_t = tlast;
         cur_a = minf_readlane(a, cnt - 1);
     }
-    if (lane == 0) {
-        run_e[nr - 1] = carried_e;
-        hdr[0] = nb;
-        hdr[1] = nr;
-        hdr[2] = V;
-        // the bitmap covers positions [0, 32 * bm_words); a list whose largest offset lies far
-        // outside the context does not fit and the row blocks fall back to searching the ranges
-        hdr[3] = (long long)V <= 32 * (idx_bm_words(rows) - 1) ? 1 : 0;
-        hdr[4] = ng;
+    st.cur_a = cur_a; st.carried_e = carried_e; st.carried_t = carried_t;
+}
+
+__device__ __forceinline__ void prep_header(int32_t *hdr, int nnz_s, int rows, int V, const PrepState &st, int nb, int nr, int ng) {
+    int32_t *run_e = hdr + IDX_TAB_HDR + 4ll * nnz_s;
+    run_e[nr - 1] = st.carried_e;
+    hdr[0] = nb;
+    hdr[1] = nr;
+    hdr[2] = V;
+    // the bitmap covers positions [0, 32 * bm_words); a list whose largest offset lies far
+    // outside the context does not fit and the row blocks fall back to searching the ranges
+    hdr[3] = (long long)V <= 32 * (idx_bm_words(rows) - 1) ? 1 : 0;
+    hdr[4] = ng;
+}
+
+// The table pass: one workgroup of PREP_WAVES wavefronts per head.  The walk over the list is a chain
+// (which range an entry belongs to depends on where the ranges before it started), but an entry more
+// than 127 above its predecessor starts a range whatever came before ("sure" start) and only entries
+// 65..127 above their predecessor ("maybe") depend on the 64-phase of the current range.  So every
+// wavefront takes a contiguous share of the chunks; all of them first mark the sure and maybe entries
+// of their chunks (independent work); a wavefront then finds the state at the head of its share by
+// going back to the last sure start before it and replaying only the maybe entries in between (none
+// inside a dense run, a handful when the offsets are scattered); it walks its share once to count its
+// blocks, ranges and gap entries, the counts are summed over the wavefronts before it, and it walks
+// the share again to write the tables.  Lists of at most two chunks, or of more chunks than the mark
+// arrays hold, are walked by one wavefront alone.
+#define PREP_WAVES 16
+#define PREP_MAX_CHUNKS 2048
+__global__ __launch_bounds__(PREP_WAVES *MINF_WAVE) void vs_index_prep_kernel(const int32_t *__restrict__ slash,
+                                                                              int32_t *__restrict__ tables, int nnz_s, int rows) {
+    __shared__ uint64_t sure_m[PREP_MAX_CHUNKS], maybe_m[PREP_MAX_CHUNKS];
+    __shared__ int cnt_b[PREP_WAVES], cnt_r[PREP_WAVES], cnt_g[PREP_WAVES];
+    const int lane = minf_lane();
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const long long bh = blockIdx.x;
+    const int32_t *sl = slash + bh * (long long)nnz_s;
+    int32_t *hdr = tables + bh * idx_tab_ints(nnz_s, rows);
+    const int V = sl[0] + 64;
+    const int nchunks = (nnz_s + MINF_WAVE - 1) / MINF_WAVE;
+
+    if (nchunks <= 2 || nchunks > PREP_MAX_CHUNKS) {        // (workgroup-uniform)
+        if (wave == 0) {
+            PrepState st{0, 0, 0};
+            int nb = 0, nr = 0, ng = 0;
+            prep_walk<true>(sl, hdr, nnz_s, V, 0, nchunks, st, nb, nr, ng);
+            if (lane == 0) prep_header(hdr, nnz_s, rows, V, st, nb, nr, ng);
+        }
+        return;
+    }
+    const int per = (nchunks + PREP_WAVES - 1) / PREP_WAVES;
+    const int c0 = wave * per, c1 = min(c0 + per, nchunks);
+    // ---- marks: entry i is a sure start when t_i > t_{i-1} + 127, a maybe when t_i > t_{i-1} + 64
+    // (entry 0 starts the first range)
+    for (int c = c0; c < c1; ++c) {
+        const int i = c * MINF_WAVE + lane;
+        const bool valid = i < nnz_s;
+        const int t = max(V - sl[min(i, nnz_s - 1)], 64);
+        const int tp = max(V - sl[min(max(i - 1, 0), nnz_s - 1)], 64);
+        const bool sure = valid && (i == 0 || t > tp + 127);
+        const bool maybe = valid && !sure && t > tp + 64;
+        const uint64_t sm = __ballot(sure), mm = __ballot(maybe);
+        if (lane == 0) { sure_m[c] = sm; maybe_m[c] = mm; }
+    }
+    __syncthreads();
+    // ---- the state at the head of this wavefront's share (wave-uniform scalar work)
+    PrepState st{0, 0, 0};
+    if (c0 > 0 && c0 < nchunks) {
+        int cs = c0 - 1;
+        while (cs > 0 && sure_m[cs] == 0) --cs;              // (chunk 0 holds entry 0, a sure start)
+        const uint64_t smask = sure_m[cs];
+        const int js = cs * MINF_WAVE + (63 - __builtin_clzll(smask));     // the last sure start before the share
+        int a = max(V - sl[js], 64) - 64;
+        for (int c = cs; c < c0; ++c) {
+            uint64_t mm = maybe_m[c];
+            if (c == cs) mm &= ~((2ull << (js - cs * MINF_WAVE)) - 1ull);    // maybes above the sure start only
+            while (mm) {
+                const int j = c * MINF_WAVE + __builtin_ctzll(mm);
+                mm &= mm - 1;
+                const int tj = max(V - sl[j], 64), tp = max(V - sl[j - 1], 64);
+                const int ep = a + ((((tp - a) + 63) >> 6) << 6);
+                if (tj > ep + 64) a = tj - 64;
+            }
+        }
+        st.cur_a = a;
+        st.carried_t = max(V - sl[c0 * MINF_WAVE - 1], 64);
+        st.carried_e = a + ((((st.carried_t - a) + 63) >> 6) << 6);
+    }
+    // ---- count, sum over the wavefronts before this one, write
+    int nb = 0, nr = 0, ng = 0;
+    if (c0 < nchunks) {
+        PrepState probe = st;
+        prep_walk<false>(sl, hdr, nnz_s, V, c0, c1, probe, nb, nr, ng);
+    }
+    if (lane == 0) { cnt_b[wave] = nb; cnt_r[wave] = nr; cnt_g[wave] = ng; }
+    __syncthreads();
+    int ob = 0, orr = 0, og = 0, tb = 0, tr = 0, tg = 0;
+#pragma unroll
+    for (int w = 0; w < PREP_WAVES; ++w) {
+        const int b = cnt_b[w], r = cnt_r[w], g = cnt_g[w];
+        if (w < wave) { ob += b; orr += r; og += g; }
+        tb += b; tr += r; tg += g;
+    }
+    if (c0 < nchunks) {
+        nb = ob; nr = orr; ng = og;
+        prep_walk<true>(sl, hdr, nnz_s, V, c0, c1, st, nb, nr, ng);
+        if (c1 == nchunks && lane == 0) prep_header(hdr, nnz_s, rows, V, st, tb, tr, tg);
     }
 }
 
@@ -661,7 +758,7 @@ static int index_build_tables(const int32_t *seqlens, const int32_t *vertical_id
                               hipStream_t stream) {
     const long long nblk = (total + IDX_WAVES - 1) / IDX_WAVES;
     if (nblk > 0x7fffffffLL || (long long)batch * heads > 65535) return MINF_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL(vs_index_prep_kernel, dim3((unsigned)(batch * heads)), dim3(MINF_WAVE), 0,
+    hipLaunchKernelGGL(vs_index_prep_kernel, dim3((unsigned)(batch * heads)), dim3(PREP_WAVES * MINF_WAVE), 0,
                        stream, slash_idx, workspace, nnz_s, rows);
     int status = minf_launch_status();
     if (status != MINF_OK) return status;
