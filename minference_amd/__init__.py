@@ -30,4 +30,4 @@ __all__ = [
     "tri_mix_forward", "tri_mix_minference_forward", "dilated_forward", "static_vertical_slash_forward",
     "a_shape_kernel", "tri_shape_kernel", "minference_patch", "patch_hf", "get_support_models",
 ]
-__version__ = "0.1.0"
+__version__ = "0.3.0"

@@ -102,6 +102,46 @@ def test_structured_lists_all_rows(gpu, mode):
         assert_same(run_gpu([seqlen], v, s, n, gpu), ref)
 
 
+@pytest.mark.parametrize("kind", ["maybe chains", "two or three chunks", "more chunks than the marks hold"])
+def test_table_pass_shares_of_the_list(gpu, kind):
+    """The table pass cuts a head's list into shares for 16 wavefronts; a wavefront finds the state at
+    the head of its share by replaying the "maybe" entries (65..127 above their predecessor) since
+    the last "sure" start (more than 127 above).  Lists built to stress that: hundreds of entries in
+    a row whose gaps are all 65..127 (no sure start for whole shares, so the replay crosses several
+    of them), lists of two chunks (walked by one wavefront) and three (shared), and a list of more
+    chunks than the mark arrays hold (walked by one wavefront).  Bit-exact against the C oracle and
+    against the plain wave-per-row builder."""
+    rng = np.random.default_rng(len(kind))
+    cases = []
+    if kind == "maybe chains":
+        for trial in range(3):
+            steps = rng.choice([65, 66, 100, 126, 127, 128, 1, 64], size=5000,
+                               p=[0.25, 0.1, 0.3, 0.1, 0.15, 0.02 * trial, 0.05, 0.05 - 0.02 * trial])
+            sl = np.concatenate([[0], np.cumsum(steps)])
+            n = int(sl[-1]) + 100
+            cases.append((n, sl[::-1], np.sort(rng.choice(n, size=300, replace=False))))
+    elif kind == "two or three chunks":
+        for S in (65, 127, 128, 129, 191, 192, 193):
+            steps = rng.choice([1, 2, 64, 65, 127, 128, 300], size=S - 1)
+            sl = np.concatenate([[0], np.cumsum(steps)])
+            n = int(sl[-1]) + 70
+            cases.append((n, sl[::-1], np.sort(rng.choice(n, size=min(n, 90), replace=False))))
+    else:
+        S = 2049 * 64 + 5
+        steps = rng.choice([1, 66, 130], size=S - 1, p=[0.999, 0.0005, 0.0005])
+        sl = np.concatenate([[0], np.cumsum(steps)])
+        n = int(sl[-1]) + 200
+        sl = sl[sl < n]
+        assert sl.size > 2048 * 64
+        cases.append((n, sl[::-1], np.sort(rng.choice(n, size=500, replace=False))))
+    for n, sl, vt in cases:
+        s = np.ascontiguousarray(sl[None, None].astype(np.int32))
+        v = np.ascontiguousarray(vt[None, None].astype(np.int32))
+        print(f"case table pass: {kind} n={n} S={s.shape[-1]} V={v.shape[-1]}", flush=True)
+        ref = O.vs_index_build([n], v, s, n)
+        assert_same(run_gpu([n], v, s, n, gpu), ref)
+
+
 def test_hand_kat(gpu):
     V = np.array([[[0, 1, 2, 3, 100, 130, 700]]], np.int32)
     S = np.array([[[500, 70, 64, 3, 0]]], np.int32)
