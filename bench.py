@@ -325,6 +325,37 @@ def sensitivity_lines(args, torch, gen, M, dev, n, hq, hk):
     return out
 
 
+def sibling_list_overlap(bc, bo, group, samples=96, seed=0):
+    """How many block-list entries neighbouring row blocks and GQA sibling heads have in common, on
+    sampled row-block pairs of sampled kv groups (numpy set intersections on the host).  Block starts
+    follow each head's own largest offset of a merged range, so sibling heads rarely land on the
+    same 64-key blocks even where they cover the same keys: a K/V tile can be shared by the two row
+    blocks of a head, hardly ever by two heads."""
+    import numpy as np
+    bcn = bc[0].cpu().numpy()
+    heads, rows = bcn.shape
+    width = int(bcn.max())
+    rng = np.random.default_rng(seed)
+    pairs = rng.choice(rows // 2, size=min(samples, rows // 2), replace=False)
+    groups = list(range(0, heads // group, max(1, heads // group // 3)))[:3]
+    acc = {"entries": [], "both_row_blocks": [], "two_siblings": [], "all_siblings": []}
+    for g in groups:
+        sub = bo[0, g * group:(g + 1) * group, :, :width].cpu().numpy()
+        for mp in pairs:
+            lists = [[set(sub[h, m, :bcn[g * group + h, m]].tolist()) for m in (2 * mp, 2 * mp + 1)] for h in range(group)]
+            acc["entries"].append(len(lists[0][0]))
+            acc["both_row_blocks"].append(len(lists[0][0] & lists[0][1]))
+            if group >= 2:
+                acc["two_siblings"].append(len(lists[0][0] & lists[0][1] & lists[1][0] & lists[1][1]))
+                allc = lists[0][0]
+                for h in range(group):
+                    allc = allc & lists[h][0] & lists[h][1]
+                acc["all_siblings"].append(len(allc))
+    out = {key: round(float(np.mean(val)), 2) for key, val in acc.items() if val}
+    out["sample"] = f"{len(pairs)} row-block pairs x {len(groups)} kv groups"
+    return out
+
+
 def measure_scattered(torch, gen, M, dev, q, k, v, reps):
     """The index lists of BASELINE config 3's generator at q's length with 600 slashes (0..63 forced,
     the rest uniform) and 1000 uniform verticals, on resident q/k/v: one attention launch, timed."""
@@ -507,6 +538,7 @@ def main():
 
     traffic = committed_traffic() if n == 131072 else None
     if not args.no_sensitivity:
+        extra["block_list_overlap"] = sibling_list_overlap(bc, bo, hq // hk)
         del out
         torch.cuda.empty_cache()
         # the same launch (same lists, same instruction stream) on all-zero operands: the chip lowers its

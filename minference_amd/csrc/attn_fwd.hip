@@ -265,33 +265,36 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
     // XCD one contiguous range of the logical order (batch, kv head, row block,
     // query head inside the GQA group) so that the row blocks and the query
     // heads that share K/V also share an L2.
-    const long long per_xcd = (p.total_wg + 7) >> 3;
-    const long long logical = (long long)(blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    if (logical >= p.total_wg) return false;
+    // (32-bit arithmetic: the launcher refuses grids beyond 2^31 workgroups, and 64-bit divisions of
+    // wave-uniform values cost a thousand scalar instructions per workgroup here)
+    const unsigned total_wg = (unsigned)p.total_wg;
+    const unsigned per_xcd = (total_wg + 7u) >> 3;
+    const unsigned logical = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
+    if (logical >= total_wg) return false;
     const int group = p.hq / p.hk;
-    long long rest = logical;
-    const int hin = (int)(rest % group); rest /= group;
+    unsigned rest = logical;
+    const int hin = (int)(rest % (unsigned)group); rest /= (unsigned)group;
     // Dense causal work grows with the row block, so the heavy (late) blocks go first.  The sparse
     // modes have near-constant work per row block once the context is long and then measure 1 %
     // faster in ascending order; up to 64K tokens their early row blocks are still growing and the
     // descending order wins for vertical-slash lists (+4 % at 16K, +1.7 % at 32K): the launcher picks.
     const int rows_wg = (p.rows + 1) >> 1;                           // row-block pairs per (batch, head)
-    const int mi = (int)(rest % rows_wg); rest /= rows_wg;
+    const int mi = (int)(rest % (unsigned)rows_wg); rest /= (unsigned)rows_wg;
     const int mslot = p.descending ? rows_wg - 1 - mi : mi;
     int hkv, b, h, hs;                               // hs: head position in the index tensors
     if (p.head_list) {
         // the selected heads in chunks of `group` consecutive list entries take the place of the kv
         // groups: neighbours in the (ascending) list mostly share a kv head
         const int nch = (p.index_heads + group - 1) / group;
-        const int ch = (int)(rest % nch);
-        b = (int)(rest / nch);
+        const int ch = (int)(rest % (unsigned)nch);
+        b = (int)(rest / (unsigned)nch);
         hs = ch * group + hin;
         if (hs >= p.index_heads) return false;       // padding of the last chunk (workgroup-uniform)
         h = as_const(p.head_list)[hs];
         hkv = h / group;
     } else {
-        hkv = (int)(rest % p.hk);
-        b = (int)(rest / p.hk);
+        hkv = (int)(rest % (unsigned)p.hk);
+        b = (int)(rest / (unsigned)p.hk);
         h = hkv * group + hin;
         hs = h;
     }
