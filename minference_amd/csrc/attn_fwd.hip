@@ -60,6 +60,7 @@
 //  * the epilogue transposes O^T through LDS so each global store is 16 B of one 256-byte row.
 #include "minf_common.h"
 #include <math.h>
+#include <string.h>
 #include <type_traits>
 
 namespace {
@@ -922,8 +923,22 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
         const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
         // pitch: 8-byte lane writes spread over all banks (four waves only fit without the pad)
         constexpr int OP = ROW_BYTES;
-        // a row sum at 2^100 or beyond (or no number at all): some probability may have overflowed
-        if (!every_max && __any(!(l_tot < 0x1p100f)) && lane == 0) lds_redo = 1;
+        // a row sum at 2^100 or beyond (or infinite, or no number at all): some probability may have
+        // overflowed.  Compared on the bit pattern: the library is compiled without NaN semantics, which
+        // lets the compiler turn !(l < x) into l >= x -- false for the NaN that inf * 0 leaves in a
+        // row sum when the maximum is raised after an overflow
+        // ... and an accumulator that is infinite or no number: O^T sums twice as many terms per tile
+        // as a lane's share of the row sum (and terms scaled by |v|), so it can overflow while the row
+        // sum still fits, and a later rescale then hides the size of the sum but not the inf / NaN
+        if constexpr (!every_max) {
+            unsigned obits = 0;
+#pragma unroll
+            for (int i = 0; i < NDB; ++i)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) obits = max(obits, __float_as_uint(oacc[i][r]) & 0x7fffffffu);
+            const bool suspect = (__float_as_uint(l_tot) & 0x7fffffffu) >= __float_as_uint(0x1p100f) || obits >= 0x7f800000u;
+            if (__any(suspect) && lane == 0) lds_redo = 1;
+        }
         __syncthreads();                                  // K/V tiles no longer needed
         char *ot = (half ? lds_v : lds_k) + wave * 32 * OP;    // 32 rows per wave
         const bool live = qrow < seqlen;
@@ -1087,7 +1102,10 @@ extern "C" int minf_trishape_attn_fwd(const minf_qkvo *t, int n_init, int n_loca
                                       float sm_scale_last, void *stream) {
     int st = check_tensors(t, true);
     if (st) return st;
-    if (n_init < 0 || n_local < 1 || n_last < 0 || !(sm_scale_last >= 0.f)) return MINF_ERR_INVALID_ARG;
+    uint32_t scale_bits;
+    memcpy(&scale_bits, &sm_scale_last, sizeof(scale_bits));          // (negative, infinite or NaN: refused)
+    if (n_init < 0 || n_local < 1 || n_last < 0 || (scale_bits >> 31) || (scale_bits & 0x7f800000u) == 0x7f800000u)
+        return MINF_ERR_INVALID_ARG;
     AttnParams p;
     fill_params(p, t);
     if (sm_scale_last > 0.f) p.scale_log2_dense = sm_scale_last * 1.4426950408889634f;

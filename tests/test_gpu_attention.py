@@ -467,6 +467,42 @@ def test_ragged_seqlens_in_a_batch(gpu):
             assert err.max() <= MAX_ABS and err.mean() <= MEAN_ABS, (b, h, err.max())
 
 
+@pytest.mark.parametrize("mult,n", [(20, 8192), (8, 16384)])
+def test_scores_rising_steadily_past_the_fp32_range(gpu, mult, n):
+    """Scores that grow with the key position by more than the whole fp32 exponent range over a row
+    (113 natural-log units = 163 powers of two between the sink keys and the latest keys at mult 20),
+    so that a walk which starts at the sink tiles and looks at the row maximum only every eighth tile
+    overflows: first to inf, and at the next maximum to inf * 0 = NaN in the running row sum.  The row
+    sum check at the end of the walk has to catch both (it compares bit patterns: the library is
+    built without NaN semantics) and the walk is run again with the maximum of every tile.  Every
+    operator, every row: finite, V = 1 gives exactly 1, and the fp32 oracle within tolerance."""
+    import minference_amd as M
+    from minference_amd.ops import _build_block_index
+    hq, hk = 2, 1
+    print(f"case rising scores mult={mult} n={n}", flush=True)
+    q, k, v, _ = gen.planted_layer(n, hq, hk, seed=100, dtype=torch.bfloat16,
+                                   decay_per_token=mult * 2.0 ** -7 / 128 ** 0.5)
+    qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
+    ones = torch.ones_like(vg)
+    ke, ve = expand(k, hq), expand(v, hq)
+    bi = _build_block_index(qg, kg, 16, force_diag_first=True)
+    v_idx, s_idx = M.estimate_vertical_slash(qg, kg, 100, 300)
+    runs = {
+        "block-sparse": (lambda vv: M.block_sparse_attention_from_index(qg, kg, vv, bi),
+                         lambda: torch.stack([O.masked_attention(q[0, h], ke[0, h], ve[0, h], O.bs_mask(bi[0, h].cpu().numpy(), n))
+                                              for h in range(hq)])[None]),
+        "a-shape": (lambda vv: M.streaming_forward(qg, kg, vv, 128, 1024), lambda: O.streaming_forward(q, ke, ve, 128, 1024)),
+        "vertical-slash": (lambda vv: M.vertical_slash_sparse_attention(qg, kg, vv, v_idx, s_idx),
+                           lambda: O.vertical_slash_sparse_attention(q, ke, ve, v_idx.cpu(), s_idx.cpu())),
+        "dense": (lambda vv: M.dense_causal_attention(qg, kg, vv), lambda: sdpa_causal(q, ke, ve)),
+    }
+    for name, (f, ref) in runs.items():
+        o1 = f(ones).float()
+        assert torch.isfinite(o1).all(), f"{name}: non-finite rows with V = 1"
+        assert (o1 - 1.0).abs().max().item() <= 2.0 ** -8, name
+        check(f(vg), ref(), f"rising {name}")
+
+
 @pytest.mark.parametrize("n", [1, 37, 63, 65])
 def test_tiny_sequences_all_operators(gpu, n):
     import minference_amd as M

@@ -346,3 +346,43 @@ def test_config4_block_sets_follow_the_reference_rounding(gpu):
               f"(fp32 arithmetic: mean {np.mean(rec32):.4f} min {np.min(rec32):.4f}); rows breaking the rule: {bad}", flush=True)
         assert bad == 0
         assert np.mean(rec) >= 0.99
+
+
+def test_full_size_rows_are_normalised_and_linear_in_v(gpu):
+    """Size-independent properties on EVERY row of every head at BASELINE's full shapes (the oracle
+    comparisons above sample row blocks): with V = 1 every output row is a weighted mean of ones, i.e.
+    exactly 1 wherever a row attends to anything -- numerator and denominator are sums of the same
+    rounded probabilities -- for the vertical-slash path (config 2: 131072 tokens, 32 q / 8 kv heads),
+    the block-sparse path (config 4) and the A-shape path (config 5's 128 + 4096); and the output is
+    linear in V: out(V1 + V2) = out(V1) + out(V2) within the 16-bit rounding of the three outputs."""
+    import minference_amd as M
+    from minference_amd.ops import _build_block_index, block_sparse_attention_from_index
+    n, hq, hk = 131072, 32, 8
+    q, k, v, _ = gen.planted_layer(n, hq, hk, seed=100, dtype=torch.bfloat16)
+    qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
+    ones = torch.ones_like(vg)
+    seqlens = torch.full((1,), n, dtype=torch.int32, device=gpu)
+    v_idx, s_idx = M.estimate_vertical_slash(qg, kg, 1000, 6096)
+    idx = M.convert_vertical_slash_indexes(seqlens, v_idx, s_idx, n, 64, 64, zero_fill=False)
+    bi = _build_block_index(qg, kg, 100, force_diag_first=True)
+    runs = {
+        "vertical-slash": lambda vv: M.vertical_slash_attention_from_index(qg, kg, vv, *idx, seqlens),
+        "block-sparse": lambda vv: block_sparse_attention_from_index(qg, kg, vv, bi),
+        "a-shape": lambda vv: M.streaming_forward(qg, kg, vv, 128, 4096),
+    }
+    g = torch.Generator().manual_seed(7)
+    v2 = torch.randn(v.shape, generator=g).to(torch.bfloat16).to(gpu)
+    for name, f in runs.items():
+        print(f"case full-size properties: {name}", flush=True)
+        o1 = f(ones)
+        dev = (o1.float() - 1.0).abs().max().item()
+        print(f"  V = 1: max |out - 1| = {dev:.3e}", flush=True)
+        assert dev <= 2.0 ** -8, name                      # half a unit of bf16 at 1.0
+        del o1
+        oa, ob, oab = f(vg), f(v2), f(vg + v2)
+        d = (oab.float() - oa.float() - ob.float()).abs()
+        scale = oab.float().abs().max().item()
+        print(f"  linearity: max {d.max().item():.3e} mean {d.mean().item():.3e} (max |out| {scale:.3e})", flush=True)
+        # three bf16 roundings of outputs of size <= scale, plus the rounding of V1 + V2 itself
+        assert d.max().item() <= 3e-2 * max(scale, 1.0) and d.mean().item() <= 2e-3 * max(scale, 1.0), name
+        del oa, ob, oab
