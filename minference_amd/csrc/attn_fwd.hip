@@ -601,6 +601,8 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
         for (int r = 0; r < 16; ++r) oacc[i][r] = 0.f;
     float m_i = -INFINITY;   // running max (log2 domain, scaled)
     int sm_steps = 0;        // tiles this wave has put through the softmax
+    int sm_prev_start = -(1 << 30);   // first key of the previous one (wave-uniform)
+    bool sm_prev_masked = false;      // ... and whether it was a boundary tile (some rows may have seen none of its keys)
     float l_i = 0.f;         // this lane's share of the running sum
 
     // LDS read addresses that do not depend on the tile
@@ -715,7 +717,15 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
         // and for every tile of a walk that is run again because a row sum left the safe range (which
         // takes a row whose scores rise by more than a hundred powers of two within MAX_PERIOD tiles).
         float alpha = 1.0f, m_use = m_i;
-        if (every_max || ((sm_steps++ & (MAX_PERIOD - 1)) == 0) || __any(m_i == -INFINITY)) {
+        // ... and wherever the walk jumps (the first tile of a run of blocks, the first window tile after
+        // the sink tiles, every gathered tile): scores move smoothly along a run of neighbouring keys
+        // but may differ by any amount across a jump.  A tile after a masked one counts as a jump too:
+        // a row that saw none of the masked tile's keys (the window starts a tile later for the last
+        // rows of a row block) still carries the maximum from before the jump.
+        const bool jump = (MODE == MODE_VS && cur.gathered) || cur.start != sm_prev_start + BN || sm_prev_masked;
+        sm_prev_start = cur.start;
+        sm_prev_masked = need_mask;
+        if (every_max || ((sm_steps++ & (MAX_PERIOD - 1)) == 0) || jump || __any(m_i == -INFINITY)) {
         float mx;
         {
             // four independent chains of three-operand maxima (8 scores each)
