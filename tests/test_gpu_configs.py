@@ -386,3 +386,51 @@ def test_full_size_rows_are_normalised_and_linear_in_v(gpu):
         # three bf16 roundings of outputs of size <= scale, plus the rounding of V1 + V2 itself
         assert d.max().item() <= 3e-2 * max(scale, 1.0) and d.mean().item() <= 2e-3 * max(scale, 1.0), name
         del oa, ob, oab
+
+
+def test_full_size_estimation_and_selection_invariants(gpu):
+    """BASELINE config 2's shape, all 32 heads: the score vectors of the estimation are two
+    decompositions of the same 64 softmax rows, so each sums to 64 before forcing (both rounding modes);
+    the selected lists are strictly ordered, inside the context and contain the forced entries
+    (first 30 columns, offsets 0..99: minference_forward.py:606, :610)."""
+    import minference_amd as M
+    from minference_amd.estimate import vertical_slash_scores
+    n, hq, hk = 131072, 32, 8
+    q, k, _, _ = gen.planted_layer(n, hq, hk, seed=100, dtype=torch.bfloat16)
+    qg, kg = q.to(gpu), k.to(gpu)
+    for rounded in (True, False):
+        vert, slash = vertical_slash_scores(qg, kg, force_vertical=0, force_slash=0, reference_rounding=rounded)
+        sv, ss = vert.double().sum(-1), slash.double().sum(-1)
+        print(f"case c2 estimation sums rounded={rounded}: vertical {sv.min().item():.4f}..{sv.max().item():.4f} "
+              f"slash {ss.min().item():.4f}..{ss.max().item():.4f}", flush=True)
+        assert torch.isfinite(vert).all() and torch.isfinite(slash).all()
+        assert (sv - 64).abs().max() <= 2e-2 and (ss - 64).abs().max() <= 2e-2
+        assert (vert >= 0).all() and (slash >= 0).all()
+    v_idx, s_idx = M.estimate_vertical_slash(qg, kg, 1000, 6096)
+    vi, si = v_idx[0].cpu().numpy(), s_idx[0].cpu().numpy()
+    assert vi.shape == (hq, 1000) and si.shape == (hq, 6096)
+    assert (np.diff(vi, axis=-1) > 0).all() and (np.diff(si, axis=-1) < 0).all()
+    assert vi.min() >= 0 and vi.max() < n and si.min() >= 0 and si.max() < n
+    assert (vi[:, :30] == np.arange(30)).all() and (si[:, -100:] == np.arange(99, -1, -1)).all()
+
+
+def test_config5_layer_slice_every_row_is_normalised(gpu):
+    """BASELINE config 5's attention layer (262144 tokens, 32 q / 8 kv heads, the seeded 70/20/10
+    table of layer 0: vertical_and_slash, block_sparse and stream_llm heads) through the per-head
+    dispatcher with V = 1: every output row of every head must be exactly 1, whichever kernel and
+    list its head took -- the planted inputs' scores span 260 powers of two between the sink keys and
+    the latest keys at this length, more than fp32's exponent range."""
+    import minference_amd as M
+    from minference_amd.llama import seeded_pattern_mix
+    n, hq, hk = 262144, 32, 8
+    q, k, v, _ = gen.planted_layer(n, hq, hk, seed=100, dtype=torch.bfloat16)
+    qg, kg = q.to(gpu), k.to(gpu)
+    del q, v
+    ones = torch.ones_like(kg)
+    table = seeded_pattern_mix(1, hq, seed=501)
+    print("case c5 layer slice, V = 1", flush=True)
+    out = M.minference_prefill_forward(qg, kg, ones, {"layer_idx": 0, "attn_forward_config": {"best_pattern": table}})
+    torch.cuda.synchronize()
+    dev = (out.float() - 1.0).abs().amax(dim=(0, 2, 3))
+    for h in range(hq):
+        assert dev[h].item() <= 2.0 ** -8, f"head {h} ({table[0][str(h)][0]}): max |out - 1| = {dev[h].item()}"
