@@ -434,3 +434,38 @@ def test_config5_layer_slice_every_row_is_normalised(gpu):
     dev = (out.float() - 1.0).abs().amax(dim=(0, 2, 3))
     for h in range(hq):
         assert dev[h].item() <= 2.0 ** -8, f"head {h} ({table[0][str(h)][0]}): max |out - 1| = {dev[h].item()}"
+
+
+def test_full_size_every_operator_reduces_to_dense_on_all_rows(gpu):
+    """Library special cases at 131072 tokens, compared on EVERY row: dense causal attention of this
+    engine against torch's own flash attention (an independent implementation; 16-bit tolerance), and
+    every sparse operator in the setting where its index keeps the whole causal triangle -- every
+    diagonal kept (block lists of 2048 entries: the walk that is not split in LDS), window wider than
+    the sequence, top_k >= number of blocks, n_last = n - 1 -- against this engine's dense output."""
+    import minference_amd as M
+    n, hq, hk = 131072, 2, 1
+    q, k, v = gen.qkv(1, hq, hk, n, 128, seed=21, scale=1.0)
+    qg, kg, vg = q.bfloat16().to(gpu), k.bfloat16().to(gpu), v.bfloat16().to(gpu)
+    print("case full-size dense vs torch SDPA", flush=True)
+    dense = M.dense_causal_attention(qg, kg, vg)
+    ref = torch.nn.functional.scaled_dot_product_attention(qg, kg, vg, is_causal=True, enable_gqa=True)
+    d = (dense.float() - ref.float()).abs()
+    print(f"  dense vs SDPA: max-abs {d.max().item():.3e} mean-abs {d.mean().item():.3e}", flush=True)
+    assert d.max().item() <= 2e-2 and d.mean().item() <= 1e-3
+    del ref, d
+
+    def same_as_dense(name, out, tol=4e-3):
+        dd = (out.float() - dense.float()).abs()
+        print(f"  {name} vs dense: max-abs {dd.max().item():.3e} mean-abs {dd.mean().item():.3e}", flush=True)
+        assert dd.max().item() <= tol, name
+
+    print("case full-size a-shape / tri-shape / block-sparse / vertical-slash in their dense limits", flush=True)
+    same_as_dense("a-shape, window > n", M.streaming_forward(qg, kg, vg, 4, n + 5))
+    same_as_dense("tri-shape, n_last = n - 1", M.tri_shape_forward(qg, kg, vg, 4, 64, n - 1))
+    same_as_dense("block-sparse, top_k >= blocks", M.block_sparse_attention(qg, kg, vg, n // 64 + 1))
+    s_idx = torch.arange(n, dtype=torch.int32, device=gpu)[None, None].expand(1, 1, n).contiguous()
+    v_idx = torch.zeros((1, 1, 1), dtype=torch.int32, device=gpu)
+    out = M.vertical_slash_sparse_attention(qg[:, :1], kg, vg, v_idx, s_idx)        # one head: 1 GiB of block lists
+    dd = (out.float() - dense[:, :1].float()).abs()
+    print(f"  vertical-slash, every diagonal vs dense: max-abs {dd.max().item():.3e} mean-abs {dd.mean().item():.3e}", flush=True)
+    assert dd.max().item() <= 4e-3
