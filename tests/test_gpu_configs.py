@@ -469,3 +469,100 @@ def test_full_size_every_operator_reduces_to_dense_on_all_rows(gpu):
     dd = (out.float() - dense[:, :1].float()).abs()
     print(f"  vertical-slash, every diagonal vs dense: max-abs {dd.max().item():.3e} mean-abs {dd.mean().item():.3e}", flush=True)
     assert dd.max().item() <= 4e-3
+
+
+def _fp32_rows_on_gpu(q_rows, k32, v32, mask):
+    s_ = (q_rows.float() @ k32.T) * (q_rows.shape[-1] ** -0.5)
+    s_ = s_.masked_fill(~mask, float("-inf"))
+    return torch.softmax(s_, dim=-1) @ v32
+
+
+def test_config2_whole_heads_against_fp32_masked_dense_on_the_gpu(gpu):
+    """BASELINE config 2 at full size, EVERY row block of two heads (one of the first and one of the last
+    kv group): the mask of each row block is expanded on the GPU from the index tensors the HIP builder
+    wrote -- keys of every listed block up to the causal limit, plus the listed columns
+    (pit_sparse_flash_attention_v2.py:104-148) -- and the rows are recomputed as an fp32 masked-dense
+    softmax in torch.  Tolerance as everywhere: max-abs 2e-2, mean-abs 1e-3 per row block.  (The
+    sampled tests above check the index rows against the reference algorithm and a few row blocks
+    against the CPU oracle; this one leaves no row of a head unchecked.)"""
+    import minference_amd as M
+    n, hq, hk = 131072, 32, 8
+    q, k, v, _ = gen.planted_layer(n, hq, hk, seed=100, dtype=torch.bfloat16)
+    qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
+    v_idx, s_idx = M.estimate_vertical_slash(qg, kg, 1000, 6096)
+    seqlens = torch.full((1,), n, dtype=torch.int32, device=gpu)
+    bc, bo, cc, ci = M.convert_vertical_slash_indexes(seqlens, v_idx, s_idx, n, 64, 64, zero_fill=False)
+    out = M.vertical_slash_attention_from_index(qg, kg, vg, bc, bo, cc, ci, seqlens)
+    torch.cuda.synchronize()
+    ar64 = torch.arange(64, device=gpu)
+    pos = torch.arange(n, device=gpu)
+    for h in (2, 29):
+        kv = h // (hq // hk)
+        k32, v32 = kg[0, kv].float(), vg[0, kv].float()
+        nb, nc = bc[0, h].tolist(), cc[0, h].tolist()
+        worst_max = worst_mean = 0.0
+        print(f"case c2 whole head {h}", flush=True)
+        for m in range(n // 64):
+            allowed = torch.zeros(n + 64, dtype=torch.bool, device=gpu)
+            starts = bo[0, h, m, :nb[m]].long()
+            allowed[(starts[:, None] + ar64[None, :]).reshape(-1).clamp_(0, n + 63)] = True
+            rows = m * 64 + ar64
+            mask = allowed[None, :n] & (pos[None, :] <= rows[:, None])
+            if nc[m]:
+                colmask = torch.zeros(n, dtype=torch.bool, device=gpu)
+                colmask[ci[0, h, m, :nc[m]].long()] = True
+                mask |= colmask[None, :]
+            ref = _fp32_rows_on_gpu(qg[0, h, m * 64:m * 64 + 64], k32, v32, mask)
+            err = (out[0, h, m * 64:m * 64 + 64].float() - ref).abs()
+            worst_max, worst_mean = max(worst_max, err.max().item()), max(worst_mean, err.mean().item())
+            assert err.max().item() <= 2e-2 and err.mean().item() <= 1e-3, (h, m, err.max().item(), err.mean().item())
+        print(f"  head {h}: worst row block max-abs {worst_max:.3e} mean-abs {worst_mean:.3e}", flush=True)
+
+
+def test_config4_and_config5_whole_heads_against_fp32_masked_dense_on_the_gpu(gpu):
+    """Every row block of one head, fp32 masked-dense softmax recomputed in torch on the GPU: the
+    block-sparse operator at BASELINE config 4's shape (131072 tokens, top-100 with diagonal and first
+    block; mask = the first min(m + 1, top_k) listed blocks up to the causal limit,
+    block_sparse_flash_attention.py:81-96) and the A-shape operator at config 5's (262144 tokens, sink 128
+    + window 4096; mask = the closed form of streaming_kernel.py:35-75)."""
+    import minference_amd as M
+    from minference_amd.ops import _build_block_index, block_sparse_attention_from_index
+    n5, hq, hk = 262144, 4, 1
+    q, k, v, _ = gen.planted_layer(n5, hq, hk, seed=100, dtype=torch.bfloat16)
+    qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
+    ar64 = torch.arange(64, device=gpu)
+
+    def sweep(tag, out, n, h, mask_of):
+        k32, v32 = kg[0, 0, :n].float(), vg[0, 0, :n].float()
+        worst_max = worst_mean = 0.0
+        for m in range(n // 64):
+            rows = m * 64 + ar64
+            ref = _fp32_rows_on_gpu(qg[0, h, m * 64:m * 64 + 64], k32, v32, mask_of(m, rows))
+            err = (out[0, h, m * 64:m * 64 + 64].float() - ref).abs()
+            worst_max, worst_mean = max(worst_max, err.max().item()), max(worst_mean, err.mean().item())
+            assert err.max().item() <= 2e-2 and err.mean().item() <= 1e-3, (tag, m, err.max().item(), err.mean().item())
+        print(f"  {tag}: worst row block max-abs {worst_max:.3e} mean-abs {worst_mean:.3e}", flush=True)
+
+    n4 = 131072
+    print("case c4 whole head", flush=True)
+    q4, k4, v4 = qg[:, :, :n4], kg[:, :, :n4], vg[:, :, :n4]
+    bi = _build_block_index(q4, k4, 100, force_diag_first=True)
+    out4 = block_sparse_attention_from_index(q4, k4, v4, bi)
+    pos4 = torch.arange(n4, device=gpu)
+
+    def bs_mask(m, rows, h=1):
+        allowed = torch.zeros(n4 + 64, dtype=torch.bool, device=gpu)
+        blocks = bi[0, h, m, :min(m + 1, 100)].long() * 64
+        allowed[(blocks[:, None] + ar64[None, :]).reshape(-1)] = True
+        return allowed[None, :n4] & (pos4[None, :] <= rows[:, None])
+    sweep("block-sparse head 1 at 131072", out4, n4, 1, bs_mask)
+    del out4, bi
+
+    print("case c5 a-shape whole head", flush=True)
+    out5 = M.streaming_forward(qg, kg, vg, 128, 4096)
+    pos5 = torch.arange(n5, device=gpu)
+
+    def ashape_mask(m, rows):
+        d = rows[:, None] - pos5[None, :]
+        return (d >= 0) & ((d < 4096) | (pos5[None, :] < 128))
+    sweep("a-shape head 3 at 262144", out5, n5, 3, ashape_mask)
