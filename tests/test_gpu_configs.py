@@ -566,3 +566,41 @@ def test_config4_and_config5_whole_heads_against_fp32_masked_dense_on_the_gpu(gp
         d = rows[:, None] - pos5[None, :]
         return (d >= 0) & ((d < 4096) | (pos5[None, :] < 128))
     sweep("a-shape head 3 at 262144", out5, n5, 3, ashape_mask)
+
+
+@pytest.mark.parametrize("d,dtype,n", [(64, torch.bfloat16, 65536), (128, torch.float16, 32768), (64, torch.float16, 20000 + 37)])
+def test_whole_head_of_the_other_instantiations(gpu, d, dtype, n):
+    """The head_dim 64 and the fp16 instantiations of the vertical-slash path (estimate -> top-k ->
+    index -> attention), every row block of one head against the fp32 masked-dense softmax in torch
+    on the GPU, incl. a length that is not a multiple of 64."""
+    import minference_amd as M
+    hq, hk = 2, 1
+    q, k, v = gen.qkv(1, hq, hk, n, d, seed=d + n, scale=1.0)
+    qg, kg, vg = q.to(dtype).to(gpu), k.to(dtype).to(gpu), v.to(dtype).to(gpu)
+    v_idx, s_idx = M.estimate_vertical_slash(qg, kg, 300, 2000)
+    seqlens = torch.full((1,), n, dtype=torch.int32, device=gpu)
+    bc, bo, cc, ci = M.convert_vertical_slash_indexes(seqlens, v_idx, s_idx, n, 64, 64, zero_fill=False)
+    out = M.vertical_slash_attention_from_index(qg, kg, vg, bc, bo, cc, ci, seqlens)
+    assert torch.isfinite(out.float()).all()
+    h = 1
+    ar64 = torch.arange(64, device=gpu)
+    pos = torch.arange(n, device=gpu)
+    k32, v32 = kg[0, 0].float(), vg[0, 0].float()
+    nb, nc = bc[0, h].tolist(), cc[0, h].tolist()
+    worst_max = worst_mean = 0.0
+    print(f"case whole head d={d} {dtype} n={n}", flush=True)
+    for m in range((n + 63) // 64):
+        rows = (m * 64 + ar64)[: min(64, n - m * 64)]
+        allowed = torch.zeros(n + 128, dtype=torch.bool, device=gpu)
+        starts = bo[0, h, m, :nb[m]].long()
+        allowed[(starts[:, None] + ar64[None, :]).reshape(-1).clamp_(0, n + 127)] = True
+        mask = allowed[None, :n] & (pos[None, :] <= rows[:, None])
+        if nc[m]:
+            colmask = torch.zeros(n, dtype=torch.bool, device=gpu)
+            colmask[ci[0, h, m, :nc[m]].long()] = True
+            mask |= colmask[None, :]
+        ref = _fp32_rows_on_gpu(qg[0, h, rows], k32, v32, mask)
+        err = (out[0, h, rows].float() - ref).abs()
+        worst_max, worst_mean = max(worst_max, err.max().item()), max(worst_mean, err.mean().item())
+        assert err.max().item() <= 2e-2 and err.mean().item() <= 1e-3, (m, err.max().item(), err.mean().item())
+    print(f"  worst row block max-abs {worst_max:.3e} mean-abs {worst_mean:.3e}", flush=True)
