@@ -747,7 +747,12 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
         const bool grow = cand > m_i + LAZY_MAX;
         const float m_new = grow ? cand : m_i;
         m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        alpha = grow ? __builtin_amdgcn_exp2f(m_i - m_use) : 1.0f;
+        // `alpha` is the SQUARE ROOT of the rescale factor and is applied twice.  With a maximum that
+        // is looked at only now and then, the sums accumulated under the old one may be as large as
+        // 2^127 (probabilities far above 1 that have not overflowed), so a factor below 2^-126 does
+        // not mean that they are negligible -- and exp2 of such an exponent is flushed to zero.  Half
+        // the exponent twice is exact down to 2^-252, beyond which nothing finite is left of them.
+        alpha = grow ? __builtin_amdgcn_exp2f(fmaxf(0.5f * (m_i - m_use), -126.0f)) : 1.0f;
         m_i = m_new;
         }
         float psum = 0.f;
@@ -766,7 +771,7 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
 #pragma unroll
             for (int i = 0; i < NDB; ++i)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
+                for (int r = 0; r < 16; ++r) oacc[i][r] = (oacc[i][r] * alpha) * alpha;
         }
 
         __builtin_amdgcn_s_setprio(2);
@@ -775,7 +780,7 @@ __device__ __forceinline__ bool attn_walk(const AttnParams &p, char (&lds_k)[Att
             probs(1);
             probs(2);
             probs(3);
-            l_i = l_i * alpha + psum;
+            l_i = (l_i * alpha) * alpha + psum;
             if constexpr (VF_AHEAD) {
 #pragma unroll
             for (int s = 0; s < 4; ++s)

@@ -503,6 +503,42 @@ def test_scores_rising_steadily_past_the_fp32_range(gpu, mult, n):
         check(f(vg), ref(), f"rising {name}")
 
 
+@pytest.mark.parametrize("d,dtype", [(64, torch.bfloat16), (128, torch.bfloat16), (64, torch.float16)])
+def test_maximum_raised_by_more_than_the_fp32_exponent_range_at_once(gpu, d, dtype):
+    """Scores that climb steeply and steadily along the keys (300 sin(2 pi s / 8192) natural-log units,
+    about 21 powers of two per tile).  A walk that looks at the row maximum on the first tiles and
+    then on the eighth finds, under the old maximum, sums near 2^126 -- finite, nothing overflowed --
+    and a new maximum more than 126 powers of two higher: the rescale factor underflows although
+    what it scales is far from negligible (for a row just past a tile boundary the keys of the
+    previous tile weigh as much as its own).  The factor is therefore applied as the square of its
+    root.  Every operator, every row, against the fp32 oracle."""
+    import math
+    import minference_amd as M
+    from minference_amd.ops import _build_block_index
+    n, hq, hk = 2304, 2, 1
+    g = torch.Generator().manual_seed(38)
+    q = torch.randn(1, hq, n, d, generator=g) * 0.5
+    k = torch.randn(1, hk, n, d, generator=g) * 0.5
+    v = torch.randn(1, hk, n, d, generator=g)
+    q[..., 0] = 8.0
+    k[..., 0] = (torch.sin(2 * math.pi * torch.arange(n).float() / 8192) * 300.0 * d ** 0.5 / 8.0)[None, None, :]
+    q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
+    qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
+    ke, ve = expand(k, hq), expand(v, hq)
+    print(f"case steep rise d={d} {dtype}", flush=True)
+    check(M.streaming_forward(qg, kg, vg, 4, 512), O.streaming_forward(q, ke, ve, 4, 512), "steep a-shape")
+    check(M.tri_shape_forward(qg, kg, vg, 4, 512, 64), O.tri_shape_forward(q, ke, ve, 4, 512, 64), "steep tri-shape")
+    check(M.dense_causal_attention(qg, kg, vg), sdpa_causal(q, ke, ve), "steep dense")
+    bi = _build_block_index(qg, kg, 12, force_diag_first=True)
+    ref = torch.stack([O.masked_attention(q[0, h], ke[0, h], ve[0, h], O.bs_mask(bi[0, h].cpu().numpy(), n)) for h in range(hq)])[None]
+    check(M.block_sparse_attention_from_index(qg, kg, vg, bi), ref, "steep block-sparse")
+    # slashes 0..639: a window of ten tiles per row, walked as one run of blocks
+    v_idx = torch.arange(4, dtype=torch.int32, device=gpu).repeat(1, hq, 1)
+    s_idx = torch.arange(639, -1, -1, dtype=torch.int32, device=gpu).repeat(1, hq, 1)
+    check(M.vertical_slash_sparse_attention(qg, kg, vg, v_idx, s_idx),
+          O.vertical_slash_sparse_attention(q, ke, ve, v_idx.cpu(), s_idx.cpu()), "steep vertical-slash")
+
+
 @pytest.mark.parametrize("n", [1, 37, 63, 65])
 def test_tiny_sequences_all_operators(gpu, n):
     import minference_amd as M
