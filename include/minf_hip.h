@@ -272,6 +272,9 @@ int minf_vs_estimate_heads(const void *q, const void *k, const int64_t *q_stride
  * with out_stride.  reverse_base < 0: out = index; otherwise out =
  * reverse_base - index (slash: reverse_base = n-1 turns ascending j into
  * descending diagonal offsets, the order the index builder wants).
+ * Values are ordered by their bit patterns: -0.0 ranks below +0.0 and denormals are told apart
+ * (the scores of this path are sums of probabilities or matrix products, which hold no -0.0);
+ * NaN has no defined rank.
  */
 int minf_topk_indices(const float *scores, int rows, int n, int64_t row_stride, int k,
                       int32_t *out, int64_t out_stride, int reverse_base, void *stream);
