@@ -44,7 +44,10 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
 typedef __attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned u32x4_t;
 
 constexpr int LQ = 64;          // query rows held per head (last_q <= LQ)
-constexpr int KC = 2048;        // keys per workgroup
+#ifndef EST_KC
+#define EST_KC 2048
+#endif
+constexpr int KC = EST_KC;      // keys per workgroup
 constexpr int EST_THREADS = 256;
 constexpr int WIN = KC + LQ;    // diagonal window of one chunk
 
