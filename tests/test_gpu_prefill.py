@@ -406,3 +406,42 @@ def test_config5_ashape_heads_full_size_sampled_row_blocks(gpu):
         assert err.max() <= 2e-2 and err.mean() <= 1e-3
         # and relative to the size of the outputs (rows that average over thousands of keys are small)
         assert err.max() <= 2e-2 * scale and err.mean() <= 1e-3 * scale
+
+
+def test_mixed_layer_replays_from_a_hip_graph(gpu):
+    """Every launch chain of a mixed layer (estimate -> ragged top-k -> index build -> vertical-slash
+    attention; block index -> block-sparse attention; A-shape) recorded once into a HIP graph through
+    torch.cuda.graph and replayed on new inputs written into the captured buffers: each replay must be
+    bit-identical to the eager call on the same inputs.  Between the replays the process does eager
+    work and synchronises, and the layer's host-side plan (head lists, per-head sizes) is already on
+    the device, so the capture contains no host-to-device copy and no allocation outside torch's
+    graph pool."""
+    import minference_amd as M
+    n, hq, hk = 8192 + 64, 8, 2
+    layer = {"0": ["vertical_and_slash", 1000, 6096, 1.0], "1": ["vertical_and_slash", 100, 800, 1.0],
+             "2": ["block_sparse", 100, 0, 1.0], "3": ["stream_llm", 64, 1024, 1.0],
+             "4": ["vertical_and_slash", 500, 3000, 1.0], "5": ["block_sparse", 100, 0, 1.0],
+             "6": ["stream_llm", 128, 512, 1.0]}                      # head 7: the default pattern
+    kwargs = {"layer_idx": 0, "attn_forward_config": {"best_pattern": [layer]}}
+    inputs = [tuple(t.to(gpu) for t in gen.planted_layer(n, hq, hk, seed=s, dtype=torch.bfloat16)[:3]) for s in (1, 2, 3)]
+    qs, ks, vs = (t.clone() for t in inputs[0])
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            M.minference_prefill_forward(qs, ks, vs, kwargs)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    print("case graph capture of a mixed layer", flush=True)
+    with torch.cuda.graph(graph):
+        out_static = M.minference_prefill_forward(qs, ks, vs, kwargs)
+    for rep, (q, k, v) in enumerate(inputs + inputs[:1]):
+        qs.copy_(q); ks.copy_(k); vs.copy_(v)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out_static.clone()
+        eager = M.minference_prefill_forward(q, k, v, kwargs)          # eager work between the replays
+        torch.cuda.synchronize()
+        assert torch.isfinite(got.float()).all()
+        assert torch.equal(got, eager), f"replay {rep} differs from the eager call"
