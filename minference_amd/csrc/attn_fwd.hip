@@ -77,7 +77,7 @@ enum { MODE_VS = 0, MODE_BS = 1, MODE_ASHAPE = 2, MODE_DENSE = 3 };
 
 constexpr int BM = 64;        // query rows per workgroup
 constexpr int BN = 64;        // keys per tile
-constexpr int HD_MAX = 256;   // head_dim: 64, 128 or (dense / A-shape / tri-shape only) 256: template parameter HD of the kernel
+// head_dim (template parameter HD of the kernel): 64, 128 or, for dense / A-shape / tri-shape only, 256
 constexpr int NTHREADS = 128; // 2 wavefronts per 64-row block, two row blocks per workgroup
 // Scheduling constants (measured on MI355X): K fragments are read QK_AHEAD k-steps ahead of their
 // MFMAs; VALU_PER_MFMA softmax instructions are placed behind each of the first twelve PV MFMAs.

@@ -248,7 +248,9 @@ __global__ __launch_bounds__(64) void pattern_recall_finalize(const float *parti
 #pragma unroll
         for (int d = 32; d >= 1; d >>= 1) x += __shfl_xor(x, d);
         // no rows to average over -> NaN, like the mean of an empty slice in the reference
-        if (lane == 0) recall[head_lin * NC + t] = n > row_begin ? x / (float)(n - max(row_begin, 0)) : NAN;
+        // (written as a bit pattern: the library is built without NaN semantics, under which the constant
+        // itself is undefined)
+        if (lane == 0) recall[head_lin * NC + t] = n > row_begin ? x / (float)(n - max(row_begin, 0)) : __uint_as_float(0x7fc00000u);
     }
 }
 

@@ -78,7 +78,7 @@ __global__ __launch_bounds__(TK_THREADS) void topk_kernel(const TopkProblem p0, 
 
     // ---- 1. radix select --------------------------------------------------
     const int nvec = (((uintptr_t)x & 15) == 0) ? (n >> 2) : 0;
-    unsigned prefix = 0, mask = 0;
+    unsigned prefix = 0;
     unsigned need = (unsigned)k;     // rank (from the top) inside the current prefix bucket
     for (int shift = 24; shift >= 0; shift -= 8) {
         for (int i = tid; i < 256 * 32; i += TK_THREADS) hist[i] = 0;
@@ -143,7 +143,6 @@ __global__ __launch_bounds__(TK_THREADS) void topk_kernel(const TopkProblem p0, 
         __syncthreads();
         prefix = sh_prefix;
         need = sh_need;
-        mask |= 255u << shift;
     }
     const unsigned T = prefix;       // key of the k-th largest; `need` entries equal to T are taken
 

@@ -59,7 +59,6 @@ struct EstParams {
     float scale;                // sm_scale itself (the rounded form scales in the natural-log domain)
     int nchunks;
     float *stats;               // [B, Hq, nchunks, LQ, 2]
-    float *rowstat;             // [B, Hq, LQ] (part of the workspace layout; no longer used)
     float *win;                 // [B, Hq, nchunks, WIN]
     float *vertical, *slash;    // [B, Hq, N]
     int force_v, force_s;
@@ -608,13 +607,11 @@ int fill(EstParams &p, const void *q, const void *k, const int64_t *q_stride, co
     p.nchunks = (n + KC - 1) / KC;
     const long long bh = (long long)batch * index_heads;
     const size_t stats_b = (size_t)bh * p.nchunks * LQ * 2 * sizeof(float);
-    const size_t row_b = (size_t)bh * LQ * sizeof(float);
     const size_t win_b = (size_t)bh * p.nchunks * WIN * sizeof(float);
-    if (ws_bytes < stats_b + row_b + win_b) return MINF_ERR_WORKSPACE;
+    if (ws_bytes < stats_b + win_b) return MINF_ERR_WORKSPACE;
     if ((uintptr_t)ws & 15) return MINF_ERR_ALIGNMENT;
     p.stats = (float *)ws;
-    p.rowstat = (float *)((char *)ws + stats_b);
-    p.win = (float *)((char *)ws + stats_b + row_b);
+    p.win = (float *)((char *)ws + stats_b);
     p.vertical = vertical; p.slash = slash;
     p.force_v = force_v; p.force_s = force_s;
     // heads per workgroup: neighbours in head order that (mostly) share a kv head
@@ -633,7 +630,7 @@ extern "C" size_t minf_vs_estimate_workspace_bytes(int batch, int heads_q, int n
     if (batch <= 0 || heads_q <= 0 || n <= 0) return 0;
     const size_t bh = (size_t)batch * heads_q;
     const size_t nchunks = ((size_t)n + KC - 1) / KC;
-    return bh * nchunks * LQ * 2 * sizeof(float) + bh * LQ * sizeof(float) + bh * nchunks * WIN * sizeof(float);
+    return bh * nchunks * LQ * 2 * sizeof(float) + bh * nchunks * WIN * sizeof(float);
 }
 
 static int estimate_launch(const void *q, const void *k, const int64_t *q_stride, const int64_t *k_stride,
