@@ -604,3 +604,53 @@ def test_whole_head_of_the_other_instantiations(gpu, d, dtype, n):
         worst_max, worst_mean = max(worst_max, err.max().item()), max(worst_mean, err.mean().item())
         assert err.max().item() <= 2e-2 and err.mean().item() <= 1e-3, (m, err.max().item(), err.mean().item())
     print(f"  worst row block max-abs {worst_max:.3e} mean-abs {worst_mean:.3e}", flush=True)
+
+
+def test_index_tensors_of_more_than_2_to_31_elements(gpu):
+    """32 heads x 16384 row blocks x 6096 slash slots at 1 048 576 tokens: block_offset holds 1.49 x 2^31
+    elements (12.8 GB), so every offset into it -- in the index builder and in the attention kernel's
+    list walk -- has to be 64-bit (the reference's int offsets overflow here,
+    csrc/vertical_slash_index.cu:55-59).  The lists keep the attention cheap (a window of 64..192
+    diagonals, twenty far ones, the rest beyond the context, i.e. skipped; 1000 verticals); sampled
+    (head, row block) pairs from the first and the last heads: index rows against the reference
+    algorithm, attention rows against an fp32 masked-dense softmax in torch on the GPU."""
+    import minference_amd as M
+    n, hq, hk, S, V = 1048576, 32, 8, 6096, 1000
+    g = torch.Generator(device=gpu).manual_seed(5)
+    q = torch.randn(1, hq, n, 128, generator=g, device=gpu, dtype=torch.bfloat16)
+    k = torch.randn(1, hk, n, 128, generator=g, device=gpu, dtype=torch.bfloat16)
+    v = torch.randn(1, hk, n, 128, generator=g, device=gpu, dtype=torch.bfloat16)
+    rng = np.random.default_rng(7)
+    s_np, v_np = np.zeros((1, hq, S), np.int64), np.zeros((1, hq, V), np.int64)
+    for h in range(hq):
+        near = np.arange(int(rng.integers(64, 193)))
+        far = rng.choice(np.arange(1000, n), size=20, replace=False)
+        beyond = n + np.arange(S - len(near) - len(far)) * 3 + int(rng.integers(0, 1000))
+        s_np[0, h] = np.sort(np.concatenate([near, far, beyond]))[::-1]
+        v_np[0, h] = np.sort(np.concatenate([np.arange(4), rng.choice(np.arange(4, n), size=V - 4, replace=False)]))
+    s_idx, v_idx = torch.from_numpy(s_np.astype(np.int32)).to(gpu), torch.from_numpy(v_np.astype(np.int32)).to(gpu)
+    seqlens = torch.full((1,), n, dtype=torch.int32, device=gpu)
+    print("case index tensors beyond 2^31 elements", flush=True)
+    bc, bo, cc, ci = M.convert_vertical_slash_indexes(seqlens, v_idx, s_idx, n, 64, 64, zero_fill=False)
+    assert bo.numel() > 2 ** 31
+    out = M.vertical_slash_attention_from_index(q, k, v, bc, bo, cc, ci, seqlens)
+    torch.cuda.synchronize()
+    rows = n // 64
+    pos = torch.arange(n, device=gpu)
+    for h, m in [(0, 0), (0, rows - 1), (20, 5), (21, 8000), (22, rows - 1), (31, 0), (31, 12345), (31, rows - 1), (30, rows - 2)]:
+        rbo, rci = O.vs_index_row_py(v_np[0, h].tolist(), s_np[0, h].tolist(), m, n)
+        assert int(bc[0, h, m]) == len(rbo) and int(cc[0, h, m]) == len(rci), (h, m)
+        assert bo[0, h, m, :len(rbo)].cpu().tolist() == rbo and ci[0, h, m, :len(rci)].cpu().tolist() == rci, (h, m)
+        allowed = torch.zeros(n + 128, dtype=torch.bool, device=gpu)
+        for st in rbo:
+            allowed[st:st + 64] = True
+        rows_m = m * 64 + torch.arange(64, device=gpu)
+        mask = allowed[None, :n] & (pos[None, :] <= rows_m[:, None])
+        if rci:
+            col = torch.zeros(n, dtype=torch.bool, device=gpu)
+            col[torch.tensor(rci, device=gpu)] = True
+            mask |= col[None, :]
+        ref = _fp32_rows_on_gpu(q[0, h, rows_m], k[0, h // 4].float(), v[0, h // 4].float(), mask)
+        err = (out[0, h, rows_m].float() - ref).abs()
+        print(f"  head {h} row block {m}: blocks {len(rbo)} cols {len(rci)} max-abs {err.max().item():.3e}", flush=True)
+        assert err.max().item() <= 2e-2 and err.mean().item() <= 1e-3, (h, m)
