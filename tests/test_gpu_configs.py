@@ -654,3 +654,38 @@ def test_index_tensors_of_more_than_2_to_31_elements(gpu):
         err = (out[0, h, rows_m].float() - ref).abs()
         print(f"  head {h} row block {m}: blocks {len(rbo)} cols {len(rci)} max-abs {err.max().item():.3e}", flush=True)
         assert err.max().item() <= 2e-2 and err.mean().item() <= 1e-3, (h, m)
+
+
+def test_block_index_at_one_million_tokens(gpu):
+    """The block index of 32 heads at 1 048 576 tokens: 16385 block rows, so the pooled score matrix in
+    the workspace has 8.6e9 elements (more than 2^31; 34 GB) and the general top-k runs on 524 320 rows
+    of 16388 scores.  Sampled rows of the first, a middle and the last head against the reference's
+    arithmetic restated with torch on the GPU (bf16 means, bf16 pooled products,
+    block_sparse_flash_attention.py:159-163; an entry the restatement lacks must lie within one bf16
+    unit of its k-th score)."""
+    from minference_amd.ops import _build_block_index
+    n, hq, hk = 1048576, 32, 8
+    g = torch.Generator(device=gpu).manual_seed(5)
+    q = torch.randn(1, hq, n, 128, generator=g, device=gpu, dtype=torch.bfloat16)
+    k = torch.randn(1, hk, n, 128, generator=g, device=gpu, dtype=torch.bfloat16)
+    # a slow drift shared by q and k, so that the pooled scores separate
+    drift = torch.cumsum(torch.randn(n // 64 + 1, 128, generator=g, device=gpu) * 0.3, 0).repeat_interleave(64, 0)[:n]
+    q, k = (q.float() + drift[None, None]).bfloat16(), (k.float() + drift[None, None]).bfloat16()
+    del drift
+    print("case block index at 1M tokens", flush=True)
+    bi = _build_block_index(q, k, 100, force_diag_first=True)
+    R = bi.shape[2]
+    assert bi.shape == (1, hq, n // 64 + 1, 100)
+    for h in (0, 13, 31):
+        qp = torch.nn.functional.pad(q[0, h].float(), [0, 0, 0, 64]).reshape(R, 64, 128).mean(1).bfloat16().float()
+        kp = torch.nn.functional.pad(k[0, h // 4].float(), [0, 0, 0, 64]).reshape(R, 64, 128).mean(1).bfloat16().float()
+        for m in (0, 1, 99, 100, 5000, 12000, R - 2, R - 1):
+            sc = (kp[: m + 1] @ qp[m]).bfloat16().float()
+            sc[m] = sc[0] = float("inf")
+            kk = min(100, m + 1)
+            want = torch.argsort(sc, descending=True, stable=True)[:kk]
+            got = bi[0, h, m, :kk].long()
+            assert bool((got[1:] > got[:-1]).all()), (h, m)
+            kth = sc[want].min().item()
+            extra = set(got.tolist()) - set(want.tolist())
+            assert all(x <= m and sc[x].item() >= kth - abs(kth) * 2.0 ** -6 - 1e-6 for x in extra), (h, m, sorted(extra)[:5])
