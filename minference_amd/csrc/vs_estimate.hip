@@ -50,6 +50,14 @@ constexpr int LQ = 64;          // query rows held per head (last_q <= LQ)
 constexpr int KC = EST_KC;      // keys per workgroup
 constexpr int EST_THREADS = 256;
 constexpr int WIN = KC + LQ;    // diagonal window of one chunk
+// A chunk is always summed as four pieces of KC/4 keys, each piece by one wave from its first key to
+// its last, and the pieces are combined in ascending order -- whether one wave walks the whole chunk
+// (four heads per workgroup) or four waves a piece each (one head per workgroup).  The scores of a
+// head therefore do not depend, not even in the last bit, on which other heads share its launch.
+constexpr int PIECE = KC / 4;
+constexpr int PB = PIECE / 32;  // 32-key blocks per piece
+constexpr int PWIN = PIECE + LQ;
+static_assert(KC % 128 == 0, "a chunk is four pieces of whole 32-key blocks");
 
 struct EstParams {
     const char *q, *k;
@@ -228,16 +236,36 @@ __device__ __forceinline__ int common_kv_head(const EstParams &p, const WgId &w,
 template <typename T, int HD, bool RR>
 __global__ __launch_bounds__(EST_THREADS, 3) void est_stats_kernel(const EstParams p) {
     constexpr int KS = HD / 16;       // k-steps of one 32x32 score block
-    __shared__ float lds_m[4][LQ], lds_l[4][LQ];
+    __shared__ float lds_m[16][LQ], lds_l[16][LQ];     // [head of the workgroup * 4 + piece][row]
     const int tid = (int)threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);       // wave-uniform: addresses built from it stay scalar
     const WgId w = decode_wg(p, wave, false);
     if (!w.valid) return;
     const int l32 = lane & 31, g = lane >> 5;
     const int nq = 4 / p.gw, klen = KC / nq;          // key sub-ranges per head, keys per wave
+    const int ppw = p.gw;                             // pieces per wave (klen / PIECE)
+    const int piece0 = (wave % p.gw) * 4 + w.kq * ppw; // this wave's first (head, piece) slot
 
     // lane <-> query rows i = l32 and 32 + l32; regs <-> keys 8*(r/4) + 4*g + r%4 of the block
     float m_run[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.f, 0.f};
+    int pieces_done = 0;
+    // the running pair of a finished piece: merge the two lane halves, park it, start afresh
+    auto flush_piece = [&]() {
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) {
+            const float mo = __shfl_xor(m_run[nb], 32), lo = __shfl_xor(l_run[nb], 32);
+            const float m_new = fmaxf(m_run[nb], mo);
+            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+            const float l_new = l_run[nb] * __builtin_amdgcn_exp2f(m_run[nb] - m_use) + lo * __builtin_amdgcn_exp2f(mo - m_use);
+            if (g == 0) {
+                lds_m[piece0 + pieces_done][32 * nb + l32] = m_new;
+                lds_l[piece0 + pieces_done][32 * nb + l32] = l_new;
+            }
+            m_run[nb] = -INFINITY;
+            l_run[nb] = 0.f;
+        }
+        ++pieces_done;
+    };
     __shared__ __attribute__((aligned(16))) char lds_kt[2][2 * KShare<HD>::TILE];
     __shared__ int lds_hkv[4];
     const int kv_common = common_kv_head(p, w, wave, lane, lds_hkv);       // (workgroup-uniform)
@@ -310,6 +338,7 @@ __global__ __launch_bounds__(EST_THREADS, 3) void est_stats_kernel(const EstPara
                 ks_.template frags<KS>(blk & 1, lane, kf);
                 score_block(c0, kf);
             }
+            if (w.wave_valid && (blk + 1) % PB == 0) flush_piece();
         }
     } else if (w.wave_valid) {
         const char *kb = p.k + ((long long)w.b * p.ks[0] + (long long)w.hkv * p.ks[1]) * 2;
@@ -322,30 +351,21 @@ __global__ __launch_bounds__(EST_THREADS, 3) void est_stats_kernel(const EstPara
             for (int ks = 0; ks < KS; ++ks) kf[ks] = kn[ks];
             load_k(p, kb, min(c0 + 32, p.n - 1), lane, kn);      // next block, in flight during this one
             score_block(c0, kf);
+            if ((blk + 1) % PB == 0) flush_piece();
         }
     }
-    // merge the two lane halves, then the waves that share a head
-#pragma unroll
-    for (int nb = 0; nb < 2; ++nb) {
-        const float mo = __shfl_xor(m_run[nb], 32), lo = __shfl_xor(l_run[nb], 32);
-        const float m_new = fmaxf(m_run[nb], mo);
-        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        l_run[nb] = l_run[nb] * __builtin_amdgcn_exp2f(m_run[nb] - m_use) + lo * __builtin_amdgcn_exp2f(mo - m_use);
-        m_run[nb] = m_new;
-        if (g == 0) {
-            lds_m[wave][32 * nb + l32] = m_run[nb];
-            lds_l[wave][32 * nb + l32] = l_run[nb];
-        }
-    }
+    // (pieces past the end of the sequence: what is left of the running pair, then empty pairs)
+    if (w.wave_valid)
+        while (pieces_done < ppw) flush_piece();
     __syncthreads();
-    // thread (hsub, row): the nq waves hsub, hsub + gw, ... hold the pieces of head hsub's row
+    // thread (hsub, row) folds the four pieces of head hsub's row in ascending order
     const int hsub = tid / LQ, row = tid % LQ;
     if (hsub < p.gw) {
         const WgId wh = decode_wg(p, hsub, false);
         if (wh.wave_valid) {
-            float m = lds_m[hsub][row], l = lds_l[hsub][row];
-            for (int kq = 1; kq < nq; ++kq) {
-                const float mo = lds_m[kq * p.gw + hsub][row], lo = lds_l[kq * p.gw + hsub][row];
+            float m = lds_m[hsub * 4][row], l = lds_l[hsub * 4][row];
+            for (int pc = 1; pc < 4; ++pc) {
+                const float mo = lds_m[hsub * 4 + pc][row], lo = lds_l[hsub * 4 + pc][row];
                 const float m_new = fmaxf(m, mo);
                 const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
                 l = l * __builtin_amdgcn_exp2f(m - m_use) + lo * __builtin_amdgcn_exp2f(mo - m_use);
@@ -366,9 +386,8 @@ __global__ __launch_bounds__(EST_THREADS, 3) void est_stats_kernel(const EstPara
 // v_add_f32 with the whole-wave DPP shift wave_shr:1 per row) leaves in lane L the sum of the
 // diagonal n - i = L - 31: 16 swaps + 32 adds per block instead of 32 LDS writes, 64 LDS reads and
 // 64 adds (LDS float atomics, tried first, run at a fraction of a lane per clock).  The 63 sums
-// are added into a private per-wave window in LDS with plain read-modify-write (one wave,
-// in-order LDS: no race).
-constexpr int WWIN = KC + LQ;                // per-wave diagonal window: at most the whole chunk + 64
+// are added into the window of the block's piece in LDS (PIECE keys + 64 slots, private to the wave
+// that walks the piece) with plain read-modify-write (one wave, in-order LDS: no race).
 __device__ __forceinline__ float wave_shr1(float x) {      // lane L <- lane L - 1, lane 0 <- 0
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x138, 0xf, 0xf, true));
 }
@@ -378,18 +397,18 @@ __device__ __forceinline__ float wave_shr1(float x) {      // lane L <- lane L -
 template <typename T, int HD, bool RR>
 __global__ __launch_bounds__(EST_THREADS, 2) void est_scores_kernel(const EstParams p) {
     constexpr int KS = HD / 16;
-    __shared__ float lds_wwin[4][WWIN];
+    __shared__ float lds_pwin[16][PWIN];               // [head of the workgroup * 4 + piece][slot]
     const int tid = (int)threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);       // wave-uniform: addresses built from it stay scalar
     const WgId w = decode_wg(p, wave, true);
     if (!w.valid) return;
     const int l32 = lane & 31, g = lane >> 5;
     const int nq = 4 / p.gw, klen = KC / nq;          // key sub-ranges per head, keys per wave
-    const int wwin_len = klen + LQ;
+    const int ppw = p.gw;                             // pieces per wave (klen / PIECE)
     const long long bh = (long long)w.b * p.index_heads + w.slot;
-    float *wwin = lds_wwin[wave];
+    float *const wwin0 = lds_pwin[(wave % p.gw) * 4 + w.kq * ppw];   // this wave's ppw piece windows, contiguous
 
-    for (int i = lane; i < wwin_len; i += 64) wwin[i] = 0.f;
+    for (int i = lane; i < ppw * PWIN; i += 64) wwin0[i] = 0.f;
     __syncthreads();
 
     __shared__ __attribute__((aligned(16))) char lds_kt[2][2 * KShare<HD>::TILE];
@@ -444,7 +463,8 @@ __global__ __launch_bounds__(EST_THREADS, 2) void est_scores_kernel(const EstPar
         // The block adds to 95 slots of the diagonal window, as two disjoint ranges: s1 + (0..63) and,
         // in lanes 32..62, s2 = s1 + 32.  Their old values are read now, a block's work ahead of the
         // add (window slot of lane L, row half mb: 32*blk + L + 32 - 32*mb - rshift = key - row + 63 - rshift).
-        const int s1 = 32 * blk + lane - rshift, s2 = s1 + 32;
+        float *const wwin = wwin0 + (blk / PB) * PWIN;                  // the window of this block's piece
+        const int s1 = 32 * (blk % PB) + lane - rshift, s2 = s1 + 32;
         const bool ok1 = s1 >= 0, ok2 = lane >= 32 && lane < 63 && s2 >= 0;
         const float w1 = ok1 ? wwin[s1] : 0.f;
         const float w2 = ok2 ? wwin[s2] : 0.f;
@@ -554,16 +574,16 @@ __global__ __launch_bounds__(EST_THREADS, 2) void est_scores_kernel(const EstPar
         }
     }
     __syncthreads();
-    // chunk window of head hsub, position q = (key - chunk0) + (last_q - 1 - i): wave kq * gw + hsub
-    // contributes its slot q - kq * klen
+    // chunk window of head hsub, position q = (key - chunk0) + (last_q - 1 - i): piece pc contributes
+    // its slot q - pc * PIECE; the pieces are added in ascending order
     for (int idx = tid; idx < p.gw * WIN; idx += EST_THREADS) {
         const int hsub = idx / WIN, q = idx - hsub * WIN;
         const WgId wh = decode_wg(p, hsub, true);
         if (!wh.wave_valid) continue;
         float acc = 0.f;
-        for (int kq = 0; kq < nq; ++kq) {
-            const int sl = q - kq * klen;
-            if (sl >= 0 && sl < wwin_len) acc += lds_wwin[kq * p.gw + hsub][sl];
+        for (int pc = 0; pc < 4; ++pc) {
+            const int sl = q - pc * PIECE;
+            if (sl >= 0 && sl < PWIN) acc += lds_pwin[hsub * 4 + pc][sl];
         }
         p.win[(((long long)wh.b * p.index_heads + wh.slot) * p.nchunks + wh.chunk) * WIN + q] = acc;
     }

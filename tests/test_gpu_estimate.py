@@ -136,3 +136,25 @@ def test_ragged_topk_pads_with_noop_entries(gpu, n):
         want_b = topk_indices(b[r:r + 1].contiguous(), kb[r], reverse_base=n - 1)[0]
         assert torch.equal(out_b[r, :kb[r]], want_b)
         assert (out_b[r, kb[r]:] == want_b[-1]).all()
+
+
+@pytest.mark.parametrize("hq,hk,n,dtype,d", [(4, 1, 20000 + 37, torch.bfloat16, 128), (8, 2, 9000, torch.float16, 64),
+                                              (2, 1, 5000, torch.bfloat16, 128), (6, 2, 2048 * 3, torch.bfloat16, 64)])
+def test_a_heads_scores_do_not_depend_on_the_heads_it_is_launched_with(gpu, hq, hk, n, dtype, d):
+    """Grouped-query launches score four (or two) heads per workgroup, one wave per head over a whole
+    2048-key chunk; a head on its own is scored by four waves of 512 keys.  Both sum a chunk as the same
+    four pieces in the same order, so the score vectors -- and with them the selected sets and the
+    attention output of the per-head dispatcher -- are identical bit for bit however the heads are
+    grouped into launches."""
+    from minference_amd.estimate import vertical_slash_scores
+    q, k, _ = gen.qkv(1, hq, hk, n, d, seed=n + hq, scale=1.0)
+    qg, kg = q.to(dtype).to(gpu), k.to(dtype).to(gpu)
+    group = hq // hk
+    for rounded in (True, False):
+        vert, slash = vertical_slash_scores(qg, kg, reference_rounding=rounded)
+        for h in range(hq):
+            v1, s1 = vertical_slash_scores(qg[:, h:h + 1], kg[:, h // group:h // group + 1], reference_rounding=rounded)
+            assert torch.equal(v1[0, 0], vert[0, h]) and torch.equal(s1[0, 0], slash[0, h]), (h, rounded)
+        if group > 1:      # ... and two heads of a group launched as a pair
+            v2, s2 = vertical_slash_scores(qg[:, :2], kg[:, :1], reference_rounding=rounded)
+            assert torch.equal(v2[0], vert[0, :2]) and torch.equal(s2[0], slash[0, :2]), rounded
